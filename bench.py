@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): the Q4_K x Q8_1 GEMV at the four decode
+shapes, batch 1 — qkv 2048->6144, gate+up 2048->12288, down 6144->2048, lm_head
+2048->151936.  One "step" is one launch of each shape.  Weights are resident in HBM before
+timing and every launch reads a different copy out of a > 512 MiB rotation, so neither L2
+nor the 256 MiB Infinity Cache serves re-reads.  `value` is algorithmic GB/s over the whole
+timed region (formula: N*K*144/256 + (K/32)*36 + N*4 bytes per launch).
+
+The timed region holds exactly K steps; launches are grouped by shape with a HIP event
+between groups (recorded on the library's stream), which gives each kernel's average
+launch duration from the same region that `value` is taken from.
+
+Prints ONE JSON line.  `python bench.py --gpus 1 --steps 200 --warmup 20`.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
+ROTATION = 4            # weight sets; one set is 203 MB, so the rotation spans 813 MB
+
+
+def gemv_bytes(N, K, batch=1):
+    return N * K * 144 // 256 + batch * (K // 32) * 36 + batch * N * 4
+
+
+def cpu_baseline(seconds_target=12.0):
+    """Time the CPU oracle's Q4_K x Q8_1 GEMV (OpenMP) on a bounded sample of the workload."""
+    from oracle import oracle as orc
+    from bunker_amd import synth
+
+    orc.build()
+    threads = min(16, os.cpu_count() or 1)
+    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+    threads = int(os.environ["OMP_NUM_THREADS"])
+    name, N, K = SHAPES[1]
+    g = synth.rng(1)
+    W = synth.q4k_random(g, N, K)
+    xq = orc.pack_q8_1(g.standard_normal(K).astype(np.float32))
+    orc.gemv_q4k_q8_1(W, xq, N, K, acc64=False)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        orc.gemv_q4k_q8_1(W, xq, N, K, acc64=False)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds_target or reps >= 2000:
+            break
+    gbs = reps * gemv_bytes(N, K) / dt / 1e9
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} x {name} GEMV (N={N}, K={K}, batch 1) with the C oracle, "
+                      f"{dt:.1f} s on {threads} OpenMP threads of the host CPU"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
+                    help="graph: each shape's K launches are replayed from one HIP graph; "
+                         "stream: K individual launches from Python")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives, no sharding).", file=sys.stderr)
+        sys.exit(2)
+
+    from bunker_amd import runtime as rt
+    from bunker_amd import synth
+
+    rt.cu(0)
+    info = rt.device_info()
+    g = synth.rng(2026)
+
+    # one weight set on the host, ROTATION copies on the device
+    sets = []          # sets[r][shape] = device pointer
+    host = {}
+    for name, N, K in SHAPES:
+        host[name] = synth.q4k_random(g, N, K)
+    for r in range(ROTATION):
+        ptrs = {}
+        for name, N, K in SHAPES:
+            if r == 0:
+                ptrs[name] = rt.to_device(host[name])
+            else:
+                ptrs[name] = rt.cuAlloc(host[name].nbytes)
+                rt.cuDtoD(ptrs[name], sets[0][name], host[name].nbytes)
+        sets.append(ptrs)
+    del host
+    xq, y = {}, {}
+    for name, N, K in SHAPES:
+        x = g.standard_normal(K).astype(np.float32)
+        dx = rt.to_device(x)
+        xq[name] = rt.cuAlloc(K // 32 * 36)
+        rt.quantize_q8_1(dx, xq[name], K, 1, rt.F32)
+        y[name] = rt.cuAlloc(N * 4)
+    rt.cuSync()
+
+    def launch(name, N, K, i):
+        rt.gemv_q4k_q8_1(sets[i % ROTATION][name], xq[name], y[name], N, K)
+
+    for w in range(args.warmup):
+        for name, N, K in SHAPES:
+            launch(name, N, K, w)
+    rt.cuSync()
+
+    graphs = []
+    if args.mode == "graph":
+        for name, N, K in SHAPES:
+            with rt.Graph() as gr:
+                for i in range(args.steps):
+                    launch(name, N, K, i)
+            graphs.append(gr)
+        rt.cuSync()
+
+    ev = [rt.Event() for _ in range(len(SHAPES) + 1)]
+    rt.cuSync()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for si, (name, N, K) in enumerate(SHAPES):
+        if graphs:
+            graphs[si].launch()
+        else:
+            for i in range(args.steps):
+                launch(name, N, K, i)
+        ev[si + 1].record()
+    rt.cuSync()
+    wall = time.perf_counter() - t0
+
+    per_shape = {}
+    total_ms = ev[0].elapsed_ms(ev[-1])
+    for si, (name, N, K) in enumerate(SHAPES):
+        ms = ev[si].elapsed_ms(ev[si + 1]) / args.steps
+        b = gemv_bytes(N, K)
+        per_shape[name] = {"N": N, "K": K, "us_per_launch": round(ms * 1e3, 3), "bytes": b,
+                           "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                           "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    step_bytes = sum(gemv_bytes(N, K) for _, N, K in SHAPES)
+    ms_per_step = total_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel: gemv_q4k_q8_1_kernel<1,0> serves every K=2048 shape (qkv, gate_up, lm_head)
+    dom = [n for n, _, K in SHAPES if K == 2048]
+    dom_bytes = sum(per_shape[n]["bytes"] for n in dom) / len(dom)
+    dom_us = sum(per_shape[n]["us_per_launch"] for n in dom) / len(dom)
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "gemv_q4k_q8_1_kernel<1,0>", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": None}
+
+    out = {
+        "metric": "Q4_K GEMV HBM GB/s (% of peak); synthetic Qwen3.5 decode tok/s at bs=1/32",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8xint4->int32 dots, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "Q4_K x Q8_1 GEMV, batch 1, decode shapes qkv/gate_up/down/lm_head "
+                               "(BASELINE configs[1]); one step = one launch of each shape",
+                   "weight_rotation_MB": round(ROTATION * sum(N * K * 144 // 256 for _, N, K in SHAPES) / 1e6),
+                   "launch_mode": args.mode, "device": info["name"], "cus": info["cus"]},
+        "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
+        "per_shape": per_shape,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

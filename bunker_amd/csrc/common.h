@@ -1,0 +1,130 @@
+// Shared host/device helpers for the gfx950 decode kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bk {
+
+// ---------------------------------------------------------------- host side
+// Every launcher returns 0 on success or a negative code after recording a
+// message that bk_last_error() hands to the caller.
+enum : int {
+  BK_OK = 0,
+  BK_ERR_ARG = -1,      // bad argument (null pointer, unsupported shape)
+  BK_ERR_HIP = -2,      // a HIP runtime call failed
+  BK_ERR_STATE = -3,    // library not initialised / unknown handle
+  BK_ERR_UNSUPPORTED = -4,
+};
+
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+hipStream_t stream();   // the stream every kernel of this library is launched on
+int num_cus();
+
+#define BK_HIP(call)                                                                   \
+  do {                                                                                 \
+    hipError_t e_ = (call);                                                            \
+    if (e_ != hipSuccess)                                                              \
+      return ::bk::set_error(::bk::BK_ERR_HIP, "%s failed: %s (%s:%d)", #call,         \
+                             hipGetErrorString(e_), __FILE__, __LINE__);               \
+  } while (0)
+
+#define BK_REQUIRE(cond, ...)                                          \
+  do {                                                                 \
+    if (!(cond)) return ::bk::set_error(::bk::BK_ERR_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define BK_LAUNCH_CHECK()                                                              \
+  do {                                                                                 \
+    hipError_t e_ = hipGetLastError();                                                 \
+    if (e_ != hipSuccess)                                                              \
+      return ::bk::set_error(::bk::BK_ERR_HIP, "kernel launch failed: %s (%s:%d)",     \
+                             hipGetErrorString(e_), __FILE__, __LINE__);               \
+  } while (0)
+
+// ---------------------------------------------------------------- device side
+#if defined(__HIPCC__)
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// f32 -> bf16, round to nearest even; NaN keeps a quiet payload.
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x7fffffu)) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// Exact IEEE binary16 -> binary32 (v_cvt_f32_f16 honours denormals).
+__device__ __forceinline__ float half_to_f32(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// Truncating binary32 -> binary16 used for the Q8_1 scales: drop the low 13
+// mantissa bits, flush below the normal range to signed zero, overflow to Inf.
+__device__ __forceinline__ uint16_t f32_to_half_trunc(float v) {
+  uint32_t bits = __float_as_uint(v);
+  if ((bits & 0x7fffffffu) == 0) return 0;
+  uint32_t s = (bits >> 16) & 0x8000u, e = (bits >> 23) & 0xffu, m = bits & 0x7fffffu;
+  int ne = (int)e - 127 + 15;
+  if (ne >= 31) return (uint16_t)(s | 0x7c00u);
+  if (ne <= 0) return (uint16_t)s;
+  return (uint16_t)(s | ((uint32_t)ne << 10) | (m >> 13));
+}
+
+// DPP controls (GFX9 encoding)
+constexpr int DPP_QUAD_XOR1 = 0xB1;      // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;      // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_MIRROR = 0x140;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Sum over each aligned group of 16 lanes; every lane of the group gets the total.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f32<DPP_QUAD_XOR1>(v);
+  v += dpp_f32<DPP_QUAD_XOR2>(v);
+  v += dpp_f32<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_f32<DPP_ROW_MIRROR>(v);
+  return v;
+}
+// Sum over the whole 64-lane wavefront; the result is wave-uniform.  The order
+// of additions is fixed, so the result does not depend on the launch shape.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  return (readlane_f32(v, 0) + readlane_f32(v, 16)) + (readlane_f32(v, 32) + readlane_f32(v, 48));
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f32<DPP_QUAD_XOR1>(v));
+  v = fmaxf(v, dpp_f32<DPP_QUAD_XOR2>(v));
+  v = fmaxf(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
+  v = fmaxf(v, dpp_f32<DPP_ROW_MIRROR>(v));
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = row16_max(v);
+  return fmaxf(fmaxf(readlane_f32(v, 0), readlane_f32(v, 16)), fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
+}
+__device__ __forceinline__ int row16_sum_i32(int v) {
+  v += dpp_i32<DPP_QUAD_XOR1>(v);
+  v += dpp_i32<DPP_QUAD_XOR2>(v);
+  v += dpp_i32<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_i32<DPP_ROW_MIRROR>(v);
+  return v;
+}
+
+__device__ __forceinline__ float sigmoidf_dev(float v) { return 1.0f / (1.0f + __expf(-v)); }
+
+#endif  // __HIPCC__
+}  // namespace bk

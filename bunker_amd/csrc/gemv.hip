@@ -1,0 +1,397 @@
+// Q4_K dequant-GEMV kernels for gfx950: y[N] = W[N,K] . x[K], W in 144-byte
+// super-blocks, streamed once from HBM with 128-bit loads.
+//
+// Lane mapping (all kernels here).  A wavefront walks whole weight rows.  The
+// 128 nibble bytes of a super-block are 8 chunks of 16 bytes; "slot"
+// s = 64*round + lane covers chunk c = s & 7 of block s >> 3, so one wave-wide
+// 16-byte load fetches the nibbles of 8 consecutive blocks (1 KiB contiguous
+// but for the 16-byte headers, which a second, 8-way broadcast load fetches).
+// Chunk c holds, for l in [16*(c&1), 16*(c&1)+16), the low nibbles of
+// sub-block 2*(c>>1) and the high nibbles of sub-block 2*(c>>1)+1.  The slice
+// of the activation a lane needs therefore depends on the lane only, not on
+// the row: it is loaded once into registers and reused for every row.
+#include "ops.h"
+
+namespace bk {
+
+constexpr int GEMV_WAVES = 4;           // waves per workgroup
+constexpr int GEMV_RPI = 4;             // rows in flight per wave (independent loads)
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+  return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Lane c of an 8-lane group extracts scale and min of sub-block j = c from the
+// 12 packed bytes (dwords s0, s1, s2).  cA/cW/cB are lane constants:
+//   c < 4 : sc = (s0 >> 8c) & 63 ; m = (s1 >> 8c) & 63
+//   c >= 4: sc = ((s2 >> 8(c-4)) & 15) | ((s0 >> (8(c-4)+6)) & 3) << 4 ; m likewise from s1
+struct ScaleSel {
+  uint32_t sh;     // 8 * (c & 3)
+  uint32_t wlo;    // 6 or 4 : width of the low field
+  uint32_t whi;    // 0 or 2 : width of the high field
+  bool hi;         // c >= 4
+};
+__device__ __forceinline__ ScaleSel make_scale_sel(int c) {
+  ScaleSel s;
+  s.sh = 8u * (c & 3);
+  s.hi = c >= 4;
+  s.wlo = s.hi ? 4u : 6u;
+  s.whi = s.hi ? 2u : 0u;
+  return s;
+}
+__device__ __forceinline__ uint32_t bfe(uint32_t v, uint32_t off, uint32_t width) {
+  return __builtin_amdgcn_ubfe(v, off, width);
+}
+__device__ __forceinline__ void lane_scale_min(const ScaleSel& s, uint32_t s0, uint32_t s1, uint32_t s2,
+                                               uint32_t& sc, uint32_t& m) {
+  const uint32_t t = s2 >> s.sh;
+  const uint32_t a = s.hi ? t : (s0 >> s.sh);
+  const uint32_t b = s.hi ? (t >> 4) : (s1 >> s.sh);
+  sc = bfe(a, 0, s.wlo) | (bfe(s0, s.sh + 6, s.whi) << 4);
+  m = bfe(b, 0, s.wlo) | (bfe(s1, s.sh + 6, s.whi) << 4);
+}
+
+// quad_perm:[0,0,2,2] and [1,1,3,3]: the even / odd lane of each lane pair
+constexpr int DPP_PAIR_EVEN = 0xA0;
+constexpr int DPP_PAIR_ODD = 0xF5;
+
+// Activation slice of one slot, Q8_1 layout (int8 q[32] @0, fp16 d @32, fp16 s @34).
+struct XQ {
+  uint32_t lo[4], hi[4];   // 16 int8 of sub-block 2g and of sub-block 2g+1
+  float d8c, s8c;          // d and s of sub-block c (for the lane's share of scales / mins)
+};
+
+__device__ __forceinline__ void load_xq(XQ& x, const uint8_t* __restrict__ xq, int blk, int c, bool active) {
+  if (!active) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) { x.lo[i] = 0; x.hi[i] = 0; }
+    x.d8c = 0.0f; x.s8c = 0.0f;
+    return;
+  }
+  const int g = c >> 1, half = c & 1;
+  const uint32_t* p0 = (const uint32_t*)(xq + (int64_t)(blk * 8 + 2 * g) * 36 + 16 * half);
+  const uint32_t* p1 = (const uint32_t*)(xq + (int64_t)(blk * 8 + 2 * g + 1) * 36 + 16 * half);
+#pragma unroll
+  for (int i = 0; i < 4; i++) { x.lo[i] = p0[i]; x.hi[i] = p1[i]; }
+  const uint32_t ds = *(const uint32_t*)(xq + (int64_t)(blk * 8 + c) * 36 + 32);
+  x.d8c = half_to_f32((uint16_t)(ds & 0xffffu));
+  x.s8c = half_to_f32((uint16_t)(ds >> 16));
+}
+
+// One slot's contribution to a row: returns the f32 partial; I0/I1 are the
+// exact int32 half-sub-block dots (low / high nibbles).
+__device__ __forceinline__ float slot_dot(const uint4& hdr, const uint4& q, const XQ& x, const ScaleSel& sel,
+                                          int& I0, int& I1) {
+  const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu));
+  const float dmin = half_to_f32((uint16_t)(hdr.x >> 16));
+  uint32_t sc, m;
+  lane_scale_min(sel, hdr.y, hdr.z, hdr.w, sc, m);
+  const float fsc = (d * x.d8c) * (float)sc;
+  const float fm = (dmin * x.s8c) * (float)m;
+  int a = 0, b = 0;
+  a = sdot4(q.x & 0x0f0f0f0fu, x.lo[0], a);
+  b = sdot4((q.x >> 4) & 0x0f0f0f0fu, x.hi[0], b);
+  a = sdot4(q.y & 0x0f0f0f0fu, x.lo[1], a);
+  b = sdot4((q.y >> 4) & 0x0f0f0f0fu, x.hi[1], b);
+  a = sdot4(q.z & 0x0f0f0f0fu, x.lo[2], a);
+  b = sdot4((q.z >> 4) & 0x0f0f0f0fu, x.hi[2], b);
+  a = sdot4(q.w & 0x0f0f0f0fu, x.lo[3], a);
+  b = sdot4((q.w >> 4) & 0x0f0f0f0fu, x.hi[3], b);
+  I0 = a; I1 = b;
+  const float f0 = dpp_f32<DPP_PAIR_EVEN>(fsc);   // combined scale of sub-block 2g
+  const float f1 = dpp_f32<DPP_PAIR_ODD>(fsc);    // combined scale of sub-block 2g+1
+  return (f0 * (float)a + f1 * (float)b) - fm;
+}
+
+enum : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_BF16_ADD = 2 };
+
+template <int EPI>
+__device__ __forceinline__ void store_out(void* __restrict__ y, const uint16_t* __restrict__ res, int64_t i, float v) {
+  if (EPI == EPI_F32) {
+    ((float*)y)[i] = v;
+  } else if (EPI == EPI_BF16) {
+    ((uint16_t*)y)[i] = f32_to_bf16(v);
+  } else {
+    // gemm(f32) -> cast(bf16) -> add(bf16, bf16): two roundings, as the model graph orders them
+    const float c = bf16_to_f32(f32_to_bf16(v));
+    ((uint16_t*)y)[i] = f32_to_bf16(c + bf16_to_f32(res[i]));
+  }
+}
+
+// NR = number of 64-slot rounds per row (K = 2048*NR when the row fills every round).
+template <int NR, int EPI>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
+    const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq_all, void* __restrict__ y,
+    const uint16_t* __restrict__ res, int N, int nb) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int bidx = blockIdx.y;
+  const uint8_t* xq = xq_all + (int64_t)bidx * nb * 8 * 36;
+  const int c = lane & 7;
+  const ScaleSel sel = make_scale_sel(c);
+  const int64_t row_bytes = (int64_t)nb * 144;
+
+  XQ x[NR];
+  int boff[NR];   // byte offset of the slot's block inside a row
+#pragma unroll
+  for (int r = 0; r < NR; r++) {
+    const int blk = r * 8 + (lane >> 3);
+    const bool active = blk < nb;
+    load_xq(x[r], xq, blk, c, active);
+    boff[r] = (active ? blk : 0) * 144;
+  }
+
+  for (int row0 = wave * GEMV_RPI; row0 < N; row0 += nwaves * GEMV_RPI) {
+    uint4 hdr[GEMV_RPI][NR], q[GEMV_RPI][NR];
+#pragma unroll
+    for (int i = 0; i < GEMV_RPI; i++) {
+      const int row = min(row0 + i, N - 1);
+      const uint8_t* rp = W + (int64_t)row * row_bytes;
+#pragma unroll
+      for (int r = 0; r < NR; r++) {
+        hdr[i][r] = *(const uint4*)(rp + boff[r]);
+        q[i][r] = *(const uint4*)(rp + boff[r] + 16 + 16 * c);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < GEMV_RPI; i++) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int r = 0; r < NR; r++) {
+        int I0, I1;
+        acc += slot_dot(hdr[i][r], q[i][r], x[r], sel, I0, I1);
+      }
+      const float tot = wave_sum(acc);
+      if (lane == 0 && row0 + i < N) store_out<EPI>(y, res, (int64_t)bidx * N + row0 + i, tot);
+    }
+  }
+}
+
+// Any K that is a multiple of 256: rounds are a run-time loop and the activation
+// slice is re-read (from L2) in every round.
+template <int EPI>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_generic_kernel(
+    const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq_all, void* __restrict__ y,
+    const uint16_t* __restrict__ res, int N, int nb) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int bidx = blockIdx.y;
+  const uint8_t* xq = xq_all + (int64_t)bidx * nb * 8 * 36;
+  const int c = lane & 7;
+  const ScaleSel sel = make_scale_sel(c);
+  const int64_t row_bytes = (int64_t)nb * 144;
+  const int rounds = (nb + 7) / 8;
+  for (int row = wave; row < N; row += nwaves) {
+    const uint8_t* rp = W + (int64_t)row * row_bytes;
+    float acc = 0.0f;
+    for (int r = 0; r < rounds; r++) {
+      const int blk = r * 8 + (lane >> 3);
+      const bool active = blk < nb;
+      XQ x;
+      load_xq(x, xq, blk, c, active);
+      const int bo = (active ? blk : 0) * 144;
+      const uint4 hdr = *(const uint4*)(rp + bo);
+      const uint4 q = *(const uint4*)(rp + bo + 16 + 16 * c);
+      int I0, I1;
+      acc += slot_dot(hdr, q, x, sel, I0, I1);
+    }
+    const float tot = wave_sum(acc);
+    if (lane == 0) store_out<EPI>(y, res, (int64_t)bidx * N + row, tot);
+  }
+}
+
+// Exact int32 sub-block dots I[N, 8*nb]: lane pairs (c even, c odd) hold the two
+// 16-element halves of sub-blocks 2g and 2g+1.
+__global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
+    const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq, int32_t* __restrict__ I, int N, int nb) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int c = lane & 7;
+  const ScaleSel sel = make_scale_sel(c);
+  const int64_t row_bytes = (int64_t)nb * 144;
+  const int rounds = (nb + 7) / 8;
+  for (int row = wave; row < N; row += nwaves) {
+    const uint8_t* rp = W + (int64_t)row * row_bytes;
+    for (int r = 0; r < rounds; r++) {
+      const int blk = r * 8 + (lane >> 3);
+      const bool active = blk < nb;
+      XQ x;
+      load_xq(x, xq, blk, c, active);
+      const int bo = (active ? blk : 0) * 144;
+      const uint4 hdr = *(const uint4*)(rp + bo);
+      const uint4 q = *(const uint4*)(rp + bo + 16 + 16 * c);
+      int I0, I1;
+      (void)slot_dot(hdr, q, x, sel, I0, I1);
+      const int s0 = I0 + dpp_i32<DPP_QUAD_XOR1>(I0);
+      const int s1 = I1 + dpp_i32<DPP_QUAD_XOR1>(I1);
+      if (active) I[(int64_t)row * nb * 8 + blk * 8 + c] = (c & 1) ? s1 : s0;
+    }
+  }
+}
+
+static int gemv_grid(int N, int rows_per_wg) {
+  int wgs = (N + rows_per_wg - 1) / rows_per_wg;
+  const int cap = num_cus() * 8;
+  return wgs < cap ? wgs : cap;
+}
+
+template <int EPI>
+static void launch_q8_1_variant(const void* W, const void* xq, void* y, const void* res, int N, int nb, int batch) {
+  const int rounds = (nb + 7) / 8;
+  dim3 block(GEMV_WAVES * 64);
+  dim3 grid(gemv_grid(N, GEMV_WAVES * GEMV_RPI), batch);
+  const uint8_t* w = (const uint8_t*)W; const uint8_t* x = (const uint8_t*)xq; const uint16_t* r = (const uint16_t*)res;
+  switch (rounds) {
+    case 1: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<1, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
+    case 2: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<2, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
+    case 3: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<3, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
+    default:
+      grid.x = gemv_grid(N, GEMV_WAVES);
+      hipLaunchKernelGGL((gemv_q4k_q8_1_generic_kernel<EPI>), grid, block, 0, stream(), w, x, y, r, N, nb);
+  }
+}
+
+int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
+                         const void* residual) {
+  BK_REQUIRE(W && xq && y, "gemv_q4k_q8_1: null pointer");
+  BK_REQUIRE(N > 0 && K > 0 && K % 256 == 0, "gemv_q4k_q8_1: K=%d must be a positive multiple of 256 (N=%d)", K, N);
+  BK_REQUIRE(batch > 0 && batch <= 65535, "gemv_q4k_q8_1: bad batch=%d", batch);
+  BK_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gemv_q4k_q8_1: out_dtype must be 0 (f32) or 1 (bf16)");
+  BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemv_q4k_q8_1: a residual needs bf16 output");
+  BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "gemv_q4k_q8_1: W must be 16-byte and xq 4-byte aligned");
+  const int nb = K / 256;
+  if (out_dtype == DT_F32) launch_q8_1_variant<EPI_F32>(W, xq, y, nullptr, N, nb, batch);
+  else if (!residual) launch_q8_1_variant<EPI_BF16>(W, xq, y, nullptr, N, nb, batch);
+  else launch_q8_1_variant<EPI_BF16_ADD>(W, xq, y, residual, N, nb, batch);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, int K) {
+  BK_REQUIRE(W && xq && I, "q4k_q8_1_subdots: null pointer");
+  BK_REQUIRE(N > 0 && K > 0 && K % 256 == 0, "q4k_q8_1_subdots: K=%d must be a positive multiple of 256", K);
+  BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "q4k_q8_1_subdots: misaligned pointer");
+  hipLaunchKernelGGL(q4k_q8_1_subdots_kernel, dim3(gemv_grid(N, GEMV_WAVES)), dim3(GEMV_WAVES * 64), 0, stream(),
+                     (const uint8_t*)W, (const uint8_t*)xq, I, N, K / 256);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- f32 activations
+// Dequantise-and-dot with x in f32: per slot, 16 low-nibble and 16 high-nibble
+// weights against 32 activation values held in registers.
+//   y += d*sc0*sum(nib_lo*x_lo) - dmin*m0*sum(x_lo) + d*sc1*sum(nib_hi*x_hi) - dmin*m1*sum(x_hi)
+struct XF {
+  float lo[16], hi[16];
+  float sum_c;   // sum of the 32 activations of sub-block c (for the lane's share of the mins)
+};
+
+__device__ __forceinline__ float nibdot4(uint32_t n4, const float* x, float acc) {
+  acc = fmaf((float)(n4 & 0xffu), x[0], acc);
+  acc = fmaf((float)((n4 >> 8) & 0xffu), x[1], acc);
+  acc = fmaf((float)((n4 >> 16) & 0xffu), x[2], acc);
+  acc = fmaf((float)(n4 >> 24), x[3], acc);
+  return acc;
+}
+
+template <int NR>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_f32_kernel(
+    const uint8_t* __restrict__ W, const float* __restrict__ xf, float* __restrict__ y, int N, int nb) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int c = lane & 7, g = c >> 1, half = c & 1;
+  const ScaleSel sel = make_scale_sel(c);
+  const int64_t row_bytes = (int64_t)nb * 144;
+  const int rounds = NR > 0 ? NR : (nb + 7) / 8;
+
+  XF x[NR > 0 ? NR : 1];
+  int boff[NR > 0 ? NR : 1];
+  auto load_x = [&](XF& xx, int blk, bool active) {
+    if (!active) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) { xx.lo[i] = 0.0f; xx.hi[i] = 0.0f; }
+      xx.sum_c = 0.0f;
+      return;
+    }
+    const float4* p0 = (const float4*)(xf + blk * 256 + 64 * g + 16 * half);
+    const float4* p1 = (const float4*)(xf + blk * 256 + 64 * g + 32 + 16 * half);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const float4 a = p0[i], b = p1[i];
+      xx.lo[4 * i] = a.x; xx.lo[4 * i + 1] = a.y; xx.lo[4 * i + 2] = a.z; xx.lo[4 * i + 3] = a.w;
+      xx.hi[4 * i] = b.x; xx.hi[4 * i + 1] = b.y; xx.hi[4 * i + 2] = b.z; xx.hi[4 * i + 3] = b.w;
+    }
+    // sum of sub-block c = elements [32c', ...): sub-block j covers 64*(j>>1) + 32*(j&1) + [0,32)
+    const float4* ps = (const float4*)(xf + blk * 256 + 64 * (c >> 1) + 32 * (c & 1));
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) { const float4 v = ps[i]; s += (v.x + v.y) + (v.z + v.w); }
+    xx.sum_c = s;
+  };
+  if (NR > 0) {
+#pragma unroll
+    for (int r = 0; r < (NR > 0 ? NR : 1); r++) {
+      const int blk = r * 8 + (lane >> 3);
+      load_x(x[r], blk, blk < nb);
+      boff[r] = (blk < nb ? blk : 0) * 144;
+    }
+  }
+
+  for (int row = wave; row < N; row += nwaves) {
+    const uint8_t* rp = W + (int64_t)row * row_bytes;
+    float acc = 0.0f;
+#pragma unroll
+    for (int r = 0; r < rounds; r++) {
+      const int ri = NR > 0 ? r : 0;
+      if (NR == 0) {
+        const int blk = r * 8 + (lane >> 3);
+        load_x(x[0], blk, blk < nb);
+        boff[0] = (blk < nb ? blk : 0) * 144;
+      }
+      const uint4 hdr = *(const uint4*)(rp + boff[ri]);
+      const uint4 q = *(const uint4*)(rp + boff[ri] + 16 + 16 * c);
+      const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu));
+      const float dmin = half_to_f32((uint16_t)(hdr.x >> 16));
+      uint32_t sc, m;
+      lane_scale_min(sel, hdr.y, hdr.z, hdr.w, sc, m);
+      const float fsc = d * (float)sc;
+      const float fm = (dmin * (float)m) * x[ri].sum_c;
+      float a = 0.0f, b = 0.0f;
+      a = nibdot4(q.x & 0x0f0f0f0fu, &x[ri].lo[0], a);
+      b = nibdot4((q.x >> 4) & 0x0f0f0f0fu, &x[ri].hi[0], b);
+      a = nibdot4(q.y & 0x0f0f0f0fu, &x[ri].lo[4], a);
+      b = nibdot4((q.y >> 4) & 0x0f0f0f0fu, &x[ri].hi[4], b);
+      a = nibdot4(q.z & 0x0f0f0f0fu, &x[ri].lo[8], a);
+      b = nibdot4((q.z >> 4) & 0x0f0f0f0fu, &x[ri].hi[8], b);
+      a = nibdot4(q.w & 0x0f0f0f0fu, &x[ri].lo[12], a);
+      b = nibdot4((q.w >> 4) & 0x0f0f0f0fu, &x[ri].hi[12], b);
+      const float f0 = dpp_f32<DPP_PAIR_EVEN>(fsc);
+      const float f1 = dpp_f32<DPP_PAIR_ODD>(fsc);
+      acc += (f0 * a + f1 * b) - fm;
+    }
+    const float tot = wave_sum(acc);
+    if (lane == 0) y[row] = tot;
+  }
+}
+
+int launch_gemv_q4k_f32(const void* W, const float* x, float* y, int N, int K) {
+  BK_REQUIRE(W && x && y, "gemv_q4k_f32: null pointer");
+  BK_REQUIRE(N > 0 && K > 0 && K % 256 == 0, "gemv_q4k_f32: K=%d must be a positive multiple of 256 (N=%d)", K, N);
+  BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)x & 15) == 0, "gemv_q4k_f32: W and x must be 16-byte aligned");
+  const int nb = K / 256, rounds = (nb + 7) / 8;
+  dim3 block(GEMV_WAVES * 64), grid(gemv_grid(N, GEMV_WAVES));
+  const uint8_t* w = (const uint8_t*)W;
+  switch (rounds) {
+    case 1: hipLaunchKernelGGL((gemv_q4k_f32_kernel<1>), grid, block, 0, stream(), w, x, y, N, nb); break;
+    case 2: hipLaunchKernelGGL((gemv_q4k_f32_kernel<2>), grid, block, 0, stream(), w, x, y, N, nb); break;
+    default: hipLaunchKernelGGL((gemv_q4k_f32_kernel<0>), grid, block, 0, stream(), w, x, y, N, nb);
+  }
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

@@ -1,0 +1,267 @@
+// Runtime half of the C ABI: device, stream, memory, events, error text and the
+// per-launch profiler.  Replaces the CUDA-driver binding of src/ttir.ts:225-417.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/bunker_hip.h"
+#include "ops.h"
+
+namespace bk {
+
+static thread_local char g_err[1024] = "";
+static bool g_inited = false;
+static int g_device = -1;
+static hipStream_t g_stream = nullptr;
+static int g_cus = 256;
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+hipStream_t stream() { return g_stream; }
+int num_cus() { return g_cus; }
+bool inited() { return g_inited; }
+
+// ---- profiler: an event pair around every bk_launch, summed per kernel label
+struct ProfPending { hipEvent_t a, b; int kernel; };
+static bool g_prof = false;
+static std::vector<ProfPending> g_pending;
+static std::vector<hipEvent_t> g_pool;
+static std::map<std::string, std::pair<double, long>> g_totals;   // label -> (ms, count)
+
+bool prof_on() { return g_prof; }
+int prof_begin(int kernel) {
+  hipEvent_t a, b;
+  if (g_pool.size() >= 2) { a = g_pool.back(); g_pool.pop_back(); b = g_pool.back(); g_pool.pop_back(); }
+  else { BK_HIP(hipEventCreate(&a)); BK_HIP(hipEventCreate(&b)); }
+  BK_HIP(hipEventRecord(a, g_stream));
+  g_pending.push_back({a, b, kernel});
+  return BK_OK;
+}
+int prof_end() {
+  BK_HIP(hipEventRecord(g_pending.back().b, g_stream));
+  return BK_OK;
+}
+std::string kernel_label(int kernel);   // api.hip
+static int prof_collect() {
+  BK_HIP(hipStreamSynchronize(g_stream));
+  for (auto& p : g_pending) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+      auto& t = g_totals[kernel_label(p.kernel)];
+      t.first += ms; t.second += 1;
+    }
+    g_pool.push_back(p.a); g_pool.push_back(p.b);
+  }
+  g_pending.clear();
+  return BK_OK;
+}
+
+}  // namespace bk
+
+using namespace bk;
+
+#define BK_NEED_INIT() \
+  do { if (!g_inited) return set_error(BK_ERR_STATE, "bk_init has not been called"); } while (0)
+
+extern "C" {
+
+int bk_init(int device) {
+  if (g_inited) {
+    if (device == g_device) return BK_OK;
+    return set_error(BK_ERR_STATE, "already initialised on device %d", g_device);
+  }
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n == 0)
+    return set_error(BK_ERR_HIP, "no HIP device available (%s): the gfx950 kernels need an MI355X",
+                     e != hipSuccess ? hipGetErrorString(e) : "device count 0");
+  if (device < 0 || device >= n) return set_error(BK_ERR_ARG, "device %d out of range (0..%d)", device, n - 1);
+  BK_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  BK_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return set_error(BK_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+  g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  BK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  g_device = device;
+  g_inited = true;
+  return BK_OK;
+}
+
+int bk_shutdown(void) {
+  if (!g_inited) return BK_OK;
+  (void)hipStreamSynchronize(g_stream);
+  for (auto& p : g_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+  for (auto& ev : g_pool) (void)hipEventDestroy(ev);
+  g_pending.clear(); g_pool.clear(); g_totals.clear();
+  (void)hipStreamDestroy(g_stream);
+  g_stream = nullptr; g_inited = false; g_device = -1;
+  return BK_OK;
+}
+
+const char* bk_last_error(void) { return g_err; }
+
+int bk_device_info(char* buf, int cap) {
+  BK_NEED_INIT();
+  BK_REQUIRE(buf && cap > 0, "bk_device_info: bad buffer");
+  hipDeviceProp_t prop;
+  BK_HIP(hipGetDeviceProperties(&prop, g_device));
+  snprintf(buf, cap, "%s|%s|%d|%zu", prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.totalGlobalMem);
+  return BK_OK;
+}
+
+int bk_alloc(uint64_t bytes, uint64_t* out) {
+  BK_NEED_INIT();
+  BK_REQUIRE(out, "bk_alloc: null out");
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+  if (e != hipSuccess) return set_error(BK_ERR_HIP, "hipMalloc(%llu bytes) failed: %s", (unsigned long long)bytes, hipGetErrorString(e));
+  *out = (uint64_t)(uintptr_t)p;
+  return BK_OK;
+}
+int bk_free(uint64_t ptr) {
+  BK_NEED_INIT();
+  if (!ptr) return BK_OK;
+  BK_HIP(hipStreamSynchronize(g_stream));
+  BK_HIP(hipFree((void*)(uintptr_t)ptr));
+  return BK_OK;
+}
+// Copies are ordered with the kernels: they go through the library's stream and
+// the call returns when the copy is complete, as cuMemcpyHtoD/DtoH do.
+int bk_htod(uint64_t dst, const void* src, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst && src, "bk_htod: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+  BK_HIP(hipStreamSynchronize(g_stream));
+  return BK_OK;
+}
+int bk_dtoh(void* dst, uint64_t src, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst && src, "bk_dtoh: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemcpyAsync(dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToHost, g_stream));
+  BK_HIP(hipStreamSynchronize(g_stream));
+  return BK_OK;
+}
+int bk_dtod(uint64_t dst, uint64_t src, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst && src, "bk_dtod: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToDevice, g_stream));
+  return BK_OK;
+}
+int bk_memset(uint64_t dst, int value, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst, "bk_memset: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemsetAsync((void*)(uintptr_t)dst, value, bytes, g_stream));
+  return BK_OK;
+}
+int bk_sync(void) {
+  BK_NEED_INIT();
+  BK_HIP(hipStreamSynchronize(g_stream));
+  return BK_OK;
+}
+
+int bk_event_create(uint64_t* out) {
+  BK_NEED_INIT();
+  BK_REQUIRE(out, "bk_event_create: null out");
+  hipEvent_t ev;
+  BK_HIP(hipEventCreate(&ev));
+  *out = (uint64_t)(uintptr_t)ev;
+  return BK_OK;
+}
+int bk_event_record(uint64_t ev) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ev, "bk_event_record: null event");
+  BK_HIP(hipEventRecord((hipEvent_t)(uintptr_t)ev, g_stream));
+  return BK_OK;
+}
+int bk_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms) {
+  BK_NEED_INIT();
+  BK_REQUIRE(start && stop && ms, "bk_event_elapsed_ms: null argument");
+  BK_HIP(hipEventSynchronize((hipEvent_t)(uintptr_t)stop));
+  BK_HIP(hipEventElapsedTime(ms, (hipEvent_t)(uintptr_t)start, (hipEvent_t)(uintptr_t)stop));
+  return BK_OK;
+}
+int bk_event_destroy(uint64_t ev) {
+  BK_NEED_INIT();
+  if (ev) BK_HIP(hipEventDestroy((hipEvent_t)(uintptr_t)ev));
+  return BK_OK;
+}
+
+static bool g_capturing = false;
+
+int bk_capture_begin(void) {
+  BK_NEED_INIT();
+  if (g_capturing) return set_error(BK_ERR_STATE, "bk_capture_begin: a capture is already open");
+  if (g_prof) return set_error(BK_ERR_STATE, "bk_capture_begin: switch the per-launch profiler off first");
+  BK_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+  g_capturing = true;
+  return BK_OK;
+}
+int bk_capture_end(uint64_t* graph) {
+  BK_NEED_INIT();
+  BK_REQUIRE(graph, "bk_capture_end: null out");
+  if (!g_capturing) return set_error(BK_ERR_STATE, "bk_capture_end: no capture is open");
+  g_capturing = false;
+  hipGraph_t g = nullptr;
+  BK_HIP(hipStreamEndCapture(g_stream, &g));
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) return set_error(BK_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  *graph = (uint64_t)(uintptr_t)exec;
+  return BK_OK;
+}
+int bk_graph_launch(uint64_t graph) {
+  BK_NEED_INIT();
+  BK_REQUIRE(graph, "bk_graph_launch: null graph");
+  BK_HIP(hipGraphLaunch((hipGraphExec_t)(uintptr_t)graph, g_stream));
+  return BK_OK;
+}
+int bk_graph_destroy(uint64_t graph) {
+  BK_NEED_INIT();
+  if (graph) BK_HIP(hipGraphExecDestroy((hipGraphExec_t)(uintptr_t)graph));
+  return BK_OK;
+}
+
+int bk_prof_enable(int on) { g_prof = on != 0; return BK_OK; }
+int bk_prof_reset(void) {
+  BK_NEED_INIT();
+  int rc = prof_collect();
+  g_totals.clear();
+  return rc;
+}
+int bk_prof_report(char* buf, int cap) {
+  BK_NEED_INIT();
+  BK_REQUIRE(buf && cap > 0, "bk_prof_report: bad buffer");
+  int rc = prof_collect();
+  if (rc) return rc;
+  std::vector<std::pair<std::string, std::pair<double, long>>> rows(g_totals.begin(), g_totals.end());
+  for (size_t i = 0; i < rows.size(); i++)
+    for (size_t j = i + 1; j < rows.size(); j++)
+      if (rows[j].second.first > rows[i].second.first) std::swap(rows[i], rows[j]);
+  double total = 0;
+  for (auto& r : rows) total += r.second.first;
+  int off = snprintf(buf, cap, "kernel elapsed (library stream), total %.3f ms\n", total);
+  for (auto& r : rows) {
+    if (off >= cap - 1) break;
+    off += snprintf(buf + off, cap - off, "%10.3f ms %5.1f%% x%-6ld avg %8.2f us  %s\n", r.second.first,
+                    total > 0 ? 100.0 * r.second.first / total : 0.0, r.second.second,
+                    1000.0 * r.second.first / (double)r.second.second, r.first.c_str());
+  }
+  return BK_OK;
+}
+
+}  // extern "C"

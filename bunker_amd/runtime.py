@@ -1,0 +1,304 @@
+"""Launch surface of the decode path over ``libbunker_hip.so``.
+
+Host-side counterpart of the reference's runtime boundary (src/ttir.ts:225-491):
+the same function names and argument meaning — ``cuAlloc``, ``cuHtoD``, ``cuDtoH``,
+``cuFree``, ``cuSync``, ``compileAndLoad``, ``cuLaunch``, ``profGpuReset``,
+``profGpuReport`` — bound with ctypes to the C ABI of ``include/bunker_hip.h``
+instead of to libcuda and the Triton shim.  Device pointers are plain ints, as
+they are bigints in the reference.
+
+There is no CPU fallback: importing works anywhere, but every call needs the
+compiled library and an MI355X and raises ``BunkerError`` otherwise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import re
+from dataclasses import dataclass
+from typing import Sequence
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libbunker_hip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_PKG), "include", "bunker_hip.h")
+
+
+class BunkerError(RuntimeError):
+    pass
+
+
+_lib = None
+_inited = False
+
+u64, i32, i64, vp = C.c_uint64, C.c_int, C.c_int64, C.c_void_p
+_SIGS = {
+    "bk_init": [i32], "bk_shutdown": [], "bk_device_info": [C.c_char_p, i32],
+    "bk_alloc": [u64, C.POINTER(u64)], "bk_free": [u64],
+    "bk_htod": [u64, vp, u64], "bk_dtoh": [vp, u64, u64], "bk_dtod": [u64, u64, u64],
+    "bk_memset": [u64, i32, u64], "bk_sync": [],
+    "bk_event_create": [C.POINTER(u64)], "bk_event_record": [u64],
+    "bk_event_elapsed_ms": [u64, u64, C.POINTER(C.c_float)], "bk_event_destroy": [u64],
+    "bk_prof_enable": [i32], "bk_prof_reset": [], "bk_prof_report": [C.c_char_p, i32],
+    "bk_capture_begin": [], "bk_capture_end": [C.POINTER(u64)], "bk_graph_launch": [u64],
+    "bk_graph_destroy": [u64],
+    "bk_kernel_create": [C.c_char_p], "bk_launch": [i32, C.POINTER(u64), i32],
+    "bk_kernel_describe": [i32, C.c_char_p, i32],
+    "bk_quantize_q8_1": [u64, i32, u64, i32, i32],
+    "bk_gemv_q4k_f32": [u64, u64, u64, i32, i32],
+    "bk_gemv_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
+    "bk_q4k_q8_1_subdots": [u64, u64, u64, i32, i32],
+    "bk_dequant_legacy_i8": [u64, u64, i64], "bk_q4k_nibbles": [u64, u64, i64],
+    "bk_q4k_dequant_f32": [u64, u64, i64],
+}
+
+
+def declared_symbols() -> list[str]:
+    """Every function name that include/bunker_hip.h declares."""
+    with open(HEADER_PATH) as f:
+        return re.findall(r"^BK_API\s+[\w\s\*]+?\b(bk_\w+)\(", f.read(), flags=re.M)
+
+
+def load_library(path: str | None = None):
+    """dlopen the C-ABI library (no GPU needed) and attach argument types."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise BunkerError(
+            f"{p} is missing: build it with `make -C bunker_amd/csrc` (hipcc --offload-arch=gfx950); "
+            "there is no CPU fallback for the decode kernels")
+    lib = C.CDLL(p)
+    lib.bk_last_error.restype = C.c_char_p
+    lib.bk_last_error.argtypes = []
+    for name, args in _SIGS.items():
+        fn = getattr(lib, name)
+        fn.restype = i32
+        fn.argtypes = args
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def _check(rc: int, what: str = "") -> int:
+    if rc < 0:
+        msg = _lib.bk_last_error().decode("utf-8", "replace") if _lib is not None else ""
+        raise BunkerError(f"{what}: {msg} (rc={rc})" if what else f"{msg} (rc={rc})")
+    return rc
+
+
+def cu(device: int = 0):
+    """Initialise the device once and return the bound library (src/ttir.ts:225-262)."""
+    global _inited
+    lib = load_library()
+    if not _inited:
+        _check(lib.bk_init(device), "bk_init")
+        _inited = True
+    return lib
+
+
+def device_info() -> dict:
+    buf = C.create_string_buffer(256)
+    _check(cu().bk_device_info(buf, 256), "bk_device_info")
+    name, arch, cus, mem = buf.value.decode().split("|")
+    return {"name": name, "arch": arch, "cus": int(cus), "mem_bytes": int(mem)}
+
+
+# ---------------------------------------------------------------- memory (src/ttir.ts:266-285)
+def cuAlloc(nbytes: int) -> int:
+    out = u64(0)
+    _check(cu().bk_alloc(int(nbytes), C.byref(out)), f"cuAlloc({nbytes})")
+    return int(out.value)
+
+
+def _host_view(buf):
+    if isinstance(buf, np.ndarray):
+        if not buf.flags.c_contiguous:
+            raise BunkerError("host array must be C-contiguous")
+        return buf.ctypes.data, buf.nbytes
+    mv = memoryview(buf)
+    arr = np.frombuffer(mv, dtype=np.uint8)
+    return arr.ctypes.data, arr.nbytes
+
+
+def cuHtoD(dev: int, host, nbytes: int | None = None) -> None:
+    addr, n = _host_view(host)
+    _check(cu().bk_htod(dev, addr, int(nbytes if nbytes is not None else n)), "cuHtoD")
+
+
+def cuDtoH(host, dev: int, nbytes: int | None = None) -> None:
+    addr, n = _host_view(host)
+    _check(cu().bk_dtoh(addr, dev, int(nbytes if nbytes is not None else n)), "cuDtoH")
+
+
+def cuFree(dev: int) -> None:
+    _check(cu().bk_free(dev), "cuFree")
+
+
+def cuSync() -> int:
+    return _check(cu().bk_sync(), "cuSync")
+
+
+def cuMemset(dev: int, value: int, nbytes: int) -> None:
+    _check(cu().bk_memset(dev, value, nbytes), "cuMemset")
+
+
+def cuDtoD(dst: int, src: int, nbytes: int) -> None:
+    _check(cu().bk_dtod(dst, src, nbytes), "cuDtoD")
+
+
+def to_device(arr: np.ndarray) -> int:
+    """Allocate and upload a numpy array; returns the device pointer."""
+    arr = np.ascontiguousarray(arr)
+    p = cuAlloc(max(arr.nbytes, 1))
+    if arr.nbytes:
+        cuHtoD(p, arr)
+    return p
+
+
+def from_device(dev: int, shape, dtype) -> np.ndarray:
+    out = np.empty(shape, dtype)
+    if out.nbytes:
+        cuDtoH(out, dev)
+    return out
+
+
+# ---------------------------------------------------------------- kernels (src/ttir.ts:321-350, 488-491)
+@dataclass(frozen=True)
+class LoadedKernel:
+    module: int
+    fn: int
+    shmem: int
+    label: str = ""
+
+
+def compileAndLoad(spec: str, funcName: str | None = None, numWarps: int = 4, label: str | None = None) -> LoadedKernel:
+    """Look up the pre-compiled kernel for an op spec such as ``"gemm N=6144 K=2048 cast=1"``.
+
+    Takes the place of compileAndLoad(ttir, funcName, numWarps, label): the op name and
+    the constants the reference baked into TTIR text arrive in ``spec``; ``funcName`` and
+    ``numWarps`` are accepted for call-site compatibility and ignored.
+    """
+    h = _check(cu().bk_kernel_create(spec.encode()), f"compileAndLoad({spec!r})")
+    return LoadedKernel(module=0, fn=h, shmem=0, label=label or spec)
+
+
+def cuLaunch(k: LoadedKernel, grid: Sequence[int], block: Sequence[int], args: Sequence[int]) -> int:
+    """Launch with the reference's slot packing: one 8-byte slot per argument.
+
+    ``grid`` and ``block`` are accepted and ignored (each kernel owns its launch shape).
+    Returns the library's return code without raising, as cuLaunch returns the driver's.
+    """
+    n = len(args)
+    slots = (u64 * n)(*[int(a) & 0xFFFFFFFFFFFFFFFF for a in args])
+    return cu().bk_launch(k.fn, slots, n)
+
+
+def last_error() -> str:
+    return load_library().bk_last_error().decode("utf-8", "replace")
+
+
+def profGpuEnable(on: bool = True) -> None:
+    _check(cu().bk_prof_enable(1 if on else 0))
+
+
+def profGpuReset() -> None:
+    _check(cu().bk_prof_reset(), "profGpuReset")
+
+
+def profGpuReport(print_fn=print) -> str:
+    buf = C.create_string_buffer(1 << 16)
+    _check(cu().bk_prof_report(buf, len(buf)), "profGpuReport")
+    text = buf.value.decode()
+    if print_fn:
+        print_fn(text)
+    return text
+
+
+class Event:
+    """HIP event on the library's stream (the cuEvent* calls of src/ttir.ts:352-417)."""
+
+    def __init__(self):
+        h = u64(0)
+        _check(cu().bk_event_create(C.byref(h)), "bk_event_create")
+        self.h = int(h.value)
+
+    def record(self):
+        _check(cu().bk_event_record(self.h), "bk_event_record")
+        return self
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float(0)
+        _check(cu().bk_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "bk_event_elapsed_ms")
+        return float(ms.value)
+
+    def destroy(self):
+        if self.h:
+            cu().bk_event_destroy(self.h)
+            self.h = 0
+
+
+class Graph:
+    """A recorded launch sequence: ``with Graph() as g: ...launches...`` then ``g.launch()``.
+
+    Everything enqueued inside the ``with`` block is captured into a HIP graph instead of
+    running; only kernel launches are legal there (no alloc, copy, sync or event call).
+    """
+
+    def __init__(self):
+        self.h = 0
+
+    def __enter__(self):
+        _check(cu().bk_capture_begin(), "bk_capture_begin")
+        return self
+
+    def __exit__(self, et, ev, tb):
+        h = u64(0)
+        rc = cu().bk_capture_end(C.byref(h))
+        if et is None:
+            _check(rc, "bk_capture_end")
+        self.h = int(h.value)
+        return False
+
+    def launch(self):
+        _check(cu().bk_graph_launch(self.h), "bk_graph_launch")
+
+    def destroy(self):
+        if self.h:
+            cu().bk_graph_destroy(self.h)
+            self.h = 0
+
+
+# ---------------------------------------------------------------- typed entry points
+F32, BF16 = 0, 1
+
+
+def quantize_q8_1(x: int, out: int, K: int, batch: int = 1, x_dtype: int = F32) -> None:
+    _check(cu().bk_quantize_q8_1(x, x_dtype, out, K, batch), "bk_quantize_q8_1")
+
+
+def gemv_q4k_f32(W: int, x: int, y: int, N: int, K: int) -> None:
+    _check(cu().bk_gemv_q4k_f32(W, x, y, N, K), "bk_gemv_q4k_f32")
+
+
+def gemv_q4k_q8_1(W: int, xq: int, y: int, N: int, K: int, batch: int = 1, out_dtype: int = F32,
+                  residual: int = 0) -> None:
+    _check(cu().bk_gemv_q4k_q8_1(W, xq, y, N, K, batch, out_dtype, residual), "bk_gemv_q4k_q8_1")
+
+
+def q4k_q8_1_subdots(W: int, xq: int, I: int, N: int, K: int) -> None:
+    _check(cu().bk_q4k_q8_1_subdots(W, xq, I, N, K), "bk_q4k_q8_1_subdots")
+
+
+def dequant_legacy_i8(blocks: int, out: int, nblocks: int) -> None:
+    _check(cu().bk_dequant_legacy_i8(blocks, out, nblocks), "bk_dequant_legacy_i8")
+
+
+def q4k_nibbles(blocks: int, out: int, nblocks: int) -> None:
+    _check(cu().bk_q4k_nibbles(blocks, out, nblocks), "bk_q4k_nibbles")
+
+
+def q4k_dequant_f32(blocks: int, out: int, nblocks: int) -> None:
+    _check(cu().bk_q4k_dequant_f32(blocks, out, nblocks), "bk_q4k_dequant_f32")

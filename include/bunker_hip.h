@@ -1,0 +1,111 @@
+/*
+ * bunker_hip.h — C ABI of libbunker_hip.so: bunker's Qwen3.5 single-token decode
+ * hot path as pre-compiled gfx950 (MI355X) HIP kernels.
+ *
+ * The library replaces, for this path only, the two native boundaries of the
+ * reference: the Triton shim (shim/triton_shim.c:139-141, bound at
+ * src/ttir.ts:137-141) and the CUDA driver binding (src/ttir.ts:225-248), and it
+ * carries the kernels that src/emitters.ts and src/fusion.ts:264-355 used to
+ * generate.  Conventions, chosen so that bun:ffi, ctypes and plain C can all
+ * bind it:
+ *   - only scalars and raw pointers cross the boundary, never structs;
+ *   - device pointers are uint64_t (bun passes bigint, src/ttir.ts:266-271);
+ *   - every function returns int32: 0 = ok, < 0 = error; bk_last_error() then
+ *     returns a message owned by the library (thread-local, never freed by the
+ *     caller);
+ *   - one HIP stream per process; launches are asynchronous, bk_sync() waits;
+ *   - single-threaded use, like the reference (one JS thread, one context).
+ */
+#ifndef BUNKER_HIP_H
+#define BUNKER_HIP_H
+
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define BK_API __attribute__((visibility("default")))
+#else
+#define BK_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- runtime: replaces cu()/cuAlloc/cuHtoD/cuDtoH/cuFree/cuSync (src/ttir.ts:225-285) */
+BK_API int bk_init(int device);                      /* cuInit + cuCtxCreate, src/ttir.ts:249-258 */
+BK_API int bk_shutdown(void);
+BK_API const char* bk_last_error(void);              /* the "ERROR:" string of triton_shim.c:146-149 */
+BK_API int bk_device_info(char* buf, int cap);       /* "name|gcnArch|CUs|bytes" for logs */
+BK_API int bk_alloc(uint64_t bytes, uint64_t* out);  /* cuAlloc, src/ttir.ts:266-271 */
+BK_API int bk_free(uint64_t ptr);                    /* cuFree, src/ttir.ts:283 */
+BK_API int bk_htod(uint64_t dst, const void* src, uint64_t bytes);   /* cuHtoD, src/ttir.ts:273-276 */
+BK_API int bk_dtoh(void* dst, uint64_t src, uint64_t bytes);         /* cuDtoH, src/ttir.ts:278-281 */
+BK_API int bk_dtod(uint64_t dst, uint64_t src, uint64_t bytes);
+BK_API int bk_memset(uint64_t dst, int value, uint64_t bytes);
+BK_API int bk_sync(void);                            /* cuSync, src/ttir.ts:285 */
+
+/* ---- timing: replaces the cuEvent* calls of src/ttir.ts:352-417 */
+BK_API int bk_event_create(uint64_t* out);
+BK_API int bk_event_record(uint64_t ev);             /* on the library's stream */
+BK_API int bk_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms);  /* waits for stop */
+BK_API int bk_event_destroy(uint64_t ev);
+BK_API int bk_prof_enable(int on);                   /* BUNKER_GPU_PROF=1: an event pair around every bk_launch */
+BK_API int bk_prof_reset(void);                      /* profGpuReset, src/ttir.ts:385-388 */
+BK_API int bk_prof_report(char* buf, int cap);       /* profGpuReport, src/ttir.ts:391-417; text table */
+
+/* ---- launch-overhead removal: record everything enqueued between begin and end
+ * into a HIP graph (stream capture) and replay it with one call.  The reference
+ * tried the same with CUDA graphs through bun:ffi and gave up on struct-pointer
+ * crashes (LOG.md:710-738); here the graph lives behind scalar handles.
+ * Between begin and end only launches are legal: no alloc, free, copy to or from
+ * the host, sync or event call. */
+BK_API int bk_capture_begin(void);
+BK_API int bk_capture_end(uint64_t* graph);
+BK_API int bk_graph_launch(uint64_t graph);
+BK_API int bk_graph_destroy(uint64_t graph);
+
+/* ---- per-op launch surface: replaces compileAndLoad + cuLaunch
+ * (src/ttir.ts:488-491, 321-348).  bk_kernel_create takes the op name of the
+ * model graph (src/model.ts) and the constants that the reference baked into
+ * the TTIR text, e.g. "gemm N=6144 K=2048 cast=1", and returns a handle >= 0
+ * (the LoadedKernel.fn of the reference).  bk_launch takes the same 8-byte
+ * argument slots cuLaunch packs, in the same order (pointers as u64, i32
+ * scalars in the low 4 bytes); grid and block are the kernel's own business. */
+BK_API int bk_kernel_create(const char* spec);
+BK_API int bk_launch(int kernel, const uint64_t* slots, int nslots);
+BK_API int bk_kernel_describe(int kernel, char* buf, int cap);
+
+/* ---- typed entry points (C / ctypes drivers, parity tests, benchmark) ---- */
+
+/* Q8_1 activation quantizer: packQ8_1, bench/bench.ts:53-72 (host-only in the
+ * reference).  x is [batch, K] f32 (x_dtype 0) or bf16 (1); out is
+ * [batch, K/32] blocks of 36 bytes: int8 q[32] @0, fp16 d @32, fp16 s @34. */
+BK_API int bk_quantize_q8_1(uint64_t x, int x_dtype, uint64_t out, int K, int batch);
+
+/* Q4_K dequantize + f32 GEMV on 144-byte super-blocks: y[N] = W[N,K] . x[K],
+ * x f32.  The dequant-then-dot the reference's CPU path computes (packers and
+ * dot of bench/bench.ts:10-96) with no activation quantization. */
+BK_API int bk_gemv_q4k_f32(uint64_t W, uint64_t x, uint64_t y, int N, int K);
+
+/* Q4_K x Q8_1 GEMV: qmm, bench/bench.ts:10-38, on super-blocks; the decode
+ * path's M=1 "gemm" (src/fusion.ts:276-293, prototypes/decode.ts:123-186).
+ * y is f32 [batch, N] (out_dtype 0) or bf16 (1, the graph's cast=true);
+ * residual (0 or bf16 [batch, N]) is added after the bf16 rounding, giving
+ * bf16(f32(bf16(acc)) + f32(res)): model.ts:110-117's gemm -> cast -> add. */
+BK_API int bk_gemv_q4k_q8_1(uint64_t W, uint64_t xq, uint64_t y, int N, int K, int batch,
+                     int out_dtype, uint64_t residual);
+
+/* Exact int32 sub-block dots I[N, K/32] of the same product (parity hook). */
+BK_API int bk_q4k_q8_1_subdots(uint64_t W, uint64_t xq, uint64_t I, int N, int K);
+
+/* Nibble dequant kernels: DequantKernel, src/kernel.ts:584-713.
+ * legacy: 20-byte blocks -> int8 (nib-8), interleaved lo/hi (tests/test_dequant.ts:13-24).
+ * q4k:    144-byte super-blocks -> uint8 nibbles in element order, or f32 weights. */
+BK_API int bk_dequant_legacy_i8(uint64_t blocks, uint64_t out, int64_t nblocks);
+BK_API int bk_q4k_nibbles(uint64_t blocks, uint64_t out, int64_t nblocks);
+BK_API int bk_q4k_dequant_f32(uint64_t blocks, uint64_t out, int64_t nblocks);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BUNKER_HIP_H */

@@ -1,0 +1,59 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every declared symbol, and
+refuses work cleanly when there is no device (no kernel is launched here)."""
+import ctypes as C
+import os
+
+import pytest
+
+from bunker_amd import runtime as rt
+
+
+def _lib_or_skip():
+    if not os.path.exists(rt.LIB_PATH):
+        pytest.fail(f"{rt.LIB_PATH} not built: run `make -C bunker_amd/csrc`")
+    return rt.load_library(rt.LIB_PATH)
+
+
+def test_header_symbols_are_exported():
+    lib = _lib_or_skip()
+    names = rt.declared_symbols()
+    assert len(names) >= 32 and len(set(names)) == len(names)
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    # the Python binding table covers the header exactly
+    assert set(rt._SIGS) | {"bk_last_error"} == set(names)
+
+
+def test_calls_before_init_fail_with_message():
+    lib = _lib_or_skip()
+    out = C.c_uint64(0)
+    rc = lib.bk_alloc(1024, C.byref(out))
+    if rc == 0:          # a GPU box where another test already initialised the library
+        lib.bk_free(out)
+        pytest.skip("library already initialised")
+    assert rc < 0
+    assert b"bk_init" in lib.bk_last_error()
+    assert lib.bk_gemv_q4k_q8_1(0, 0, 0, 16, 256, 1, 0, 0) < 0
+    assert lib.bk_kernel_create(b"gemm N=16 K=256") < 0
+
+
+def test_init_without_gpu_reports_no_device():
+    import subprocess, sys
+    # run in a child: bk_init touches the HIP runtime
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "from bunker_amd import runtime as rt\n"
+        "lib = rt.load_library()\n"
+        "rc = lib.bk_init(0)\n"
+        "print(rc, lib.bk_last_error().decode())\n" % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    rc, _, msg = r.stdout.strip().partition(" ")
+    if int(rc) == 0:
+        pytest.skip("a GPU is present")
+    assert int(rc) < 0 and ("no HIP device" in msg or "gfx950" in msg), r.stdout
+
+
+def test_missing_library_raises():
+    with pytest.raises(rt.BunkerError, match="no CPU fallback"):
+        rt.load_library("/nonexistent/libbunker_hip.so")
