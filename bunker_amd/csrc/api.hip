@@ -74,8 +74,126 @@ static int run_gemm(Kernel& k, const uint64_t* s) {
   return launch_gemv_q4k_q8_1(P<void>(s[1]), k.scratch, P<void>(s[2]), N, K, batch, (int)k.get("cast", 0), nullptr);
 }
 
+// ---- op: embed (src/model.ts:53-56)   slots: embed.weight, token_id, out
+// params: H, VOCAB, batch=1, ids_dev=0 (1: slot 1 is a device pointer to int32 [batch])
+static int run_embed(Kernel& k, const uint64_t* s) {
+  const bool dev = k.get("ids_dev", 0) != 0;
+  return launch_embed(P<void>(s[0]), dev ? P<int32_t>(s[1]) : nullptr, dev ? 0 : (int32_t)(uint32_t)s[1], P<void>(s[2]),
+                      (int)k.get("H", 0), (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
+}
+// ---- op: rmsnorm (src/model.ts:65-67)   slots: x, w, out     params: N, batch=1
+static int run_rmsnorm(Kernel& k, const uint64_t* s) {
+  return launch_rmsnorm(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), nullptr, (int)k.get("N", 0), (int)k.get("batch", 1));
+}
+// ---- op: rmsnorm_q8_1   slots: x, w, out (bf16, may be 0), xq (Q8_1)   params: N, batch=1
+static int run_rmsnorm_q8(Kernel& k, const uint64_t* s) {
+  return launch_rmsnorm(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), (int)k.get("N", 0), (int)k.get("batch", 1));
+}
+// ---- ops: cast (x, out), add (a, b, out), swiglu (g, u, out)   params: N, batch=1
+static int run_cast(Kernel& k, const uint64_t* s) {
+  return launch_elementwise(EW_CAST_OP, P<void>(s[0]), nullptr, P<void>(s[1]), k.get("N", 0) * k.get("batch", 1));
+}
+static int run_add(Kernel& k, const uint64_t* s) {
+  return launch_elementwise(EW_ADD_OP, P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), k.get("N", 0) * k.get("batch", 1));
+}
+static int run_swiglu(Kernel& k, const uint64_t* s) {
+  return launch_elementwise(EW_SWIGLU_OP, P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), k.get("N", 0) * k.get("batch", 1));
+}
+// ---- op: conv1d_decode (src/model.ts:77-87)   slots: qkv, conv_state_in, weight, out, conv_state_new
+static int run_conv1d(Kernel& k, const uint64_t* s) {
+  return launch_conv1d_decode(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), (int)k.get("QKVD", 0),
+                              (int)k.get("batch", 1));
+}
+// ---- op: gdn_delta_rule (src/model.ts:94-109)
+// slots: conv_out, z, A_log, dt_bias, a_p, b_p, norm_w, s_state_in, out, s_state_new     params: LVH, batch=1
+static int run_gdn(Kernel& k, const uint64_t* s) {
+  return launch_gdn_fused(P<void>(s[0]), P<void>(s[1]), P<float>(s[2]), P<void>(s[3]), P<float>(s[4]), P<float>(s[5]),
+                          P<float>(s[6]), P<float>(s[7]), P<void>(s[8]), P<float>(s[9]), (int)k.get("LVH", 0), (int)k.get("batch", 1));
+}
+// ---- ops: qnorm (q-gate buffer, w, out; NH heads, input rows 2*HD apart), knorm (k, w, out; NKV heads)
+static int run_qnorm(Kernel& k, const uint64_t* s) {
+  const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0);
+  return launch_headnorm(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), NH, HD, 2 * HD, (int64_t)NH * 2 * HD, (int)k.get("batch", 1),
+                         nullptr, nullptr, nullptr, 0, 0, 0);
+}
+static int run_knorm(Kernel& k, const uint64_t* s) {
+  const int HD = (int)k.get("HD", 0), NKV = (int)k.get("NKV", 0);
+  return launch_headnorm(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), NKV, HD, HD, (int64_t)NKV * HD, (int)k.get("batch", 1),
+                         nullptr, nullptr, nullptr, 0, 0, 0);
+}
+// ---- ops: rope / ropek (src/model.ts:133-143)   slots: Q (in place), rope_cos, rope_sin, pos
+// params: HD, NH | NKV, ROT_HALF, MAX_LEN, batch=1, pos_dev=0 (1: slot 3 is a device pointer to int32 [batch])
+static int run_rope(Kernel& k, const uint64_t* s) {
+  const bool dev = k.get("pos_dev", 0) != 0;
+  const int nh = (int)(k.has("NH") ? k.get("NH", 0) : k.get("NKV", 0));
+  return launch_rope(P<void>(s[0]), P<float>(s[1]), P<float>(s[2]), dev ? P<int32_t>(s[3]) : nullptr, dev ? 0 : (int)(int32_t)s[3],
+                     nh, (int)k.get("HD", 0), (int)k.get("ROT_HALF", 0), (int)k.get("MAX_LEN", 0), (int)k.get("batch", 1));
+}
+// ---- op: fa2_attn (src/model.ts:144-157)
+// slots: q, k, v, qgate, kv_k_in, kv_v_in, pos, out, kv_k_new, kv_v_new; like the reference's emitter only
+// kv_*_in are touched (the caller maps in and new to one buffer).  This step's k, v go into the cache at
+// pos, then the query attends to tokens 0..pos.  Each sequence owns MAX_LEN/16 consecutive pages.
+// params: HD, NH, NKV, MAX_LEN, batch=1, pos_dev=0
+static int run_fa2(Kernel& k, const uint64_t* s) {
+  const bool dev = k.get("pos_dev", 0) != 0;
+  const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0), NKV = (int)k.get("NKV", 0), batch = (int)k.get("batch", 1);
+  const int max_len = (int)k.get("MAX_LEN", 0), bt_stride = (max_len + 15) / 16;
+  const int32_t* pos_dev = dev ? P<int32_t>(s[6]) : nullptr;
+  const int pos = dev ? 0 : (int)(int32_t)s[6];
+  if (!dev) BK_REQUIRE(pos >= 0 && pos < max_len, "fa2_attn: pos=%d outside the cache (MAX_LEN=%d)", pos, max_len);
+  int rc = launch_kv_append(P<void>(s[1]), P<void>(s[2]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, batch, NKV, HD, 16);
+  if (rc) return rc;
+  // the context of each sequence is its pos + 1
+  return launch_attn_decode(P<void>(s[0]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, 1, max_len,
+                            P<uint16_t>(s[3]) + HD, (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[7]), nullptr, k.scratch, k.scratch_bytes,
+                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
+}
+// ---- op: argmax (src/model.ts:198-201)   slots: logits, val, idx     params: VOCAB, batch=1
+static int run_argmax(Kernel& k, const uint64_t* s) {
+  return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
+}
+
 static int build_kernel(Kernel& k) {
   int rc;
+  struct Simple { const char* op; RunFn run; int nslots; const char* need1; const char* need2; };
+  static const Simple simple[] = {
+      {"embed", run_embed, 3, "H", "VOCAB"},       {"rmsnorm", run_rmsnorm, 3, "N", nullptr},
+      {"rmsnorm_q8_1", run_rmsnorm_q8, 4, "N", nullptr}, {"cast", run_cast, 2, "N", nullptr},
+      {"add", run_add, 3, "N", nullptr},            {"swiglu", run_swiglu, 3, "N", nullptr},
+      {"conv1d_decode", run_conv1d, 5, "QKVD", nullptr}, {"gdn_delta_rule", run_gdn, 10, "LVH", nullptr},
+      {"qnorm", run_qnorm, 3, "HD", "NH"},          {"knorm", run_knorm, 3, "HD", "NKV"},
+      {"rope", run_rope, 4, "HD", "NH"},            {"ropek", run_rope, 4, "HD", "NKV"},
+  };
+  for (const Simple& sp : simple) {
+    if (k.op != sp.op) continue;
+    if ((rc = need(k, sp.need1))) return rc;
+    if (sp.need2 && (rc = need(k, sp.need2))) return rc;
+    if (k.op == "rope" || k.op == "ropek") {
+      if ((rc = need(k, "ROT_HALF")) || (rc = need(k, "MAX_LEN"))) return rc;
+    }
+    if (k.op == "gdn_delta_rule")
+      BK_REQUIRE(k.get("LKD", 128) == 128 && k.get("LVD", 128) == 128, "gdn_delta_rule: dk = dv = 128 only");
+    k.run = sp.run; k.nslots = sp.nslots;
+    return BK_OK;
+  }
+  if (k.op == "fa2_attn") {
+    if ((rc = need(k, "HD")) || (rc = need(k, "NH")) || (rc = need(k, "NKV")) || (rc = need(k, "MAX_LEN"))) return rc;
+    const int batch = (int)k.get("batch", 1), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
+    BK_REQUIRE(batch >= 1 && NKV >= 1 && max_len >= 1, "fa2_attn: bad batch/NKV/MAX_LEN");
+    int splits = (int)k.get("splits", 0);
+    if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
+    if (splits > 1 && (rc = alloc_scratch(k, attn_workspace_bytes(batch, NKV, splits)))) return rc;
+    k.run = run_fa2; k.nslots = 10;
+    return BK_OK;
+  }
+  if (k.op == "argmax") {
+    if ((rc = need(k, "VOCAB"))) return rc;
+    const int batch = (int)k.get("batch", 1), V = (int)k.get("VOCAB", 0);
+    BK_REQUIRE(batch >= 1 && V >= 1, "argmax: bad VOCAB/batch");
+    if ((rc = alloc_scratch(k, argmax_workspace_bytes(V, batch)))) return rc;
+    k.run = run_argmax; k.nslots = 3;
+    return BK_OK;
+  }
   if (k.op == "quantize_q8_1") {
     if ((rc = need(k, "K"))) return rc;
     k.run = run_quantize; k.nslots = 2;
@@ -177,6 +295,40 @@ int bk_q4k_nibbles(uint64_t blocks, uint64_t out, int64_t nblocks) {
 int bk_q4k_dequant_f32(uint64_t blocks, uint64_t out, int64_t nblocks) {
   BK_NEED_INIT();
   return launch_q4k_dequant_f32(P<void>(blocks), P<void>(out), nblocks);
+}
+
+int bk_gdn_core(uint64_t q, uint64_t k, uint64_t v, uint64_t g, uint64_t beta, uint64_t S_in, uint64_t out, uint64_t S_out,
+                int Hg, int batch) {
+  BK_NEED_INIT();
+  return launch_gdn_core(P<void>(q), P<void>(k), P<void>(v), P<float>(g), P<float>(beta), P<float>(S_in), P<void>(out),
+                         P<float>(S_out), Hg, batch);
+}
+int bk_attn_plan(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(splits && workspace_bytes, "bk_attn_plan: null out");
+  BK_REQUIRE(batch > 0 && NKV > 0 && max_ctx > 0, "bk_attn_plan: bad shape");
+  int s = *splits > 0 ? *splits : attn_choose_splits(batch, NKV, max_ctx);
+  const int pages = (max_ctx + 15) / 16;
+  if (s > pages) s = pages;
+  *splits = s;
+  *workspace_bytes = s > 1 ? attn_workspace_bytes(batch, NKV, s) : 0;
+  return BK_OK;
+}
+int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t ctx_len, int max_ctx,
+                   uint64_t gate, int64_t gate_bstride, int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
+                   uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size, int splits) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ctx_len, "bk_attn_decode: ctx_len is required");
+  return launch_attn_decode(P<void>(q), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride, P<int32_t>(ctx_len), 0, 0,
+                            max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse), P<void>(workspace),
+                            (size_t)workspace_bytes, batch, NH, NKV, HD, page_size, splits);
+}
+int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t pos, int batch,
+                 int NKV, int HD, int page_size) {
+  BK_NEED_INIT();
+  BK_REQUIRE(pos, "bk_kv_append: pos is required");
+  return launch_kv_append(P<void>(k), P<void>(v), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride, P<int32_t>(pos), 0,
+                          batch, NKV, HD, page_size);
 }
 
 }  // extern "C"

@@ -1,0 +1,290 @@
+// Split-K decode attention over a paged bf16 GQA KV cache (one query token per
+// sequence).  Math of src/emitters.ts:188-226 (scores * 1/sqrt(HD) over the valid
+// prefix, softmax, sum p*V, optional * sigmoid(gate)) with the log-sum-exp returned,
+// on a cache that is shared by the query heads of a KV group and cut into 16-token
+// pages.
+//
+// Cache layout (per layer; one array for K, one for V; HD = 256, page = 16 tokens):
+//   K page p, kv head h:  bf16 [16 tok][256 dim]   at ((p*NKV + h) * 4096) elements
+//   V page p, kv head h:  bf16 [256 dim][16 tok]   at ((p*NKV + h) * 4096) elements
+// V is stored dim-major inside the page so that both matrix products read their
+// MFMA operands straight from global memory with contiguous 16/8-byte pieces:
+//   S^T[tok, head] = sum_d K[tok, d] * Q[head, d]        v_mfma_f32_16x16x32_bf16, A = K page
+//   O^T[d, head]   = sum_tok V^T[d, tok] * P^T[tok, head] v_mfma_f32_16x16x16_bf16, A = V page,
+// and P^T comes out of the first product in exactly the register layout the second
+// wants as its B operand.  The query heads of a KV group (<= 16) are the N dimension.
+//
+// grid = (splits, NKV, B), 4 waves per workgroup.  Each wave walks pages of its
+// split with its own running (max, sum, O^T); the four are merged through LDS in a
+// fixed order; with more than one split the workgroup partials go to a workspace
+// and a second kernel merges them, again in a fixed order.
+#include "ops.h"
+
+namespace bk {
+
+constexpr int ATT_HD = 256;
+constexpr int ATT_PAGE = 16;
+constexpr int ATT_WAVES = 4;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+struct AttnArgs {
+  const uint16_t* q;          // bf16 [B, NH, 256]
+  const uint16_t* kc;         // K pages
+  const uint16_t* vc;         // V pages (dim-major inside a page)
+  const int32_t* block_table; // int32 [B, bt_stride]; null = identity (page i of sequence b is b*bt_stride + i)
+  const int32_t* ctx_len;     // int32 [B]; null = ctx_scalar for every sequence; ctx_add is added to either
+  const uint16_t* gate;       // bf16 or null: gate of (b, head, i) at gate[b*gate_bstride + head*gate_hstride + i]
+  uint16_t* out;              // bf16 [B, NH, 256]
+  float* lse;                 // f32 [B, NH] or null
+  float* part_o;              // f32 [B, NKV, splits, 16, 256] unnormalised partial outputs
+  float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
+  int64_t gate_bstride, gate_hstride;
+  int bt_stride, ctx_scalar, ctx_add, NH, NKV, G, splits, pages_per_split;
+  float scale;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+__global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A) {
+  __shared__ float lds_o[ATT_HD][16];           // merged O^T, 16 KiB
+  __shared__ float lds_m[ATT_WAVES][16], lds_l[ATT_WAVES][16];
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 15, kg = lane >> 4;      // n: token (A operand) / head (B operand, C column); kg: lane group
+  const int len = (A.ctx_len ? A.ctx_len[b] : A.ctx_scalar) + A.ctx_add;
+  const int npages = (len + ATT_PAGE - 1) / ATT_PAGE;
+  const int p_begin = split * A.pages_per_split;
+  const int p_end = min(npages, p_begin + A.pages_per_split);
+
+  // Q as the B operand of the first product: lane (head n, group kg) holds dims 32*s + 8*kg .. +8
+  uint4 qreg[8];
+  {
+    const bool valid = n < A.G;
+    const uint16_t* qp = A.q + ((int64_t)b * A.NH + kvh * A.G + (valid ? n : 0)) * ATT_HD + 8 * kg;
+#pragma unroll
+    for (int s = 0; s < 8; s++) qreg[s] = valid ? *(const uint4*)(qp + 32 * s) : make_uint4(0, 0, 0, 0);
+  }
+
+  f32x4_t oacc[16];
+#pragma unroll
+  for (int t = 0; t < 16; t++) oacc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY;     // running max of head n (same in the 4 lanes that share n)
+  float l_run = 0.0f;          // this lane's share of the running sum (tokens 4*kg .. 4*kg+3 of every page)
+
+  for (int pg = p_begin + wave; pg < p_end; pg += ATT_WAVES) {
+    const int phys = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + pg] : b * A.bt_stride + pg;
+    const int64_t base = ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
+    // K page as the A operand: lane (token n, group kg) holds dims 32*s + 8*kg .. +8
+    const uint16_t* kp = A.kc + base + n * ATT_HD + 8 * kg;
+    uint4 kreg[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++) kreg[s] = *(const uint4*)(kp + 32 * s);
+    // V page as the A operand: lane (dim 16*t + n, group kg) holds tokens 4*kg .. +4
+    const uint16_t* vp = A.vc + base + n * ATT_PAGE + 4 * kg;
+    uint2 vreg[16];
+#pragma unroll
+    for (int t = 0; t < 16; t++) vreg[t] = *(const uint2*)(vp + t * 16 * ATT_PAGE);
+
+    f32x4_t s4 = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kreg[s]), __builtin_bit_cast(bf16x8_t, qreg[s]),
+                                                   s4, 0, 0, 0);
+    // lane holds S^T[token 4*kg + r][head n], r = 0..3
+    float sc[4];
+    const int tok0 = pg * ATT_PAGE + 4 * kg;
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      sc[r] = (tok0 + r < len) ? s4[r] * A.scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[r]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float m_new = fmaxf(m_run, tmax);        // finite: every page in range holds at least one valid token
+    const float alpha = __expf(m_run - m_new);     // exp(-inf) = 0 on the first page
+    float p[4], psum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) { p[r] = __expf(sc[r] - m_new); psum += p[r]; }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (alpha != 1.0f) {
+#pragma unroll
+      for (int t = 0; t < 16; t++) { oacc[t][0] *= alpha; oacc[t][1] *= alpha; oacc[t][2] *= alpha; oacc[t][3] *= alpha; }
+    }
+    const uint2 pb = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
+#pragma unroll
+    for (int t = 0; t < 16; t++)
+      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pb),
+                                                          oacc[t], 0, 0, 0);
+  }
+
+  // ---- merge the four waves (fixed order 0,1,2,3)
+  float l_tot = l_run + __shfl_xor(l_run, 16);
+  l_tot += __shfl_xor(l_tot, 32);
+  if (kg == 0) { lds_m[wave][n] = m_run; lds_l[wave][n] = l_tot; }
+  __syncthreads();
+  float M = lds_m[0][n];
+#pragma unroll
+  for (int w = 1; w < ATT_WAVES; w++) M = fmaxf(M, lds_m[w][n]);
+  const float wscale = (m_run == -INFINITY) ? 0.0f : __expf(m_run - M);
+  float L = 0.0f;
+#pragma unroll
+  for (int w = 0; w < ATT_WAVES; w++) {
+    const float mw = lds_m[w][n];
+    L += (mw == -INFINITY) ? 0.0f : lds_l[w][n] * __expf(mw - M);
+  }
+  for (int w = 0; w < ATT_WAVES; w++) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < 16; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          float* dst = &lds_o[16 * t + 4 * kg + r][n];
+          const float v = oacc[t][r] * wscale;
+          *dst = (w == 0) ? v : (*dst + v);
+        }
+    }
+    __syncthreads();
+  }
+
+  // ---- write: thread = dim, loop over the G heads of the group
+  const int d = threadIdx.x;   // 0..255
+  if (A.splits == 1) {
+    for (int h = 0; h < A.G; h++) {
+      const int head = kvh * A.G + h;
+      // M and L live in the lanes with n == h; fetch them through LDS
+      float Mh = lds_m[0][h];
+      for (int w = 1; w < ATT_WAVES; w++) Mh = fmaxf(Mh, lds_m[w][h]);
+      float Lh = 0.0f;
+      for (int w = 0; w < ATT_WAVES; w++) {
+        const float mw = lds_m[w][h];
+        Lh += (mw == -INFINITY) ? 0.0f : lds_l[w][h] * __expf(mw - Mh);
+      }
+      float o = lds_o[d][h] / Lh;
+      if (A.gate) {
+        const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
+        o = o * (1.0f / (1.0f + expf(gv * -1.0f)));
+      }
+      A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
+      if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = Mh + logf(Lh);
+    }
+  } else {
+    const int64_t pidx = ((int64_t)b * A.NKV + kvh) * A.splits + split;
+    float* po = A.part_o + pidx * 16 * ATT_HD;
+    for (int h = 0; h < A.G; h++) po[h * ATT_HD + d] = lds_o[d][h];
+    if (kg == 0 && wave == 0 && n < A.G) {
+      A.part_ml[(pidx * 16 + n) * 2] = M;
+      A.part_ml[(pidx * 16 + n) * 2 + 1] = L;
+    }
+  }
+}
+
+// Merge of the split partials: one workgroup per (head, batch), thread = dim.
+__global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int kvh = head / A.G, h = head % A.G;
+  const int64_t p0 = ((int64_t)b * A.NKV + kvh) * A.splits;
+  float M = -INFINITY;
+  for (int s = 0; s < A.splits; s++) M = fmaxf(M, A.part_ml[((p0 + s) * 16 + h) * 2]);
+  float L = 0.0f, o = 0.0f;
+  for (int s = 0; s < A.splits; s++) {
+    const float ms = A.part_ml[((p0 + s) * 16 + h) * 2];
+    if (ms == -INFINITY) continue;
+    const float w = __expf(ms - M);
+    L += A.part_ml[((p0 + s) * 16 + h) * 2 + 1] * w;
+    o += A.part_o[((p0 + s) * 16 + h) * ATT_HD + d] * w;
+  }
+  o = o / L;
+  if (A.gate) {
+    const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
+    o = o * (1.0f / (1.0f + expf(gv * -1.0f)));
+  }
+  A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
+  if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = M + logf(L);
+}
+
+size_t attn_workspace_bytes(int batch, int NKV, int max_splits) {
+  return (size_t)batch * NKV * max_splits * 16 * (ATT_HD + 2) * sizeof(float);
+}
+
+int attn_choose_splits(int batch, int NKV, int max_ctx) {
+  const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
+  // aim at ~4 workgroups per CU, but keep at least 8 pages (2 per wave) in a split
+  int want = (4 * num_cus() + batch * NKV - 1) / (batch * NKV);
+  int cap = (pages + 7) / 8;
+  int s = want < cap ? want : cap;
+  return s < 1 ? 1 : (s > 256 ? 256 : s);
+}
+
+int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
+                       const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
+                       int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
+                       int NH, int NKV, int HD, int page_size, int splits) {
+  BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
+  BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
+  BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
+  BK_REQUIRE(batch > 0 && batch <= 65535 && NKV <= 65535, "attn_decode: bad batch=%d", batch);
+  BK_REQUIRE(ctx_len || ctx_scalar + ctx_add >= 1, "attn_decode: context length must be >= 1");
+  BK_REQUIRE(max_ctx >= 1 && (ctx_len || ctx_scalar + ctx_add <= max_ctx), "attn_decode: context %d exceeds max_ctx=%d", ctx_scalar + ctx_add, max_ctx);
+  BK_REQUIRE(bt_stride >= (max_ctx + ATT_PAGE - 1) / ATT_PAGE, "attn_decode: block table rows hold %d pages, context needs %d", bt_stride, (max_ctx + ATT_PAGE - 1) / ATT_PAGE);
+  BK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kc & 15) == 0 && ((uintptr_t)vc & 15) == 0, "attn_decode: q, K and V must be 16-byte aligned");
+  if (splits <= 0) splits = attn_choose_splits(batch, NKV, max_ctx);
+  const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
+  if (splits > pages) splits = pages;
+  AttnArgs A{};
+  A.q = (const uint16_t*)q; A.kc = (const uint16_t*)kc; A.vc = (const uint16_t*)vc;
+  A.block_table = block_table; A.ctx_len = ctx_len; A.gate = (const uint16_t*)gate;
+  A.out = (uint16_t*)out; A.lse = lse;
+  A.gate_bstride = gate_bstride; A.gate_hstride = gate_hstride;
+  A.bt_stride = bt_stride; A.ctx_scalar = ctx_scalar; A.ctx_add = ctx_add; A.NH = NH; A.NKV = NKV; A.G = NH / NKV;
+  A.splits = splits; A.pages_per_split = (pages + splits - 1) / splits;
+  A.scale = (float)(1.0 / sqrt((double)HD));
+  if (splits > 1) {
+    BK_REQUIRE(workspace && workspace_bytes >= attn_workspace_bytes(batch, NKV, splits),
+               "attn_decode: workspace of %zu bytes needed for %d splits", attn_workspace_bytes(batch, NKV, splits), splits);
+    A.part_o = (float*)workspace;
+    A.part_ml = A.part_o + (size_t)batch * NKV * splits * 16 * ATT_HD;
+  }
+  hipLaunchKernelGGL(attn_decode_kernel, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
+  if (splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, batch), dim3(256), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- cache append
+// The cache write of src/emitters.ts:202-205: token `pos` of every sequence gets this
+// step's k and v (bf16 [B, NKV, 256]); V goes in dim-major.
+__global__ __launch_bounds__(256) void kv_append_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                                                        uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                                        const int32_t* __restrict__ block_table, int bt_stride,
+                                                        const int32_t* __restrict__ pos_dev, int pos_scalar, int NKV) {
+  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  const int pg = pos / ATT_PAGE, slot = pos % ATT_PAGE;
+  const int phys = block_table ? block_table[(int64_t)b * bt_stride + pg] : b * bt_stride + pg;
+  const int64_t base = ((int64_t)phys * NKV + kvh) * (ATT_PAGE * ATT_HD);
+  const int64_t src = ((int64_t)b * NKV + kvh) * ATT_HD + d;
+  kc[base + slot * ATT_HD + d] = k[src];
+  vc[base + d * ATT_PAGE + slot] = v[src];
+}
+
+int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
+                     const int32_t* pos_dev, int pos_scalar, int batch, int NKV, int HD, int page_size) {
+  BK_REQUIRE(k && v && kc && vc, "kv_append: null pointer");
+  BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "kv_append: head_dim 256 and 16-token pages only");
+  BK_REQUIRE(batch > 0 && batch <= 65535 && NKV > 0 && NKV <= 65535, "kv_append: bad shape");
+  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar / ATT_PAGE < bt_stride), "kv_append: pos=%d outside the block table", pos_scalar);
+  hipLaunchKernelGGL(kv_append_kernel, dim3(NKV, batch), dim3(256), 0, stream(), (const uint16_t*)k, (const uint16_t*)v,
+                     (uint16_t*)kc, (uint16_t*)vc, block_table, bt_stride, pos_dev, pos_scalar, NKV);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

@@ -1,0 +1,197 @@
+// Gated DeltaNet single-token recurrent update (src/emitters.ts:75-120,
+// prototypes/decode.ts:314-388; recurrence of prototypes/gdn_gated.ts:67-88).
+//
+//   Sd = g*S ; kS[v] = sum_k k^[k]*Sd[k,v] ; delta = (v - kS)*beta
+//   S' = Sd + k^ (x) delta ; o[v] = sum_k q^[k]*S'[k,v]
+//
+// S is f32 [B, Hg, 128(k), 128(v)], row-major.  Every v column is independent, so a
+// head is cut into CS column slabs, one 256-thread workgroup each.  A thread owns
+// ROWS k-rows x 4 v-columns of the slab in registers for the whole step: S is read
+// from HBM once (float4, rows of the slab contiguous) and S' written once; the two
+// k-reductions are in-thread sums over the owned rows plus one LDS exchange across
+// the row groups, in a fixed order.
+#include "ops.h"
+
+namespace bk {
+
+constexpr int GDN_D = 128;          // dk = dv = 128
+constexpr int GDN_THREADS = 256;
+
+struct GdnArgs {
+  // q, k, v: bf16, element (b, h, i) at ptr[b*bstride + h*128 + i]
+  const uint16_t *q, *k, *v;
+  int64_t qkv_bstride;
+  // fused mode (src/emitters.ts:86-99): decay and beta from A_log, dt_bias, a_p, b_p; gated RMSNorm with z, norm_w
+  const uint16_t* z;        // bf16 [B, Hg*128]
+  const float* A_log;       // f32 [Hg]
+  const uint16_t* dt_bias;  // bf16 [Hg]
+  const float* a_p;         // f32 [B, Hg]
+  const float* b_p;         // f32 [B, Hg]
+  const float* norm_w;      // f32 [128]
+  // core mode: decay = exp(g), beta given; q, k used as they are
+  const float* g;           // f32 [B, Hg]
+  const float* beta;        // f32 [B, Hg]
+  const float* S_in;
+  float* S_out;
+  uint16_t* out;            // bf16 [B, Hg*128]
+  int Hg;
+};
+
+template <int CS, bool FUSED>
+__global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
+  constexpr int COLS = GDN_D / CS;          // v columns of this workgroup
+  constexpr int VQ = COLS / 4;              // float4 column groups
+  constexpr int KG = GDN_THREADS / VQ;      // k-row groups
+  constexpr int ROWS = GDN_D / KG;          // rows per thread
+  static_assert(!FUSED || CS == 1, "the gated norm needs the whole head in one workgroup");
+  __shared__ float kn[GDN_D], qn[GDN_D];
+  __shared__ float part[KG][COLS];
+  __shared__ float red[4];
+
+  const int h = blockIdx.x, slab = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int vq = tid % VQ, kg = tid / VQ;
+  const int col0 = slab * COLS + vq * 4;    // first of the thread's 4 columns (within the head)
+  const int64_t bh = (int64_t)b * A.Hg + h;
+
+  // S rows go out first: the loads are in flight while q, k and the gates are prepared
+  const float* Sp = A.S_in + bh * GDN_D * GDN_D;
+  float4 S[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) S[r] = *(const float4*)(Sp + (int64_t)(kg * ROWS + r) * GDN_D + col0);
+
+  const uint16_t* qp = A.q + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* kp = A.k + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* vp = A.v + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  float decay, beta;
+  if (FUSED) {
+    // waves 0,1 hold q (2 values per lane... 128 values over 128 threads), waves 2,3 hold k
+    const bool isk = tid >= 128;
+    const int i = tid & 127;
+    const float x = bf16_to_f32((isk ? kp : qp)[i]);
+    float ss = wave_sum(x * x);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float tot = isk ? (red[2] + red[3]) : (red[0] + red[1]);
+    const float rs = 1.0f / sqrtf(tot + 1e-6f);
+    if (isk) kn[i] = x * rs;
+    else qn[i] = x * (rs * 0.08838834764831845f);     // 1/sqrt(128)
+    const float sp_in = A.a_p[bh] + bf16_to_f32(A.dt_bias[h]);
+    const float softplus = log2f(1.0f + expf(sp_in)) * 0.6931471805599453f;
+    decay = expf(-1.0f * (expf(A.A_log[h]) * softplus));
+    beta = 1.0f / (1.0f + expf(A.b_p[bh] * -1.0f));
+  } else {
+    if (tid < 128) qn[tid] = bf16_to_f32(qp[tid]);
+    else kn[tid - 128] = bf16_to_f32(kp[tid - 128]);
+    decay = expf(A.g[bh]);
+    beta = A.beta[bh];
+  }
+  __syncthreads();
+
+  float kr[ROWS], qr[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) { kr[r] = kn[kg * ROWS + r]; qr[r] = qn[kg * ROWS + r]; }
+
+  // decay, then the thread's share of kS
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    S[r].x *= decay; S[r].y *= decay; S[r].z *= decay; S[r].w *= decay;
+    acc.x = fmaf(kr[r], S[r].x, acc.x); acc.y = fmaf(kr[r], S[r].y, acc.y);
+    acc.z = fmaf(kr[r], S[r].z, acc.z); acc.w = fmaf(kr[r], S[r].w, acc.w);
+  }
+  *(float4*)&part[kg][vq * 4] = acc;
+  __syncthreads();
+  float4 kS = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int j = 0; j < KG; j++) {
+    const float4 p = *(const float4*)&part[j][vq * 4];
+    kS.x += p.x; kS.y += p.y; kS.z += p.z; kS.w += p.w;
+  }
+  __syncthreads();   // part is reused for o below
+  const uint2 vv = *(const uint2*)(vp + col0);
+  float4 d;
+  d.x = (__uint_as_float(vv.x << 16) - kS.x) * beta;
+  d.y = (__uint_as_float(vv.x & 0xffff0000u) - kS.y) * beta;
+  d.z = (__uint_as_float(vv.y << 16) - kS.z) * beta;
+  d.w = (__uint_as_float(vv.y & 0xffff0000u) - kS.w) * beta;
+
+  float* So = A.S_out + bh * GDN_D * GDN_D;
+  acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    S[r].x = fmaf(kr[r], d.x, S[r].x); S[r].y = fmaf(kr[r], d.y, S[r].y);
+    S[r].z = fmaf(kr[r], d.z, S[r].z); S[r].w = fmaf(kr[r], d.w, S[r].w);
+    *(float4*)(So + (int64_t)(kg * ROWS + r) * GDN_D + col0) = S[r];
+    acc.x = fmaf(qr[r], S[r].x, acc.x); acc.y = fmaf(qr[r], S[r].y, acc.y);
+    acc.z = fmaf(qr[r], S[r].z, acc.z); acc.w = fmaf(qr[r], S[r].w, acc.w);
+  }
+  *(float4*)&part[kg][vq * 4] = acc;
+  __syncthreads();
+
+  // o[v] for the slab: thread t < COLS sums column t over the row groups
+  float o = 0.0f;
+  if (tid < COLS) {
+#pragma unroll
+    for (int j = 0; j < KG; j++) o += part[j][tid];
+  }
+  uint16_t* outp = A.out + bh * GDN_D + slab * COLS;
+  if (!FUSED) {
+    if (tid < COLS) outp[tid] = f32_to_bf16(o);
+    return;
+  }
+  // gated RMSNorm over the 128 outputs of the head (threads 0..127 = waves 0, 1)
+  float ss = wave_sum(o * o);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  if (tid < GDN_D) {
+    const float orstd = 1.0f / sqrtf((red[0] + red[1]) / (float)GDN_D + 1e-6f);
+    const float zv = bf16_to_f32(A.z[bh * GDN_D + tid]);
+    const float zs = zv * (1.0f / (1.0f + expf(zv * -1.0f)));
+    outp[tid] = f32_to_bf16(((o * orstd) * A.norm_w[tid]) * zs);
+  }
+}
+
+static int check_common(const GdnArgs& A, int batch) {
+  BK_REQUIRE(A.q && A.k && A.v && A.S_in && A.S_out && A.out, "gdn_step: null pointer");
+  BK_REQUIRE(A.Hg > 0 && A.Hg <= 65535 && batch > 0 && batch <= 65535, "gdn_step: bad Hg=%d batch=%d", A.Hg, batch);
+  BK_REQUIRE(((uintptr_t)A.S_in & 15) == 0 && ((uintptr_t)A.S_out & 15) == 0, "gdn_step: S must be 16-byte aligned");
+  BK_REQUIRE(((uintptr_t)A.v & 7) == 0 && (A.qkv_bstride % 4) == 0, "gdn_step: v must be 8-byte aligned");
+  return BK_OK;
+}
+
+int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
+                     const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch) {
+  GdnArgs A{};
+  const int KEYDIM = Hg * GDN_D;
+  A.q = (const uint16_t*)conv_out; A.k = A.q + KEYDIM; A.v = A.q + 2 * KEYDIM;
+  A.qkv_bstride = 3 * (int64_t)KEYDIM;
+  A.z = (const uint16_t*)z; A.A_log = A_log; A.dt_bias = (const uint16_t*)dt_bias; A.a_p = a_p; A.b_p = b_p; A.norm_w = norm_w;
+  A.S_in = S_in; A.S_out = S_out; A.out = (uint16_t*)out; A.Hg = Hg;
+  BK_REQUIRE(conv_out && z && A_log && dt_bias && a_p && b_p && norm_w, "gdn_delta_rule: null pointer");
+  int rc = check_common(A, batch);
+  if (rc) return rc;
+  hipLaunchKernelGGL((gdn_step_kernel<1, true>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+int launch_gdn_core(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* S_in,
+                    void* out, float* S_out, int Hg, int batch) {
+  GdnArgs A{};
+  A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v;
+  A.qkv_bstride = (int64_t)Hg * GDN_D;
+  A.g = g; A.beta = beta; A.S_in = S_in; A.S_out = S_out; A.out = (uint16_t*)out; A.Hg = Hg;
+  BK_REQUIRE(g && beta, "gdn_core: null pointer");
+  int rc = check_common(A, batch);
+  if (rc) return rc;
+  // few (batch, head) pairs: cut every head into 4 column slabs so that more CUs stream S
+  if ((int64_t)Hg * batch < 2 * num_cus())
+    hipLaunchKernelGGL((gdn_step_kernel<4, false>), dim3(Hg, 4, batch), dim3(GDN_THREADS), 0, stream(), A);
+  else
+    hipLaunchKernelGGL((gdn_step_kernel<1, false>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

@@ -1,0 +1,365 @@
+// Small bf16/f32 ops around the matmuls of one decode step: embed, RMSNorm, cast,
+// add, SwiGLU, conv1d, per-head q/k norm, RoPE, argmax.  Every activation carries a
+// leading batch dimension; all math is f32 with bf16 (round-to-nearest-even) I/O,
+// as in src/fusion.ts:295-330 and src/emitters.ts:31-255.
+#include "ops.h"
+
+namespace bk {
+
+// Block-wide sum for blockDim.x = 64 * NW; every thread gets the total.  Fixed order.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+  v = wave_sum(v);
+  if (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) lds[w] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NW; i++) t += lds[i];
+  __syncthreads();
+  return t;
+}
+
+// ---------------------------------------------------------------- embed
+// src/emitters.ts:31-45: X[b, 0:H] = E[id[b], :] (bf16 row copy).  The id is a scalar
+// argument (batch 1, as the reference passes it) or comes from an int32 device array.
+__global__ __launch_bounds__(256) void embed_kernel(const uint16_t* __restrict__ E, const int32_t* __restrict__ ids,
+                                                    int32_t id_scalar, uint16_t* __restrict__ out, int H, int vocab) {
+  const int b = blockIdx.y;
+  int id = ids ? ids[b] : id_scalar;
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);     // out-of-range ids are clamped, never read out of bounds
+  const int i = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i < H) *(uint4*)(out + (int64_t)b * H + i) = *(const uint4*)(E + (int64_t)id * H + i);
+}
+
+int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void* out, int H, int vocab, int batch) {
+  BK_REQUIRE(E && out, "embed: null pointer");
+  BK_REQUIRE(H > 0 && H % 8 == 0 && vocab > 0 && batch > 0 && batch <= 65535, "embed: bad H=%d vocab=%d batch=%d", H, vocab, batch);
+  BK_REQUIRE(ids_dev || batch == 1, "embed: a scalar token id serves batch 1 only");
+  hipLaunchKernelGGL(embed_kernel, dim3((H / 8 + 255) / 256, batch), dim3(256), 0, stream(), (const uint16_t*)E, ids_dev,
+                     id_scalar, (uint16_t*)out, H, vocab);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// src/fusion.ts:310-322: y = bf16((x * rsqrt(mean(x^2) + 1e-6)) * (1 + w)).  One
+// workgroup per row, 8 elements per thread per pass.  With `xq` set the bf16 result
+// is also quantized to Q8_1 in the same pass (four lanes share one 32-element block),
+// which is what the following matmuls consume.
+template <bool QUANT>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                      uint16_t* __restrict__ out, uint8_t* __restrict__ xq, int N) {
+  __shared__ float lds[4];
+  const int row = blockIdx.x;
+  const uint16_t* xr = x + (int64_t)row * N;
+  float ss = 0.0f;
+  for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
+    const uint4 v = *(const uint4*)(xr + i);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
+      ss += a * a + b * b;
+    }
+  }
+  ss = block_sum<4>(ss, lds);
+  const float rstd = 1.0f / sqrtf(ss / (float)N + 1e-6f);
+  for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
+    const uint4 v = *(const uint4*)(xr + i);
+    const uint4 wv = *(const uint4*)(w + i);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, uw[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t o[4];
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
+      const float wa = __uint_as_float(uw[j] << 16), wb = __uint_as_float(uw[j] & 0xffff0000u);
+      const uint16_t ha = f32_to_bf16((a * rstd) * (1.0f + wa)), hb = f32_to_bf16((b * rstd) * (1.0f + wb));
+      o[j] = (uint32_t)ha | ((uint32_t)hb << 16);
+      f[2 * j] = bf16_to_f32(ha); f[2 * j + 1] = bf16_to_f32(hb);
+    }
+    if (out) *(uint4*)(out + (int64_t)row * N + i) = make_uint4(o[0], o[1], o[2], o[3]);
+    if (QUANT) {
+      // Q8_1 of the bf16-rounded values: block = 4 consecutive lanes x 8 elements
+      float amax = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(f[j]));
+      amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
+      amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
+      const double d = (double)amax / 127.0, div = d != 0.0 ? d : 1.0;
+      int sum = 0;
+      uint32_t pk[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const double qd = (double)f[j] / div;
+        double r = floor(qd);
+        if (qd - r >= 0.5) r += 1.0;
+        int q = (int)r;
+        sum += q;
+        q = q < -128 ? -128 : (q > 127 ? 127 : q);
+        pk[j >> 2] |= (uint32_t)(q & 0xff) << (8 * (j & 3));
+      }
+      sum += dpp_i32<DPP_QUAD_XOR1>(sum);
+      sum += dpp_i32<DPP_QUAD_XOR2>(sum);
+      uint8_t* ob = xq + ((int64_t)row * (N / 32) + i / 32) * 36;
+      uint32_t* oq = (uint32_t*)(ob + (i & 31));
+      oq[0] = pk[0]; oq[1] = pk[1];
+      if ((i & 31) == 0)
+        *(uint32_t*)(ob + 32) = (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);
+    }
+  }
+}
+
+int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows) {
+  BK_REQUIRE(x && w && (out || xq), "rmsnorm: null pointer");
+  BK_REQUIRE(N > 0 && N % 32 == 0 && rows > 0, "rmsnorm: N=%d must be a positive multiple of 32 (rows=%d)", N, rows);
+  if (xq)
+    hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
+                       (uint16_t*)out, (uint8_t*)xq, N);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
+                       (uint16_t*)out, (uint8_t*)nullptr, N);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- elementwise
+constexpr int EW_CAST = EW_CAST_OP, EW_ADD = EW_ADD_OP, EW_SWIGLU = EW_SWIGLU_OP;
+
+// cast:   out = bf16(x)                      x f32            src/fusion.ts:295-299
+// add:    out = bf16(f32(a) + f32(b))        a, b bf16        src/fusion.ts:301-308
+// swiglu: out = bf16((g * sigmoid(g)) * u)   g, u f32         src/fusion.ts:324-330
+template <int OP>
+__global__ __launch_bounds__(256) void elementwise_kernel(const void* __restrict__ a, const void* __restrict__ b,
+                                                          uint16_t* __restrict__ out, int64_t n) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= n) return;
+  float r[4];
+  if (OP == EW_CAST) {
+    const float4 v = *(const float4*)((const float*)a + i);
+    r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+  } else if (OP == EW_ADD) {
+    const uint2 va = *(const uint2*)((const uint16_t*)a + i), vb = *(const uint2*)((const uint16_t*)b + i);
+    r[0] = __uint_as_float(va.x << 16) + __uint_as_float(vb.x << 16);
+    r[1] = __uint_as_float(va.x & 0xffff0000u) + __uint_as_float(vb.x & 0xffff0000u);
+    r[2] = __uint_as_float(va.y << 16) + __uint_as_float(vb.y << 16);
+    r[3] = __uint_as_float(va.y & 0xffff0000u) + __uint_as_float(vb.y & 0xffff0000u);
+  } else {
+    const float4 g = *(const float4*)((const float*)a + i), u = *(const float4*)((const float*)b + i);
+    r[0] = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
+    r[1] = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
+    r[2] = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
+    r[3] = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+  }
+  uint2 o;
+  o.x = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
+  o.y = (uint32_t)f32_to_bf16(r[2]) | ((uint32_t)f32_to_bf16(r[3]) << 16);
+  *(uint2*)(out + i) = o;
+}
+
+int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t n) {
+  BK_REQUIRE(a && out && (op == EW_CAST || b), "elementwise: null pointer");
+  BK_REQUIRE(n > 0 && n % 4 == 0, "elementwise: n=%lld must be a positive multiple of 4", (long long)n);
+  dim3 grid((unsigned)((n / 4 + 255) / 256)), block(256);
+  if (op == EW_CAST) hipLaunchKernelGGL(elementwise_kernel<EW_CAST>, grid, block, 0, stream(), a, b, (uint16_t*)out, n);
+  else if (op == EW_ADD) hipLaunchKernelGGL(elementwise_kernel<EW_ADD>, grid, block, 0, stream(), a, b, (uint16_t*)out, n);
+  else if (op == EW_SWIGLU) hipLaunchKernelGGL(elementwise_kernel<EW_SWIGLU>, grid, block, 0, stream(), a, b, (uint16_t*)out, n);
+  else return set_error(BK_ERR_ARG, "elementwise: unknown op %d", op);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- conv1d decode
+// src/emitters.ts:48-72: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); out = bf16(r * sigmoid(r));
+// new state rows = (s1, s2, x).  state [B, 3, C] bf16, weight [C, 4] bf16.
+__global__ __launch_bounds__(256) void conv1d_decode_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ st,
+                                                            const uint16_t* __restrict__ w, uint16_t* __restrict__ out,
+                                                            uint16_t* __restrict__ stn, int C) {
+  const int b = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 2;
+  if (c >= C) return;
+  const uint32_t xv = *(const uint32_t*)(x + (int64_t)b * C + c);
+  const uint16_t* sb = st + (int64_t)b * 3 * C;
+  const uint32_t s0 = *(const uint32_t*)(sb + c), s1 = *(const uint32_t*)(sb + C + c), s2 = *(const uint32_t*)(sb + 2 * C + c);
+  const uint4 wv = *(const uint4*)(w + 4 * c);          // 8 bf16: channel c taps 0..3, channel c+1 taps 0..3
+  uint32_t o = 0;
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const uint32_t wl = k ? wv.z : wv.x, wh = k ? wv.w : wv.y;
+    const float w0 = __uint_as_float(wl << 16), w1 = __uint_as_float(wl & 0xffff0000u);
+    const float w2 = __uint_as_float(wh << 16), w3 = __uint_as_float(wh & 0xffff0000u);
+    const float f0 = k ? __uint_as_float(s0 & 0xffff0000u) : __uint_as_float(s0 << 16);
+    const float f1 = k ? __uint_as_float(s1 & 0xffff0000u) : __uint_as_float(s1 << 16);
+    const float f2 = k ? __uint_as_float(s2 & 0xffff0000u) : __uint_as_float(s2 << 16);
+    const float fx = k ? __uint_as_float(xv & 0xffff0000u) : __uint_as_float(xv << 16);
+    const float r = (w0 * f0 + w1 * f1) + (w2 * f2 + w3 * fx);
+    o |= (uint32_t)f32_to_bf16(r * (1.0f / (1.0f + expf(-r)))) << (16 * k);
+  }
+  *(uint32_t*)(out + (int64_t)b * C + c) = o;
+  uint16_t* nb = stn + (int64_t)b * 3 * C;
+  *(uint32_t*)(nb + c) = s1;
+  *(uint32_t*)(nb + C + c) = s2;
+  *(uint32_t*)(nb + 2 * C + c) = xv;
+}
+
+int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch) {
+  BK_REQUIRE(x && st && w && out && st_new, "conv1d_decode: null pointer");
+  BK_REQUIRE(C > 0 && C % 2 == 0 && batch > 0 && batch <= 65535, "conv1d_decode: bad C=%d batch=%d", C, batch);
+  BK_REQUIRE(st != st_new, "conv1d_decode: state in and out must be different buffers");
+  hipLaunchKernelGGL(conv1d_decode_kernel, dim3((C / 2 + 255) / 256, batch), dim3(256), 0, stream(), (const uint16_t*)x,
+                     (const uint16_t*)st, (const uint16_t*)w, (uint16_t*)out, (uint16_t*)st_new, C);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- per-head norm (+ RoPE)
+// src/emitters.ts:123-147 emitQNorm / emitKNorm: bf16((x * rsqrt(mean(x^2) + 1e-6)) * (1 + w))
+// per head of HD values; the input rows are `in_stride` apart (2*HD for the interleaved
+// [q | gate] buffer of q_proj, HD for k).  One wavefront per (batch, head).
+// With cos/sin tables the rotation of src/emitters.ts:150-183 is applied to the
+// bf16-rounded result in the same kernel: pairs (i, i + half), i < half:
+//   x1' = bf16(x1*c - x2*s), x2' = bf16(x2*c + x1*s).
+__global__ __launch_bounds__(64) void headnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                      uint16_t* __restrict__ out, int nheads, int HD, int in_stride,
+                                                      int64_t in_bstride, const float* __restrict__ cos_t,
+                                                      const float* __restrict__ sin_t, const int32_t* __restrict__ pos_dev,
+                                                      int pos_scalar, int half) {
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const uint16_t* xh = x + (int64_t)b * in_bstride + (int64_t)h * in_stride;
+  uint16_t* oh = out + ((int64_t)b * nheads + h) * HD;
+  float ss = 0.0f;
+  for (int i = lane; i < HD; i += 64) { const float v = bf16_to_f32(xh[i]); ss += v * v; }
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)HD + 1e-6f);
+  if (!cos_t) {
+    for (int i = lane; i < HD; i += 64) oh[i] = f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i])));
+    return;
+  }
+  const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  for (int i = lane; i < HD; i += 64) {
+    if (i >= 2 * half) {
+      oh[i] = f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i])));
+    } else if (i < half) {
+      const float x1 = bf16_to_f32(f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i]))));
+      const float x2 = bf16_to_f32(f32_to_bf16((bf16_to_f32(xh[i + half]) * rstd) * (1.0f + bf16_to_f32(w[i + half]))));
+      const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
+      oh[i] = f32_to_bf16(x1 * c - x2 * s);
+      oh[i + half] = f32_to_bf16(x2 * c + x1 * s);
+    }
+  }
+}
+
+int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD, int in_stride, int64_t in_bstride,
+                    int batch, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half,
+                    int max_len) {
+  BK_REQUIRE(x && w && out, "headnorm: null pointer");
+  BK_REQUIRE(nheads > 0 && HD > 0 && in_stride >= HD && batch > 0 && batch <= 65535, "headnorm: bad shape");
+  if (cos_t) {
+    BK_REQUIRE(sin_t && half > 0 && 2 * half <= HD, "headnorm+rope: bad tables / half=%d", half);
+    BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
+  }
+  hipLaunchKernelGGL(headnorm_kernel, dim3(nheads, batch), dim3(64), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
+                     (uint16_t*)out, nheads, HD, in_stride, in_bstride, cos_t, sin_t, pos_dev, pos_scalar, half);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// src/emitters.ts:150-183 emitRoPE / emitRoPEK: in place on bf16 [B, nheads, HD].
+__global__ __launch_bounds__(256) void rope_kernel(uint16_t* __restrict__ x, const float* __restrict__ cos_t,
+                                                   const float* __restrict__ sin_t, const int32_t* __restrict__ pos_dev,
+                                                   int pos_scalar, int nheads, int HD, int half) {
+  const int b = blockIdx.y;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= nheads * half) return;
+  const int h = t / half, i = t % half;
+  const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  uint16_t* p1 = x + ((int64_t)b * nheads + h) * HD + i;
+  uint16_t* p2 = p1 + half;
+  const float x1 = bf16_to_f32(*p1), x2 = bf16_to_f32(*p2);
+  const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
+  *p1 = f32_to_bf16(x1 * c - x2 * s);
+  *p2 = f32_to_bf16(x2 * c + x1 * s);
+}
+
+int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int nheads,
+                int HD, int half, int max_len, int batch) {
+  BK_REQUIRE(x && cos_t && sin_t, "rope: null pointer");
+  BK_REQUIRE(nheads > 0 && half > 0 && 2 * half <= HD && batch > 0 && batch <= 65535, "rope: bad shape");
+  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
+  hipLaunchKernelGGL(rope_kernel, dim3((nheads * half + 255) / 256, batch), dim3(256), 0, stream(), (uint16_t*)x, cos_t, sin_t,
+                     pos_dev, pos_scalar, nheads, HD, half);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- argmax
+// prototypes/decode.ts:746-791: stage 1 takes the maximum of a tile and its index,
+// stage 2 walks the partials in index order with a strict ">", so the lowest index
+// wins ties; the running maximum starts at -FLT_MAX and NaN never wins.
+constexpr float ARGMAX_INIT = -3.40282347e38f;
+constexpr int ARGMAX_TILE = 4096;
+
+__device__ __forceinline__ void argmax_merge(float& v, int& i, float ov, int oi) {
+  // (ov, oi) beats (v, i) when larger, or equal with a lower index
+  if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+__device__ __forceinline__ void argmax_wave(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(v, off);
+    const int oi = __shfl_xor(i, off);
+    argmax_merge(v, i, ov, oi);
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_stage1_kernel(const float* __restrict__ logits, float* __restrict__ pv,
+                                                            int32_t* __restrict__ pi, int n, int ntiles) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int b = blockIdx.y, tile = blockIdx.x;
+  const float* L = logits + (int64_t)b * n;
+  float v = ARGMAX_INIT; int idx = 0x7fffffff;
+  const int base = tile * ARGMAX_TILE;
+  for (int j = threadIdx.x; j < ARGMAX_TILE; j += 256) {
+    const int e = base + j;
+    if (e < n) { const float x = L[e]; if (x > v) { v = x; idx = e; } }
+  }
+  argmax_wave(v, idx);
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = v; si[threadIdx.x >> 6] = idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; k++) argmax_merge(v, idx, sv[k], si[k]);
+    pv[(int64_t)b * ntiles + tile] = v;
+    pi[(int64_t)b * ntiles + tile] = idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_stage2_kernel(const float* __restrict__ pv, const int32_t* __restrict__ pi,
+                                                           float* __restrict__ val, int32_t* __restrict__ idx, int ntiles) {
+  const int b = blockIdx.x;
+  float v = ARGMAX_INIT; int i = 0x7fffffff;
+  for (int t = threadIdx.x; t < ntiles; t += 64) argmax_merge(v, i, pv[(int64_t)b * ntiles + t], pi[(int64_t)b * ntiles + t]);
+  argmax_wave(v, i);
+  if (threadIdx.x == 0) {
+    val[b] = v;
+    idx[b] = (i == 0x7fffffff) ? 0 : i;     // nothing above -FLT_MAX: index 0, like the sequential scan
+  }
+}
+
+size_t argmax_workspace_bytes(int n, int batch) { return (size_t)batch * ((n + ARGMAX_TILE - 1) / ARGMAX_TILE) * 8; }
+
+int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch) {
+  BK_REQUIRE(logits && val && idx && workspace, "argmax: null pointer");
+  BK_REQUIRE(n > 0 && batch > 0 && batch <= 65535, "argmax: bad n=%d batch=%d", n, batch);
+  const int ntiles = (n + ARGMAX_TILE - 1) / ARGMAX_TILE;
+  float* pv = (float*)workspace;
+  int32_t* pi = (int32_t*)(pv + (size_t)batch * ntiles);
+  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(ntiles, batch), dim3(256), 0, stream(), logits, pv, pi, n, ntiles);
+  hipLaunchKernelGGL(argmax_stage2_kernel, dim3(batch), dim3(64), 0, stream(), pv, pi, val, idx, ntiles);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

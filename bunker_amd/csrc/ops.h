@@ -26,4 +26,34 @@ int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, i
                          int out_dtype, const void* residual);
 int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, int K);
 
+// glue.hip
+enum : int { EW_CAST_OP = 0, EW_ADD_OP = 1, EW_SWIGLU_OP = 2 };
+int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void* out, int H, int vocab, int batch);
+int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows);
+int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t n);
+int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch);
+int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD, int in_stride, int64_t in_bstride,
+                    int batch, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half,
+                    int max_len);
+int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int nheads,
+                int HD, int half, int max_len, int batch);
+size_t argmax_workspace_bytes(int n, int batch);
+int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch);
+
+// gdn.hip
+int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
+                     const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch);
+int launch_gdn_core(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* S_in,
+                    void* out, float* S_out, int Hg, int batch);
+
+// attn.hip
+size_t attn_workspace_bytes(int batch, int NKV, int max_splits);
+int attn_choose_splits(int batch, int NKV, int max_ctx);
+int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
+                       const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
+                       int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
+                       int NH, int NKV, int HD, int page_size, int splits);
+int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
+                     const int32_t* pos_dev, int pos_scalar, int batch, int NKV, int HD, int page_size);
+
 }  // namespace bk

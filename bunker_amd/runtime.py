@@ -51,6 +51,10 @@ _SIGS = {
     "bk_q4k_q8_1_subdots": [u64, u64, u64, i32, i32],
     "bk_dequant_legacy_i8": [u64, u64, i64], "bk_q4k_nibbles": [u64, u64, i64],
     "bk_q4k_dequant_f32": [u64, u64, i64],
+    "bk_gdn_core": [u64, u64, u64, u64, u64, u64, u64, u64, i32, i32],
+    "bk_attn_plan": [i32, i32, i32, C.POINTER(i32), C.POINTER(u64)],
+    "bk_attn_decode": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, u64, u64, i32, i32, i32, i32, i32, i32],
+    "bk_kv_append": [u64, u64, u64, u64, u64, i32, u64, i32, i32, i32, i32],
 }
 
 
@@ -302,3 +306,33 @@ def q4k_nibbles(blocks: int, out: int, nblocks: int) -> None:
 
 def q4k_dequant_f32(blocks: int, out: int, nblocks: int) -> None:
     _check(cu().bk_q4k_dequant_f32(blocks, out, nblocks), "bk_q4k_dequant_f32")
+
+
+def gdn_core(q: int, k: int, v: int, g: int, beta: int, S_in: int, out: int, S_out: int, Hg: int, batch: int = 1) -> None:
+    _check(cu().bk_gdn_core(q, k, v, g, beta, S_in, out, S_out, Hg, batch), "bk_gdn_core")
+
+
+def attn_plan(batch: int, NKV: int, max_ctx: int, splits: int = 0) -> tuple[int, int]:
+    """Returns (splits, workspace_bytes) the attention kernel will use for this shape."""
+    s = i32(splits); nbytes = u64(0)
+    _check(cu().bk_attn_plan(batch, NKV, max_ctx, C.byref(s), C.byref(nbytes)), "bk_attn_plan")
+    return int(s.value), int(nbytes.value)
+
+
+def attn_decode(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_len: int, max_ctx: int, out: int,
+                lse: int, batch: int, NH: int = 16, NKV: int = 2, HD: int = 256, page_size: int = 16, splits: int = 0,
+                workspace: int = 0, workspace_bytes: int = 0, gate: int = 0, gate_bstride: int = 0,
+                gate_hstride: int = 0) -> None:
+    _check(cu().bk_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, max_ctx, gate, gate_bstride, gate_hstride,
+                               out, lse, workspace, workspace_bytes, batch, NH, NKV, HD, page_size, splits),
+           "bk_attn_decode")
+
+
+def kv_append(k: int, v: int, kc: int, vc: int, block_table: int, bt_stride: int, pos: int, batch: int, NKV: int = 2,
+              HD: int = 256, page_size: int = 16) -> None:
+    _check(cu().bk_kv_append(k, v, kc, vc, block_table, bt_stride, pos, batch, NKV, HD, page_size), "bk_kv_append")
+
+
+def v_pages_to_device_layout(vc) -> "np.ndarray":
+    """[pages, NKV, 16 tok, 256 dim] -> the library's dim-major V pages [pages, NKV, 256 dim, 16 tok]."""
+    return np.ascontiguousarray(np.asarray(vc).transpose(0, 1, 3, 2))

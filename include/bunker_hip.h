@@ -105,6 +105,38 @@ BK_API int bk_dequant_legacy_i8(uint64_t blocks, uint64_t out, int64_t nblocks);
 BK_API int bk_q4k_nibbles(uint64_t blocks, uint64_t out, int64_t nblocks);
 BK_API int bk_q4k_dequant_f32(uint64_t blocks, uint64_t out, int64_t nblocks);
 
+/* Gated DeltaNet single-token update, core recurrence (prototypes/gdn_gated.ts:67-88
+ * refGDN at T=1 with the delta-rule beta of src/emitters.ts:105):
+ *   S' = exp(g)*S + k (x) ((v - (exp(g)*S)^T k) * beta),  o = S'^T q  -> bf16.
+ * q, k, v bf16 [batch, Hg, 128] (q, k already normalised); g, beta f32 [batch, Hg];
+ * S f32 [batch, Hg, 128, 128]; S_out may alias S_in.  The fused form of the decode
+ * step (norms, gates, gated RMSNorm; src/emitters.ts:75-120) is the "gdn_delta_rule"
+ * op of bk_kernel_create. */
+BK_API int bk_gdn_core(uint64_t q, uint64_t k, uint64_t v, uint64_t g, uint64_t beta, uint64_t S_in,
+                       uint64_t out, uint64_t S_out, int Hg, int batch);
+
+/* Split-K decode attention over a paged bf16 GQA cache: the math of emitFA2Attn
+ * (src/emitters.ts:188-226) and refAttn (prototypes/fa2_vllm.ts:114-139) for one
+ * query token per sequence, plus lse = max + ln(sum exp).
+ * q bf16 [batch, NH, 256]; out bf16 [batch, NH, 256]; lse f32 [batch, NH] or 0.
+ * Cache: 16-token pages; K page (p, kv head h) is bf16 [16][256] and V page is
+ * bf16 [256][16] (dim-major), both at element offset (p*NKV + h)*4096.
+ * block_table int32 [batch, bt_stride] (0 = sequence b owns pages b*bt_stride..),
+ * ctx_len int32 [batch].  gate: 0, or bf16 with the gate of (b, head, i) at
+ * gate[b*gate_bstride + head*gate_hstride + i] (output *= sigmoid(gate)).
+ * splits: 0 = let the library choose; with more than one split the caller passes
+ * a workspace of bk_attn_workspace_bytes(). */
+BK_API int bk_attn_plan(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes);
+BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride,
+                          uint64_t ctx_len, int max_ctx, uint64_t gate, int64_t gate_bstride,
+                          int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
+                          uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size,
+                          int splits);
+/* The cache write of emitFA2Attn (src/emitters.ts:202-205): k, v bf16 [batch, NKV, 256]
+ * of this step go to token pos[b] of every sequence (pos int32 [batch] on the device). */
+BK_API int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table,
+                        int bt_stride, uint64_t pos, int batch, int NKV, int HD, int page_size);
+
 #ifdef __cplusplus
 }
 #endif
