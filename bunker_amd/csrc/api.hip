@@ -153,6 +153,12 @@ static int run_argmax(Kernel& k, const uint64_t* s) {
   return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
 }
 
+// ---- op: advance   slots: argmax idx, argmax val, token ids, positions, history, counter    params: batch, max_steps
+static int run_advance(Kernel& k, const uint64_t* s) {
+  return launch_advance(P<int32_t>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), P<int32_t>(s[3]), P<int32_t>(s[4]), P<int32_t>(s[5]),
+                        (int)k.get("batch", 1), (int)k.get("max_steps", 0));
+}
+
 static int build_kernel(Kernel& k) {
   int rc;
   struct Simple { const char* op; RunFn run; int nslots; const char* need1; const char* need2; };
@@ -163,6 +169,7 @@ static int build_kernel(Kernel& k) {
       {"conv1d_decode", run_conv1d, 5, "QKVD", nullptr}, {"gdn_delta_rule", run_gdn, 10, "LVH", nullptr},
       {"qnorm", run_qnorm, 3, "HD", "NH"},          {"knorm", run_knorm, 3, "HD", "NKV"},
       {"rope", run_rope, 4, "HD", "NH"},            {"ropek", run_rope, 4, "HD", "NKV"},
+      {"advance", run_advance, 6, "batch", "max_steps"},
   };
   for (const Simple& sp : simple) {
     if (k.op != sp.op) continue;

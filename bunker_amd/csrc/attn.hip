@@ -12,7 +12,8 @@
 //   S^T[tok, head] = sum_d K[tok, d] * Q[head, d]        v_mfma_f32_16x16x32_bf16, A = K page
 //   O^T[d, head]   = sum_tok V^T[d, tok] * P^T[tok, head] v_mfma_f32_16x16x16_bf16, A = V page,
 // and P^T comes out of the first product in exactly the register layout the second
-// wants as its B operand.  The query heads of a KV group (<= 16) are the N dimension.
+// wants as its B operand (fed as two bf16 terms, hi + lo, so that P carries 16 bits).
+// The query heads of a KV group (<= 16) are the N dimension.
 //
 // grid = (splits, NKV, B), 4 waves per workgroup.  Each wave walks pages of its
 // split with its own running (max, sum, O^T); the four are merged through LDS in a
@@ -118,11 +119,21 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
 #pragma unroll
       for (int t = 0; t < 16; t++) { oacc[t][0] *= alpha; oacc[t][1] *= alpha; oacc[t][2] *= alpha; oacc[t][3] *= alpha; }
     }
-    const uint2 pb = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
+    // P goes in as hi + lo (two bf16 values, 16 significand bits together): the matrix pipe has
+    // time to spare, and a single bf16 rounding of P would show up as a one-ulp change in a large
+    // share of the bf16 outputs at short contexts
+    float plo[4];
 #pragma unroll
-    for (int t = 0; t < 16; t++)
+    for (int r = 0; r < 4; r++) plo[r] = p[r] - bf16_to_f32(f32_to_bf16(p[r]));
+    const uint2 pb = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
+    const uint2 pl = make_uint2(pack_bf16x2(plo[0], plo[1]), pack_bf16x2(plo[2], plo[3]));
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
       oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pb),
                                                           oacc[t], 0, 0, 0);
+      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pl),
+                                                          oacc[t], 0, 0, 0);
+    }
   }
 
   // ---- merge the four waves (fixed order 0,1,2,3)
@@ -170,7 +181,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
       float o = lds_o[d][h] / Lh;
       if (A.gate) {
         const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
-        o = o * (1.0f / (1.0f + expf(gv * -1.0f)));
+        o = __fmul_rn(o, sigmoid_f64(gv));
       }
       A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
       if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = Mh + logf(Lh);
@@ -204,7 +215,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   o = o / L;
   if (A.gate) {
     const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
-    o = o * (1.0f / (1.0f + expf(gv * -1.0f)));
+    o = __fmul_rn(o, sigmoid_f64(gv));
   }
   A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
   if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = M + logf(L);

@@ -124,7 +124,33 @@ __device__ __forceinline__ int row16_sum_i32(int v) {
   return v;
 }
 
-__device__ __forceinline__ float sigmoidf_dev(float v) { return 1.0f / (1.0f + __expf(-v)); }
+// Transcendentals are evaluated in double and rounded once to f32, and written f32
+// arithmetic uses one IEEE operation per written operation (__fmul_rn & co. keep the
+// compiler from fusing), so that these values equal a plain host computation to the bit.
+__device__ __forceinline__ float sigmoid_f64(float v) { return (float)(1.0 / (1.0 + exp(-(double)v))); }
+__device__ __forceinline__ float rsqrt_f64(double v) { return (float)(1.0 / sqrt(v)); }
+
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+  const long long b = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_readlane((int)(b & 0xffffffffll), lane);
+  const int hi = __builtin_amdgcn_readlane((int)(b >> 32), lane);
+  return __builtin_bit_cast(double, ((long long)hi << 32) | (unsigned int)lo);
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+  const long long b = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xF, 0xF, true);
+  return __builtin_bit_cast(double, ((long long)hi << 32) | (unsigned int)lo);
+}
+// Wave-wide sum in double, wave-uniform result.
+__device__ __forceinline__ double wave_sum_f64(double v) {
+  v += dpp_f64<DPP_QUAD_XOR1>(v);
+  v += dpp_f64<DPP_QUAD_XOR2>(v);
+  v += dpp_f64<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_f64<DPP_ROW_MIRROR>(v);
+  return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
+}
 
 #endif  // __HIPCC__
 }  // namespace bk

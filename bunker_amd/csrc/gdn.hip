@@ -8,8 +8,10 @@
 // head is cut into CS column slabs, one 256-thread workgroup each.  A thread owns
 // ROWS k-rows x 4 v-columns of the slab in registers for the whole step: S is read
 // from HBM once (float4, rows of the slab contiguous) and S' written once; the two
-// k-reductions are in-thread sums over the owned rows plus one LDS exchange across
-// the row groups, in a fixed order.
+// k-reductions are in-thread fmaf chains over the owned rows plus one LDS exchange
+// across the row groups, summed in group order.  With the whole head in one workgroup
+// (CS = 1) that is "chains of 16 consecutive rows, then the 8 chain results in order",
+// the order the CPU checker follows; norms and gates are evaluated in double.
 #include "ops.h"
 
 namespace bk {
@@ -46,7 +48,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   static_assert(!FUSED || CS == 1, "the gated norm needs the whole head in one workgroup");
   __shared__ float kn[GDN_D], qn[GDN_D];
   __shared__ float part[KG][COLS];
-  __shared__ float red[4];
+  __shared__ double red[4];
 
   const int h = blockIdx.x, slab = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x;
@@ -65,25 +67,25 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   const uint16_t* vp = A.v + (int64_t)b * A.qkv_bstride + h * GDN_D;
   float decay, beta;
   if (FUSED) {
-    // waves 0,1 hold q (2 values per lane... 128 values over 128 threads), waves 2,3 hold k
+    // threads 0..127 hold q, 128..255 hold k
     const bool isk = tid >= 128;
     const int i = tid & 127;
     const float x = bf16_to_f32((isk ? kp : qp)[i]);
-    float ss = wave_sum(x * x);
+    const double ss = wave_sum_f64((double)(x * x));       // square of a bf16 value: exact in f32
     if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
-    const float tot = isk ? (red[2] + red[3]) : (red[0] + red[1]);
-    const float rs = 1.0f / sqrtf(tot + 1e-6f);
+    const double tot = isk ? (red[2] + red[3]) : (red[0] + red[1]);
+    const float rs = rsqrt_f64(tot + 1e-6);
     if (isk) kn[i] = x * rs;
     else qn[i] = x * (rs * 0.08838834764831845f);     // 1/sqrt(128)
     const float sp_in = A.a_p[bh] + bf16_to_f32(A.dt_bias[h]);
-    const float softplus = log2f(1.0f + expf(sp_in)) * 0.6931471805599453f;
-    decay = expf(-1.0f * (expf(A.A_log[h]) * softplus));
-    beta = 1.0f / (1.0f + expf(A.b_p[bh] * -1.0f));
+    const float softplus = (float)log1p(exp((double)sp_in));
+    decay = (float)exp(-(double)((float)exp((double)A.A_log[h]) * softplus));
+    beta = sigmoid_f64(A.b_p[bh]);
   } else {
     if (tid < 128) qn[tid] = bf16_to_f32(qp[tid]);
     else kn[tid - 128] = bf16_to_f32(kp[tid - 128]);
-    decay = expf(A.g[bh]);
+    decay = (float)exp((double)A.g[bh]);
     beta = A.beta[bh];
   }
   __syncthreads();
@@ -141,13 +143,13 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     return;
   }
   // gated RMSNorm over the 128 outputs of the head (threads 0..127 = waves 0, 1)
-  float ss = wave_sum(o * o);
-  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  const double oss = wave_sum_f64((double)o * (double)o);
+  if ((tid & 63) == 0) red[tid >> 6] = oss;
   __syncthreads();
   if (tid < GDN_D) {
-    const float orstd = 1.0f / sqrtf((red[0] + red[1]) / (float)GDN_D + 1e-6f);
+    const float orstd = rsqrt_f64((red[0] + red[1]) / (double)GDN_D + 1e-6);
     const float zv = bf16_to_f32(A.z[bh * GDN_D + tid]);
-    const float zs = zv * (1.0f / (1.0f + expf(zv * -1.0f)));
+    const float zs = zv * sigmoid_f64(zv);
     outp[tid] = f32_to_bf16(((o * orstd) * A.norm_w[tid]) * zs);
   }
 }

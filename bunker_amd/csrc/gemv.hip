@@ -10,6 +10,13 @@
 // sub-block 2*(c>>1) and the high nibbles of sub-block 2*(c>>1)+1.  The slice
 // of the activation a lane needs therefore depends on the lane only, not on
 // the row: it is loaded once into registers and reused for every row.
+//
+// Arithmetic.  The sub-block dots are exact int32.  Everything after them is carried
+// in double: d*d8 (two fp16 values) is exact in f32, times the 6-bit scale and the
+// integer dot it is exact in double, so a row's value is a sum of exactly known terms
+// with ~1e-16 relative accumulation error, rounded once to f32.  The result therefore
+// does not depend on the lane mapping, the launch shape or the batch size, and equals
+// a plain host loop in double to the bit (up to ~1e-8 probability per output).
 #include "ops.h"
 
 namespace bk {
@@ -78,16 +85,16 @@ __device__ __forceinline__ void load_xq(XQ& x, const uint8_t* __restrict__ xq, i
   x.s8c = half_to_f32((uint16_t)(ds >> 16));
 }
 
-// One slot's contribution to a row: returns the f32 partial; I0/I1 are the
-// exact int32 half-sub-block dots (low / high nibbles).
-__device__ __forceinline__ float slot_dot(const uint4& hdr, const uint4& q, const XQ& x, const ScaleSel& sel,
+// One slot's contribution to a row (double); I0/I1 are the exact int32
+// half-sub-block dots (low / high nibbles).
+__device__ __forceinline__ double slot_dot(const uint4& hdr, const uint4& q, const XQ& x, const ScaleSel& sel,
                                           int& I0, int& I1) {
   const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu));
   const float dmin = half_to_f32((uint16_t)(hdr.x >> 16));
   uint32_t sc, m;
   lane_scale_min(sel, hdr.y, hdr.z, hdr.w, sc, m);
-  const float fsc = (d * x.d8c) * (float)sc;
-  const float fm = (dmin * x.s8c) * (float)m;
+  const double fsc = (double)(d * x.d8c) * (double)sc;      // d*d8c: 11 x 11 significand bits, exact in f32
+  const double fm = (double)(dmin * x.s8c) * (double)m;
   int a = 0, b = 0;
   a = sdot4(q.x & 0x0f0f0f0fu, x.lo[0], a);
   b = sdot4((q.x >> 4) & 0x0f0f0f0fu, x.hi[0], b);
@@ -98,9 +105,9 @@ __device__ __forceinline__ float slot_dot(const uint4& hdr, const uint4& q, cons
   a = sdot4(q.w & 0x0f0f0f0fu, x.lo[3], a);
   b = sdot4((q.w >> 4) & 0x0f0f0f0fu, x.hi[3], b);
   I0 = a; I1 = b;
-  const float f0 = dpp_f32<DPP_PAIR_EVEN>(fsc);   // combined scale of sub-block 2g
-  const float f1 = dpp_f32<DPP_PAIR_ODD>(fsc);    // combined scale of sub-block 2g+1
-  return (f0 * (float)a + f1 * (float)b) - fm;
+  const double f0 = dpp_f64<DPP_PAIR_EVEN>(fsc);   // combined scale of sub-block 2g
+  const double f1 = dpp_f64<DPP_PAIR_ODD>(fsc);    // combined scale of sub-block 2g+1
+  return fma(f0, (double)a, fma(f1, (double)b, -fm));
 }
 
 enum : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_BF16_ADD = 2 };
@@ -156,13 +163,13 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
     }
 #pragma unroll
     for (int i = 0; i < GEMV_RPI; i++) {
-      float acc = 0.0f;
+      double acc = 0.0;
 #pragma unroll
       for (int r = 0; r < NR; r++) {
         int I0, I1;
         acc += slot_dot(hdr[i][r], q[i][r], x[r], sel, I0, I1);
       }
-      const float tot = wave_sum(acc);
+      const float tot = (float)wave_sum_f64(acc);
       if (lane == 0 && row0 + i < N) store_out<EPI>(y, res, (int64_t)bidx * N + row0 + i, tot);
     }
   }
@@ -185,7 +192,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_generic_kernel(
   const int rounds = (nb + 7) / 8;
   for (int row = wave; row < N; row += nwaves) {
     const uint8_t* rp = W + (int64_t)row * row_bytes;
-    float acc = 0.0f;
+    double acc = 0.0;
     for (int r = 0; r < rounds; r++) {
       const int blk = r * 8 + (lane >> 3);
       const bool active = blk < nb;
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_generic_kernel(
       int I0, I1;
       acc += slot_dot(hdr, q, x, sel, I0, I1);
     }
-    const float tot = wave_sum(acc);
+    const float tot = (float)wave_sum_f64(acc);
     if (lane == 0) store_out<EPI>(y, res, (int64_t)bidx * N + row, tot);
   }
 }

@@ -6,15 +6,15 @@
 
 namespace bk {
 
-// Block-wide sum for blockDim.x = 64 * NW; every thread gets the total.  Fixed order.
+// Block-wide sum in double for blockDim.x = 64 * NW; every thread gets the total.
 template <int NW>
-__device__ __forceinline__ float block_sum(float v, float* lds) {
-  v = wave_sum(v);
+__device__ __forceinline__ double block_sum_f64(double v, double* lds) {
+  v = wave_sum_f64(v);
   if (NW == 1) return v;
   const int w = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) lds[w] = v;
   __syncthreads();
-  float t = 0.0f;
+  double t = 0.0;
 #pragma unroll
   for (int i = 0; i < NW; i++) t += lds[i];
   __syncthreads();
@@ -51,21 +51,21 @@ int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void*
 template <bool QUANT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                       uint16_t* __restrict__ out, uint8_t* __restrict__ xq, int N) {
-  __shared__ float lds[4];
+  __shared__ double lds[4];
   const int row = blockIdx.x;
   const uint16_t* xr = x + (int64_t)row * N;
-  float ss = 0.0f;
+  double ss = 0.0;     // squares of bf16 values are exact in f32; their sum is carried in double
   for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
     const uint4 v = *(const uint4*)(xr + i);
     const uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
-      ss += a * a + b * b;
+      ss += (double)(a * a) + (double)(b * b);
     }
   }
-  ss = block_sum<4>(ss, lds);
-  const float rstd = 1.0f / sqrtf(ss / (float)N + 1e-6f);
+  ss = block_sum_f64<4>(ss, lds);
+  const float rstd = rsqrt_f64(ss / (double)N + 1e-6);
   for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
     const uint4 v = *(const uint4*)(xr + i);
     const uint4 wv = *(const uint4*)(w + i);
@@ -76,7 +76,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     for (int j = 0; j < 4; j++) {
       const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
       const float wa = __uint_as_float(uw[j] << 16), wb = __uint_as_float(uw[j] & 0xffff0000u);
-      const uint16_t ha = f32_to_bf16((a * rstd) * (1.0f + wa)), hb = f32_to_bf16((b * rstd) * (1.0f + wb));
+      const uint16_t ha = f32_to_bf16(__fmul_rn(__fmul_rn(a, rstd), __fadd_rn(1.0f, wa)));
+      const uint16_t hb = f32_to_bf16(__fmul_rn(__fmul_rn(b, rstd), __fadd_rn(1.0f, wb)));
       o[j] = (uint32_t)ha | ((uint32_t)hb << 16);
       f[2 * j] = bf16_to_f32(ha); f[2 * j + 1] = bf16_to_f32(hb);
     }
@@ -148,10 +149,10 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const void* __restrict
     r[3] = __uint_as_float(va.y & 0xffff0000u) + __uint_as_float(vb.y & 0xffff0000u);
   } else {
     const float4 g = *(const float4*)((const float*)a + i), u = *(const float4*)((const float*)b + i);
-    r[0] = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
-    r[1] = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
-    r[2] = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
-    r[3] = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+    r[0] = __fmul_rn(__fmul_rn(g.x, sigmoid_f64(g.x)), u.x);
+    r[1] = __fmul_rn(__fmul_rn(g.y, sigmoid_f64(g.y)), u.y);
+    r[2] = __fmul_rn(__fmul_rn(g.z, sigmoid_f64(g.z)), u.z);
+    r[3] = __fmul_rn(__fmul_rn(g.w, sigmoid_f64(g.w)), u.w);
   }
   uint2 o;
   o.x = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
@@ -173,7 +174,8 @@ int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t 
 
 // ---------------------------------------------------------------- conv1d decode
 // src/emitters.ts:48-72: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); out = bf16(r * sigmoid(r));
-// new state rows = (s1, s2, x).  state [B, 3, C] bf16, weight [C, 4] bf16.
+// new state rows = (s1, s2, x).  state [B, 3, C] bf16, weight [C, 4] bf16.  The new state may be
+// written over the old one: a thread reads its two channels' rows before it writes them.
 __global__ __launch_bounds__(256) void conv1d_decode_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ st,
                                                             const uint16_t* __restrict__ w, uint16_t* __restrict__ out,
                                                             uint16_t* __restrict__ stn, int C) {
@@ -194,8 +196,9 @@ __global__ __launch_bounds__(256) void conv1d_decode_kernel(const uint16_t* __re
     const float f1 = k ? __uint_as_float(s1 & 0xffff0000u) : __uint_as_float(s1 << 16);
     const float f2 = k ? __uint_as_float(s2 & 0xffff0000u) : __uint_as_float(s2 << 16);
     const float fx = k ? __uint_as_float(xv & 0xffff0000u) : __uint_as_float(xv << 16);
-    const float r = (w0 * f0 + w1 * f1) + (w2 * f2 + w3 * fx);
-    o |= (uint32_t)f32_to_bf16(r * (1.0f / (1.0f + expf(-r)))) << (16 * k);
+    // products of two bf16 values are exact in f32, so fusing them into the additions changes nothing
+    const float r = __fadd_rn(__fadd_rn(w0 * f0, w1 * f1), __fadd_rn(w2 * f2, w3 * fx));
+    o |= (uint32_t)f32_to_bf16(__fmul_rn(r, sigmoid_f64(r))) << (16 * k);
   }
   *(uint32_t*)(out + (int64_t)b * C + c) = o;
   uint16_t* nb = stn + (int64_t)b * 3 * C;
@@ -207,7 +210,6 @@ __global__ __launch_bounds__(256) void conv1d_decode_kernel(const uint16_t* __re
 int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch) {
   BK_REQUIRE(x && st && w && out && st_new, "conv1d_decode: null pointer");
   BK_REQUIRE(C > 0 && C % 2 == 0 && batch > 0 && batch <= 65535, "conv1d_decode: bad C=%d batch=%d", C, batch);
-  BK_REQUIRE(st != st_new, "conv1d_decode: state in and out must be different buffers");
   hipLaunchKernelGGL(conv1d_decode_kernel, dim3((C / 2 + 255) / 256, batch), dim3(256), 0, stream(), (const uint16_t*)x,
                      (const uint16_t*)st, (const uint16_t*)w, (uint16_t*)out, (uint16_t*)st_new, C);
   BK_LAUNCH_CHECK();
@@ -229,24 +231,24 @@ __global__ __launch_bounds__(64) void headnorm_kernel(const uint16_t* __restrict
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const uint16_t* xh = x + (int64_t)b * in_bstride + (int64_t)h * in_stride;
   uint16_t* oh = out + ((int64_t)b * nheads + h) * HD;
-  float ss = 0.0f;
-  for (int i = lane; i < HD; i += 64) { const float v = bf16_to_f32(xh[i]); ss += v * v; }
-  ss = wave_sum(ss);
-  const float rstd = 1.0f / sqrtf(ss / (float)HD + 1e-6f);
+  double ss = 0.0;
+  for (int i = lane; i < HD; i += 64) { const float v = bf16_to_f32(xh[i]); ss += (double)(v * v); }
+  ss = wave_sum_f64(ss);
+  const float rstd = rsqrt_f64(ss / (double)HD + 1e-6);
+  auto normed = [&](int i) { return f32_to_bf16(__fmul_rn(__fmul_rn(bf16_to_f32(xh[i]), rstd), __fadd_rn(1.0f, bf16_to_f32(w[i])))); };
   if (!cos_t) {
-    for (int i = lane; i < HD; i += 64) oh[i] = f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i])));
+    for (int i = lane; i < HD; i += 64) oh[i] = normed(i);
     return;
   }
   const int pos = pos_dev ? pos_dev[b] : pos_scalar;
   for (int i = lane; i < HD; i += 64) {
     if (i >= 2 * half) {
-      oh[i] = f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i])));
+      oh[i] = normed(i);
     } else if (i < half) {
-      const float x1 = bf16_to_f32(f32_to_bf16((bf16_to_f32(xh[i]) * rstd) * (1.0f + bf16_to_f32(w[i]))));
-      const float x2 = bf16_to_f32(f32_to_bf16((bf16_to_f32(xh[i + half]) * rstd) * (1.0f + bf16_to_f32(w[i + half]))));
+      const float x1 = bf16_to_f32(normed(i)), x2 = bf16_to_f32(normed(i + half));
       const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
-      oh[i] = f32_to_bf16(x1 * c - x2 * s);
-      oh[i + half] = f32_to_bf16(x2 * c + x1 * s);
+      oh[i] = f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+      oh[i + half] = f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s)));
     }
   }
 }
@@ -279,8 +281,8 @@ __global__ __launch_bounds__(256) void rope_kernel(uint16_t* __restrict__ x, con
   uint16_t* p2 = p1 + half;
   const float x1 = bf16_to_f32(*p1), x2 = bf16_to_f32(*p2);
   const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
-  *p1 = f32_to_bf16(x1 * c - x2 * s);
-  *p2 = f32_to_bf16(x2 * c + x1 * s);
+  *p1 = f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+  *p2 = f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s)));
 }
 
 int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int nheads,
@@ -358,6 +360,36 @@ int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace
   int32_t* pi = (int32_t*)(pv + (size_t)batch * ntiles);
   hipLaunchKernelGGL(argmax_stage1_kernel, dim3(ntiles, batch), dim3(256), 0, stream(), logits, pv, pi, n, ntiles);
   hipLaunchKernelGGL(argmax_stage2_kernel, dim3(batch), dim3(64), 0, stream(), pv, pi, val, idx, ntiles);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+// ---------------------------------------------------------------- token feedback
+// What the host loop of src/runner.ts:150-160 does between tokens, on the device: the
+// argmax index of every sequence becomes its next token id, positions advance by one and
+// (token, logit) is appended to a history the host reads at the end.
+__global__ __launch_bounds__(256) void advance_kernel(const int32_t* __restrict__ idx, const float* __restrict__ val,
+                                                      int32_t* __restrict__ ids, int32_t* __restrict__ pos,
+                                                      int32_t* __restrict__ hist, int32_t* __restrict__ counter, int batch,
+                                                      int max_steps) {
+  const int c = counter[0];
+  __syncthreads();
+  for (int b = threadIdx.x; b < batch; b += 256) {
+    if (c < max_steps) {
+      hist[((int64_t)c * batch + b) * 2] = idx[b];
+      hist[((int64_t)c * batch + b) * 2 + 1] = __float_as_int(val[b]);
+    }
+    ids[b] = idx[b];
+    pos[b] += 1;
+  }
+  if (threadIdx.x == 0) counter[0] = c + 1;
+}
+
+int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
+                   int max_steps) {
+  BK_REQUIRE(idx && val && ids && pos && hist && counter, "advance: null pointer");
+  BK_REQUIRE(batch > 0 && max_steps > 0, "advance: bad batch=%d max_steps=%d", batch, max_steps);
+  hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(256), 0, stream(), idx, val, ids, pos, hist, counter, batch, max_steps);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

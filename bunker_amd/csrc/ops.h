@@ -40,6 +40,9 @@ int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* 
 size_t argmax_workspace_bytes(int n, int batch);
 int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch);
 
+int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
+                   int max_steps);
+
 // gdn.hip
 int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
                      const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch);

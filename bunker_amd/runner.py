@@ -1,0 +1,339 @@
+"""Graph-driven decode runtime: partition -> topological order -> kernels -> token loop.
+
+Counterpart of src/runner.ts (``choosePartition``, ``topoOrder``, ``compileStep``,
+``runGraphDecode``) and of the buffer plumbing of prototypes/decode_graph.ts:66-145
+(``DecodeEnv``: state double buffers, rope tables, scratch for intermediates).  Each
+group of the partition becomes one pre-compiled kernel handle (``compileAndLoad`` of an op
+spec instead of TTIR text) and one ``cuLaunch`` per token with the node's tensors in the
+reference's slot order: inputs in declared order, then outputs (src/fusion.ts:371-401).
+
+``runGraphDecode`` is the reference's loop: token id and position are passed as scalars and
+every kernel is launched from the host each step.  ``DeviceLoop`` is the fast path of this
+build: token ids and positions live in device memory, one step is recorded once into a HIP
+graph and replayed, and the generated tokens are read back at the end.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable
+
+import numpy as np
+
+from . import runtime as rt
+from . import synth
+from .graph import Graph, GraphNode
+from .model import Dims, SYNTH, buildModelGraph
+
+Partition = list  # list[list[GraphNode]]
+
+
+@dataclass
+class KernelPlan:
+    """What compilePartition returns per group (src/fusion.ts:110-117), with an op spec for ttir."""
+    spec: str
+    name: str
+    args: list            # external tensor names, in slot order
+    grid: list
+    group: list
+
+
+@dataclass
+class CompiledStep:
+    graph: Graph
+    schedule: list        # [(KernelPlan, LoadedKernel)]
+    batch: int = 1
+    device_scalars: bool = False
+
+
+# ---------------------------------------------------------------- partition + order
+def choosePartition(graph: Graph, env=None, opts: dict | None = None) -> Partition:
+    """Every node its own kernel (src/runner.ts:40-49)."""
+    return [[n] for n in graph.nodes]
+
+
+def topoOrder(graph: Graph, partition: Partition) -> Partition:
+    """Kahn's algorithm over groups with a FIFO queue (src/runner.ts:52-91).
+
+    One rule is added: a node without outputs that rewrites its first input in place (rope,
+    ropek) must run before the later consumers of that tensor.  The reference gets that order
+    only from queue order (src/runner.ts:69-88); here it is an edge of its own.
+    """
+    node_group = {}
+    for gi, grp in enumerate(partition):
+        for n in grp:
+            node_group[n.id] = gi
+    edges: dict[int, list] = {gi: [] for gi in range(len(partition))}
+    indeg = {gi: 0 for gi in range(len(partition))}
+
+    def add_edge(a, b):
+        if a != b:
+            edges[a].append(b)
+            indeg[b] += 1
+
+    for gi, grp in enumerate(partition):
+        for n in grp:
+            for inp in n.inputs:
+                p = graph.tensors[inp.tensorName].producer
+                if p is not None:
+                    add_edge(node_group[p.id], gi)
+    for n in graph.nodes:
+        if not n.outputs and n.inputs:
+            t = graph.tensors[n.inputs[0].tensorName]
+            for c in t.consumers:
+                if c.id > n.id:
+                    add_edge(node_group[n.id], node_group[c.id])
+    queue = [gi for gi in range(len(partition)) if indeg[gi] == 0]
+    out = []
+    while queue:
+        gi = queue.pop(0)
+        out.append(partition[gi])
+        for b in edges[gi]:
+            indeg[b] -= 1
+            if indeg[b] == 0:
+                queue.append(b)
+    if len(out) != len(partition):
+        raise RuntimeError(f"topoOrder: cycle in partition ({len(out)}/{len(partition)})")
+    return out
+
+
+_SPEC_KEYS = {
+    "embed": ["H", "VOCAB"], "rmsnorm": ["N"], "gemm": ["N", "K"], "cast": ["N"], "add": ["N"], "swiglu": ["N"],
+    "conv1d_decode": ["QKVD"], "gdn_delta_rule": ["LVH", "LKD", "LVD"], "qnorm": ["HD", "NH"], "knorm": ["HD", "NKV"],
+    "rope": ["HD", "NH", "ROT_HALF", "MAX_LEN"], "ropek": ["HD", "NKV", "ROT_HALF", "MAX_LEN"],
+    "fa2_attn": ["HD", "NH", "NKV", "MAX_LEN"], "argmax": ["VOCAB"],
+}
+
+
+def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str:
+    """Op name plus the constants the reference baked into the kernel text."""
+    parts = [n.op] + [f"{k}={int(n.params[k])}" for k in _SPEC_KEYS[n.op]]
+    if n.op == "gemm" and n.params.get("cast"):
+        parts.append("cast=1")
+    if batch != 1:
+        parts.append(f"batch={batch}")
+    if device_scalars:
+        if n.op == "embed":
+            parts.append("ids_dev=1")
+        if n.op in ("rope", "ropek", "fa2_attn"):
+            parts.append("pos_dev=1")
+    return " ".join(parts)
+
+
+def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_scalars: bool = False) -> list:
+    plans = []
+    for grp in ordered:
+        if len(grp) != 1:
+            raise NotImplementedError("multi-node groups are produced by fusedPartition only")
+        n = grp[0]
+        args = [i.tensorName for i in n.inputs] + [o.tensorName for o in n.outputs]
+        plans.append(KernelPlan(node_spec(n, batch, device_scalars), f"{n.op}_{n.id}", args, n.grid, grp))
+    return plans
+
+
+def compileStep(graph: Graph, partition: Partition, batch: int = 1, device_scalars: bool = False) -> CompiledStep:
+    ordered = topoOrder(graph, partition)
+    plans = compilePartition(graph, ordered, batch, device_scalars)
+    cache: dict[str, rt.LoadedKernel] = {}
+    schedule = []
+    for p in plans:
+        # handles own workspaces, so kernels with a workspace are not shared between nodes
+        shareable = p.group[0].op not in ("gemm", "fa2_attn", "argmax")
+        if shareable and p.spec in cache:
+            k = cache[p.spec]
+        else:
+            k = rt.compileAndLoad(p.spec, p.name, 4, p.name)
+            if shareable:
+                cache[p.spec] = k
+        schedule.append((p, k))
+    return CompiledStep(graph, schedule, batch, device_scalars)
+
+
+# ---------------------------------------------------------------- token loop (src/runner.ts:116-162)
+def runGraphDecode(compiled: CompiledStep, resolve: Callable[[str], int], initialToken: int, steps: int,
+                   onToken: Callable | None = None, startPos: int = 0):
+    """Greedy decode, one host launch per kernel per token; token id and position are scalars."""
+    graph, schedule = compiled.graph, compiled.schedule
+    argmax = next((n for n in graph.nodes if n.op == "argmax"), None)
+    if argmax is None:
+        raise RuntimeError("runGraphDecode: graph has no argmax node")
+    idx_name, val_name = argmax.outputs[1].tensorName, argmax.outputs[0].tensorName
+    tokens, logits = [], []
+    for step in range(steps):
+        token = initialToken if step == 0 else tokens[-1]
+        pos = startPos + step
+        for plan, k in schedule:
+            args = [token if a == "token_id" else pos if a == "pos" else resolve(a) for a in plan.args]
+            rc = rt.cuLaunch(k, plan.grid, [128, 1, 1], args)
+            if rc != 0:
+                raise rt.BunkerError(f"{plan.name}: {rt.last_error()} (rc={rc})")
+        rt.cuSync()
+        ibuf = np.zeros(1, np.int32); vbuf = np.zeros(1, np.float32)
+        rt.cuDtoH(ibuf, resolve(idx_name), 4)
+        rt.cuDtoH(vbuf, resolve(val_name), 4)
+        tokens.append(int(ibuf[0])); logits.append(float(vbuf[0]))
+        if onToken:
+            onToken(int(ibuf[0]), float(vbuf[0]), step)
+    return {"tokens": tokens, "logits": logits}
+
+
+# ---------------------------------------------------------------- buffers (prototypes/decode_graph.ts:66-145)
+_DT_BYTES = {"bf16": 2, "f32": 4, "i32": 4}
+
+
+def tensor_bytes(t) -> int:
+    n = 1
+    for d in t.type.shape:
+        n *= d
+    if t.type.dtype == "q4_k":
+        return n // 256 * 144
+    return n * _DT_BYTES[t.type.dtype]
+
+
+def state_key(name: str) -> str:
+    """'n12_model.layers.0.conv_state_new' / 'model.layers.0.conv_state_in' -> 'model.layers.0.conv_state'."""
+    if name.startswith("n") and "_" in name and name[1:name.index("_")].isdigit():
+        name = name[name.index("_") + 1:]
+    for suf in ("_in", "_new"):
+        if name.endswith(suf):
+            name = name[: -len(suf)]
+    return name
+
+
+class DecodeEnv:
+    """Device buffers for one graph: weights, state (double-buffered), rope tables, intermediates.
+
+    ``weights`` maps external weight names to numpy arrays (Q4_K bytes as uint8, bf16 as uint16
+    bit patterns, f32); ``state`` maps state keys (``model.layers.L.conv_state`` ...) to initial
+    numpy arrays.  K/V caches are single in-place buffers; conv and S state rotate between two
+    buffers after every token unless ``inplace_state`` (both names then resolve to one buffer,
+    which the kernels allow: every thread rewrites only what it read).
+    """
+
+    def __init__(self, graph: Graph, weights: dict, state: dict, inplace_state: bool = False):
+        self.graph = graph
+        self.inplace = inplace_state
+        self.ptr: dict[str, int] = {}
+        self.state_bufs: dict[str, list] = {}
+        self.state_cur: dict[str, int] = {}
+        self.non_rotating: set = set()
+        self._owned: list = []
+        for name, t in graph.tensors.items():
+            if t.role == "scalar":
+                continue
+            if t.role == "weight":
+                if name not in weights:
+                    raise KeyError(f"DecodeEnv: no weight for '{name}'")
+                arr = np.ascontiguousarray(weights[name])
+                if arr.nbytes != tensor_bytes(t):
+                    raise ValueError(f"DecodeEnv: '{name}' has {arr.nbytes} bytes, graph says {tensor_bytes(t)}")
+                self.ptr[name] = self._own(rt.to_device(arr))
+            elif t.role == "state":
+                key = state_key(name)
+                if key in self.state_bufs:
+                    continue
+                arr = np.ascontiguousarray(state[key])
+                if arr.nbytes != tensor_bytes(t):
+                    raise ValueError(f"DecodeEnv: state '{key}' has {arr.nbytes} bytes, graph says {tensor_bytes(t)}")
+                a = self._own(rt.to_device(arr))
+                if ".kv_k" in key or ".kv_v" in key or inplace_state:
+                    self.state_bufs[key] = [a, a]
+                    self.non_rotating.add(key)
+                else:
+                    b = self._own(rt.cuAlloc(arr.nbytes))
+                    rt.cuMemset(b, 0, arr.nbytes)
+                    self.state_bufs[key] = [a, b]
+                self.state_cur[key] = 0
+            else:
+                self.ptr[name] = self._own(rt.cuAlloc(tensor_bytes(t)))
+        rt.cuSync()
+
+    def _own(self, p):
+        self._owned.append(p)
+        return p
+
+    def resolve(self, name: str) -> int:
+        t = self.graph.t(name)
+        if t.role == "scalar":
+            raise KeyError(f"resolve: scalar '{name}' is passed by the runner")
+        if t.role == "state":
+            key = state_key(name)
+            cur = self.state_cur[key]
+            is_new = name.endswith("_new")
+            return self.state_bufs[key][1 - cur if is_new else cur]
+        return self.ptr[name]
+
+    def rotateState(self):
+        for key in self.state_bufs:
+            if key not in self.non_rotating:
+                self.state_cur[key] = 1 - self.state_cur[key]
+
+    def read_state(self, key: str, shape, dtype) -> np.ndarray:
+        return rt.from_device(self.state_bufs[key][self.state_cur[key]], shape, dtype)
+
+    def close(self):
+        for p in self._owned:
+            rt.cuFree(p)
+        self._owned = []
+
+
+# ---------------------------------------------------------------- device-resident loop
+class DeviceLoop:
+    """Greedy decode with token ids and positions in device memory and the step in a HIP graph.
+
+    One replay = one token for every sequence of the batch: the step's kernels, then a small
+    kernel that feeds argmax's indices back as the next token ids, advances the positions and
+    appends the tokens to a device-side history.  State is updated in place.
+    """
+
+    def __init__(self, graph: Graph, env: DecodeEnv, batch: int, start_tokens, start_pos, max_steps: int,
+                 partition: Partition | None = None, use_graph: bool = True):
+        if not env.inplace:
+            raise ValueError("DeviceLoop needs DecodeEnv(inplace_state=True)")
+        self.graph, self.env, self.batch, self.max_steps = graph, env, batch, max_steps
+        self.compiled = compileStep(graph, partition or choosePartition(graph), batch, device_scalars=True)
+        ids = np.asarray(start_tokens, np.int32).reshape(batch)
+        pos = np.broadcast_to(np.asarray(start_pos, np.int32), (batch,)).copy()
+        self.d_ids = rt.to_device(ids)
+        self.d_pos = rt.to_device(pos)
+        self.d_hist = rt.cuAlloc(max_steps * batch * 8)
+        self.d_count = rt.to_device(np.zeros(1, np.int32))
+        argmax = next(n for n in graph.nodes if n.op == "argmax")
+        self.idx_ptr = env.resolve(argmax.outputs[1].tensorName)
+        self.val_ptr = env.resolve(argmax.outputs[0].tensorName)
+        self.k_adv = rt.compileAndLoad(f"advance batch={batch} max_steps={max_steps}")
+        self.launches = []
+        for plan, k in self.compiled.schedule:
+            args = [self.d_ids if a == "token_id" else self.d_pos if a == "pos" else env.resolve(a) for a in plan.args]
+            self.launches.append((k, plan, args))
+        self.launches.append((self.k_adv, None, [self.idx_ptr, self.val_ptr, self.d_ids, self.d_pos, self.d_hist, self.d_count]))
+        self.graph_exec = None
+        self.use_graph = use_graph
+        self.steps_done = 0
+
+    def _enqueue(self):
+        for k, plan, args in self.launches:
+            rc = rt.cuLaunch(k, [1, 1, 1], [128, 1, 1], args)
+            if rc != 0:
+                raise rt.BunkerError(f"{plan.name if plan else 'advance'}: {rt.last_error()} (rc={rc})")
+
+    def step(self, n: int = 1):
+        for _ in range(n):
+            if self.steps_done >= self.max_steps:
+                raise RuntimeError("DeviceLoop: history is full")
+            if self.graph_exec is not None:
+                self.graph_exec.launch()
+            else:
+                # the first token runs eagerly (it also loads every kernel); the recording happens after it
+                self._enqueue()
+                if self.use_graph:
+                    rt.cuSync()
+                    with rt.Graph() as gr:
+                        self._enqueue()
+                    self.graph_exec = gr
+            self.steps_done += 1
+
+    def tokens(self):
+        """(tokens int32 [steps, batch], logits f32 [steps, batch]) generated so far."""
+        rt.cuSync()
+        raw = rt.from_device(self.d_hist, (self.max_steps, self.batch, 2), np.int32)[: self.steps_done]
+        return raw[..., 0].copy(), raw[..., 1].copy().view(np.float32)

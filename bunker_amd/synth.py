@@ -127,3 +127,26 @@ def paged_kv_random(g: np.random.Generator, B: int, L: int, NKV: int = 2, HD: in
     kc = f32_to_bf16(g.standard_normal(shape, dtype=np.float32) * np.float32(sigma))
     vc = f32_to_bf16(g.standard_normal(shape, dtype=np.float32) * np.float32(sigma))
     return kc, vc, bt, ctx
+
+
+def q4k_centered(g: np.random.Generator, N: int, K: int, sigma: float) -> np.ndarray:
+    """Random Q4_K matrix whose dequantised weights are zero-mean with standard deviation ~sigma.
+
+    Per super-block: sub-block scales uniform in 8..31, mins = round(7.5/8 * scale) with
+    dmin = 8*d, so that w = d*sc*nib - dmin*m ~ d*sc*(nib - 7.5); d is drawn around
+    sigma / (4.61 * 19.5) (4.61 = std of a uniform nibble, 19.5 = mean scale).
+    Used for the synthetic model: random-nibble blocks with independent mins have a large
+    common offset per row, which no trained or initialised model has.
+    """
+    if K % Q4K_BLOCK_ELEMS:
+        raise ValueError(f"K={K} must be a multiple of 256")
+    nblk = N * (K // Q4K_BLOCK_ELEMS)
+    out = np.empty((nblk, Q4K_BLOCK_BYTES), np.uint8)
+    d = (sigma / (4.61 * 19.5)) * (0.5 + g.random(nblk, dtype=np.float32))
+    dd = np.stack([d, 8.0 * d], axis=1).astype(np.float16)
+    out[:, 0:4] = dd.view(np.uint8).reshape(nblk, 4)
+    sc = g.integers(8, 32, (nblk, 8), dtype=np.uint8)
+    mn = np.rint(sc.astype(np.float32) * (7.5 / 8.0)).astype(np.uint8)
+    out[:, 4:16] = pack_q4k_scales(sc, mn)
+    out[:, 16:144] = g.integers(0, 256, (nblk, 128), dtype=np.uint8)
+    return out

@@ -7,9 +7,19 @@
  * the HIP kernels with.
  *
  * Each function follows the reference source lines cited above it (paths are
- * relative to the skyne98/bunker tree).  Where the reference leaves the
- * reduction order unspecified (tt.sum / tt.dot), the oracle accumulates in
- * double and rounds once, so it sits in the middle of every legal f32 order.
+ * relative to the skyne98/bunker tree).
+ *
+ * Arithmetic rules (shared with the HIP kernels, so that results agree to the
+ * bit wherever the mathematics allows and do not depend on launch shapes):
+ *   - reductions whose order the reference leaves open (tt.sum / tt.dot) are
+ *     accumulated in double and rounded once to f32;
+ *   - exp, log and 1/sqrt are evaluated in double and rounded once to f32;
+ *   - elementwise f32 arithmetic is done exactly as written, one IEEE
+ *     operation per written operation (build with -ffp-contract=off); a fused
+ *     multiply-add appears only where fmaf() is written;
+ *   - the two k-reductions of the gated-DeltaNet step use f32 fmaf chains over
+ *     16 consecutive rows followed by a sequential sum of the 8 chain results
+ *     (the "canonical order"; pass rows_per_chain = 0 for double accumulation).
  *
  * Pinning status (which independent check fixes each function):
  *   orc_encode_half / orc_f32to16   exhaustive fp16 round trip + hand vectors
@@ -99,6 +109,10 @@ ORC_API uint16_t orc_f32_to_bf16(float f) {
 ORC_API float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
 #define BF(h) orc_bf16_to_f32(h)
 #define TOBF(f) orc_f32_to_bf16(f)
+
+/* transcendental helpers: evaluated in double, rounded once */
+static inline float sigmoidf_(float v) { return (float)(1.0 / (1.0 + exp(-(double)v))); }
+static inline float rsqrt_(double v) { return (float)(1.0 / sqrt(v)); }
 
 /* ------------------------------------------------------------------ */
 /* Q8_1 activation quantizer                                            */
@@ -354,8 +368,7 @@ ORC_API void orc_embed(const uint16_t* E, int32_t token, uint16_t* out, int H) {
 ORC_API void orc_rmsnorm(const uint16_t* x, const uint16_t* w, uint16_t* out, int N) {
   double ss = 0;
   for (int i = 0; i < N; i++) { float v = BF(x[i]); ss += (double)v * (double)v; }
-  float ms = (float)(ss / (double)N);
-  float rstd = (float)(1.0 / sqrt((double)(ms + 1e-6f)));
+  float rstd = rsqrt_(ss / (double)N + 1e-6);
   for (int i = 0; i < N; i++) {
     float y = BF(x[i]) * rstd;
     out[i] = TOBF(y * (1.0f + BF(w[i])));
@@ -372,7 +385,6 @@ ORC_API void orc_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, i
   for (int i = 0; i < N; i++) out[i] = TOBF(BF(a[i]) + BF(b[i]));
 }
 
-static inline float sigmoidf_(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 /* src/fusion.ts:324-330 emitSwiGLU: bf16((g*(1/(1+exp(-g))))*u), g,u f32. */
 ORC_API void orc_swiglu(const float* g, const float* u, uint16_t* out, int N) {
@@ -401,8 +413,7 @@ ORC_API void orc_headnorm(const uint16_t* x, const uint16_t* w, uint16_t* out,
     const uint16_t* xh = x + (int64_t)h * in_stride;
     double ss = 0;
     for (int i = 0; i < HD; i++) { float v = BF(xh[i]); ss += (double)v * (double)v; }
-    float ms = (float)(ss / (double)HD);
-    float rstd = (float)(1.0 / sqrt((double)(ms + 1e-6f)));
+    float rstd = rsqrt_(ss / (double)HD + 1e-6);
     for (int i = 0; i < HD; i++)
       out[(int64_t)h * HD + i] = TOBF((BF(xh[i]) * rstd) * (1.0f + BF(w[i])));
   }
@@ -448,17 +459,18 @@ ORC_API void orc_argmax(const float* logits, int64_t n, float* val, int32_t* idx
 /* src/emitters.ts:75-120 emitGDN (== prototypes/decode.ts:314-388), one head
  * at a time.  conv_out holds [q(Hg*dk) | k(Hg*dk) | v(Hg*dv)] bf16.
  *   q^ = q*rsqrt(sum q^2 + 1e-6)*dk^-1/2 ;  k^ = k*rsqrt(sum k^2 + 1e-6)
- *   g = exp(-exp(A_log)*softplus(a+dt_bias)), softplus = log2(1+e^x)*ln2
+ *   g = exp(-exp(A_log)*softplus(a+dt_bias)), softplus = ln(1+e^x)
  *   beta = 1/(1+exp(-b))
  *   Sd = g*S ; kS[v] = sum_k k^[k]*Sd[k,v] ; delta = (v-kS)*beta
  *   S' = Sd + k^ (x) delta ; o[v] = sum_k q^[k]*S'[k,v]
  *   out = bf16( o*rsqrt(mean(o^2)+1e-6) * norm_w * (z*sigmoid(z)) )
  * S is [Hg, dk, dv] f32 row-major.  dk must equal dv (the reference reads v
- * with the key tile shape). */
+ * with the key tile shape).  rows_per_chain: 16 = canonical f32 order of the
+ * two k-reductions, 0 = double accumulation. */
 ORC_API void orc_gdn_step(const uint16_t* conv_out, const uint16_t* z, const float* A_log,
                           const uint16_t* dt_bias, const float* a_p, const float* b_p,
                           const float* norm_w, const float* S_in, uint16_t* out, float* S_out,
-                          int Hg, int dk, int dv) {
+                          int Hg, int dk, int dv, int rows_per_chain) {
   int KEYDIM = Hg * dk;
 #pragma omp parallel for schedule(static)
   for (int h = 0; h < Hg; h++) {
@@ -469,8 +481,7 @@ ORC_API void orc_gdn_step(const uint16_t* conv_out, const uint16_t* z, const flo
       float q = BF(conv_out[h * dk + i]), k = BF(conv_out[KEYDIM + h * dk + i]);
       sq += (double)q * q; sk += (double)k * k;
     }
-    float qr = (float)(1.0 / sqrt((double)((float)sq + 1e-6f)));
-    float kr = (float)(1.0 / sqrt((double)((float)sk + 1e-6f)));
+    float qr = rsqrt_(sq + 1e-6), kr = rsqrt_(sk + 1e-6);
     float qscale = qr * (float)(1.0 / sqrt((double)dk));
     for (int i = 0; i < dk; i++) {
       qn[i] = BF(conv_out[h * dk + i]) * qscale;
@@ -478,29 +489,50 @@ ORC_API void orc_gdn_step(const uint16_t* conv_out, const uint16_t* z, const flo
     }
     for (int i = 0; i < dv; i++) vv[i] = BF(conv_out[2 * KEYDIM + h * dv + i]);
     float sp_in = a_p[h] + BF(dt_bias[h]);
-    float softplus = log2f(1.0f + expf(sp_in)) * (float)M_LN2;
-    float decay = expf(-1.0f * (expf(A_log[h]) * softplus));
-    float beta = 1.0f / (1.0f + expf(b_p[h] * -1.0f));
+    float softplus = (float)log1p(exp((double)sp_in));
+    float decay = (float)exp(-(double)((float)exp((double)A_log[h]) * softplus));
+    float beta = sigmoidf_(b_p[h]);
     const float* S = S_in + (int64_t)h * dk * dv;
     float* Sn = S_out + (int64_t)h * dk * dv;
     for (int v = 0; v < dv; v++) {
-      double acc = 0;
-      for (int k = 0; k < dk; k++) acc += (double)kn[k] * (double)(S[k * dv + v] * decay);
-      delta[v] = (vv[v] - (float)acc) * beta;
+      float kS;
+      if (rows_per_chain > 0) {
+        kS = 0.0f;
+        for (int k0 = 0; k0 < dk; k0 += rows_per_chain) {
+          float acc = 0.0f;
+          for (int k = k0; k < k0 + rows_per_chain; k++) acc = fmaf(kn[k], S[k * dv + v] * decay, acc);
+          kS += acc;
+        }
+      } else {
+        double acc = 0;
+        for (int k = 0; k < dk; k++) acc += (double)kn[k] * (double)(S[k * dv + v] * decay);
+        kS = (float)acc;
+      }
+      delta[v] = (vv[v] - kS) * beta;
     }
     for (int k = 0; k < dk; k++)
-      for (int v = 0; v < dv; v++) Sn[k * dv + v] = S[k * dv + v] * decay + kn[k] * delta[v];
+      for (int v = 0; v < dv; v++) Sn[k * dv + v] = fmaf(kn[k], delta[v], S[k * dv + v] * decay);
     double oss = 0;
     for (int v = 0; v < dv; v++) {
-      double acc = 0;
-      for (int k = 0; k < dk; k++) acc += (double)qn[k] * (double)Sn[k * dv + v];
-      o[v] = (float)acc; oss += (double)o[v] * o[v];
+      if (rows_per_chain > 0) {
+        float ov = 0.0f;
+        for (int k0 = 0; k0 < dk; k0 += rows_per_chain) {
+          float acc = 0.0f;
+          for (int k = k0; k < k0 + rows_per_chain; k++) acc = fmaf(qn[k], Sn[k * dv + v], acc);
+          ov += acc;
+        }
+        o[v] = ov;
+      } else {
+        double acc = 0;
+        for (int k = 0; k < dk; k++) acc += (double)qn[k] * (double)Sn[k * dv + v];
+        o[v] = (float)acc;
+      }
+      oss += (double)o[v] * o[v];
     }
-    float oms = (float)(oss / (double)dv);
-    float orstd = (float)(1.0 / sqrt((double)(oms + 1e-6f)));
+    float orstd = rsqrt_(oss / (double)dv + 1e-6);
     for (int v = 0; v < dv; v++) {
       float zv = BF(z[h * dv + v]);
-      float zs = zv * (1.0f / (1.0f + expf(zv * -1.0f)));
+      float zs = zv * sigmoidf_(zv);
       out[h * dv + v] = TOBF(((o[v] * orstd) * norm_w[v]) * zs);
     }
     free(qn);
@@ -516,7 +548,7 @@ ORC_API void orc_gdn_core(const uint16_t* q, const uint16_t* k, const uint16_t* 
                           uint16_t* out, float* S_out, int Hg, int dk, int dv) {
 #pragma omp parallel for schedule(static)
   for (int h = 0; h < Hg; h++) {
-    float decay = expf(g[h]);
+    float decay = (float)exp((double)g[h]);
     const float* S = S_in + (int64_t)h * dk * dv;
     float* Sn = S_out + (int64_t)h * dk * dv;
     float* delta = (float*)malloc(sizeof(float) * (size_t)dv);
@@ -526,7 +558,7 @@ ORC_API void orc_gdn_core(const uint16_t* q, const uint16_t* k, const uint16_t* 
       delta[j] = (BF(v[h * dv + j]) - (float)acc) * beta[h];
     }
     for (int i = 0; i < dk; i++)
-      for (int j = 0; j < dv; j++) Sn[i * dv + j] = S[i * dv + j] * decay + BF(k[h * dk + i]) * delta[j];
+      for (int j = 0; j < dv; j++) Sn[i * dv + j] = fmaf(BF(k[h * dk + i]), delta[j], S[i * dv + j] * decay);
     for (int j = 0; j < dv; j++) {
       double acc = 0;
       for (int i = 0; i < dk; i++) acc += (double)BF(q[h * dk + i]) * (double)Sn[i * dv + j];
@@ -581,7 +613,7 @@ ORC_API void orc_attn_decode_paged(const uint16_t* q, const uint16_t* kc, const 
         float o = (float)(acc[i] / l);
         if (gate) {
           float gv = BF(gate[(int64_t)b * gate_bstride + (int64_t)h * gate_hstride + i]);
-          o = o * (1.0f / (1.0f + expf(gv * -1.0f)));
+          o = o * sigmoidf_(gv);
         }
         out[((int64_t)b * NH + h) * HD + i] = TOBF(o);
       }

@@ -262,14 +262,14 @@ def argmax(logits):
 
 
 # ---------------------------------------------------------------- GDN
-def gdn_step(conv_out, z, A_log, dt_bias, a_p, b_p, norm_w, S, Hg, dk=128, dv=128):
+def gdn_step(conv_out, z, A_log, dt_bias, a_p, b_p, norm_w, S, Hg, dk=128, dv=128, rows_per_chain=16):
     conv_out = _c(conv_out, np.uint16); z = _c(z, np.uint16)
     A_log = _c(A_log, np.float32); dt_bias = _c(dt_bias, np.uint16)
     a_p = _c(a_p, np.float32); b_p = _c(b_p, np.float32); norm_w = _c(norm_w, np.float32)
     S = _c(S, np.float32)
     out = np.empty(Hg * dv, np.uint16); Sn = np.empty(Hg * dk * dv, np.float32)
     lib().orc_gdn_step(_p(conv_out), _p(z), _p(A_log), _p(dt_bias), _p(a_p), _p(b_p), _p(norm_w),
-                       _p(S), _p(out), _p(Sn), Hg, dk, dv)
+                       _p(S), _p(out), _p(Sn), Hg, dk, dv, int(rows_per_chain))
     return out, Sn.reshape(Hg, dk, dv)
 
 

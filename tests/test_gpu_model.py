@@ -1,0 +1,127 @@
+"""Full decode step on the GPU against the CPU restatement.
+
+Every op of the step except attention shares its arithmetic rules with the checker and is equal
+to it bit for bit; attention is held to 2e-2 max-abs.  Two checks follow from that:
+
+* strict: step by step, the checker recomputes the step from the same state and tokens, verifies
+  each attention output of the GPU within tolerance and continues from the GPU's value; logits
+  (all of them), the winning logit and the argmax token id must then be EQUAL, and so must the
+  recurrent state;
+* free-running: both sides decode on their own; token ids are compared, with the top-1/top-2
+  margin of the checker and the observed logit noise reported (a one-ulp bf16 difference in an
+  attention output can cross a Q8_1 rounding boundary downstream, so equality is demanded only
+  where the margin clears the noise).
+
+TINY has the model's structure at small dims; SYNTH is the benchmark's synthetic Qwen3.5-style
+model (BASELINE configs[4]) with KV prefilled to 4096."""
+import numpy as np
+import pytest
+
+from bunker_amd import model, runner, synth_model
+from bunker_amd import runtime as rt
+from bunker_amd.model import SYNTH, TINY
+
+pytestmark = pytest.mark.gpu
+
+
+def _fa_layers(D):
+    return [l for l in range(D.NL) if D.is_full_attention(l)]
+
+
+def _strict_decode(D, W, S, starts, pos0, steps, use_graph):
+    """GPU DeviceLoop one token at a time against the checker continued from the GPU's attention outputs."""
+    from oracle import oracle as orc
+    from oracle.model_ref import RefModel
+    B = len(starts)
+    g = model.buildModelGraph(D, B)
+    env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+    loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=use_graph)
+    fa_nodes = [n for n in g.nodes if n.op == "fa2_attn"]
+    logits_name = next(n for n in g.nodes if n.op == "argmax").inputs[0].tensorName
+    ref = RefModel(D, W, S, batch=B)
+    toks = np.asarray(starts, np.int32); pos = np.full(B, pos0, np.int32)
+    for step in range(steps):
+        loop.step(1)
+        rt.cuSync()
+        inj = {l: rt.from_device(env.resolve(n.outputs[0].tensorName), (B, D.NH * D.HD), np.uint16)
+               for l, n in zip(_fa_layers(D), fa_nodes)}
+        glogits = rt.from_device(env.resolve(logits_name), (B, D.VOCAB), np.float32)
+        idx, val, rlogits = ref.step(toks, pos, attn_override=inj)
+        gt, gv = loop.tokens()
+        assert np.array_equal(glogits.view(np.uint32), rlogits.view(np.uint32)), \
+            f"step {step}: {int((glogits != rlogits).sum())} logits differ, worst {np.abs(glogits - rlogits).max():.3e}"
+        assert np.array_equal(gt[step], idx) and np.array_equal(gv[step].view(np.uint32), val.view(np.uint32)), (step, gt[step], idx)
+        toks, pos = idx, pos + 1
+    print("strict: tokens", loop.tokens()[0].T.tolist(), "max attention |gpu-ref| %.3g" % max(ref.attn_err), flush=True)
+    assert max(ref.attn_err) <= 2e-2
+    # recurrent state after the last token
+    for l in range(D.NL):
+        p = f"model.layers.{l}"
+        if not D.is_full_attention(l):
+            Sg = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32)
+            assert np.array_equal(Sg.view(np.uint32), ref.S[f"{p}.s_state"].view(np.uint32)), p
+            cg = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)
+            assert np.array_equal(cg, ref.S[f"{p}.conv_state"]), p
+        else:
+            kg = env.read_state(f"{p}.kv_k", ref.S[f"{p}.kv_k"].shape, np.uint16)
+            assert np.array_equal(kg, ref.S[f"{p}.kv_k"]), p
+            vg = env.read_state(f"{p}.kv_v", (B, D.MAX_LEN // 16, D.NKV, D.HD, 16), np.uint16).swapaxes(-1, -2)
+            assert np.array_equal(vg, ref.S[f"{p}.kv_v"]), p
+    env.close()
+    return loop.tokens()
+
+
+def _free_running(D, W, S, starts, pos0, steps, got_tokens, got_vals):
+    from oracle.model_ref import RefModel
+    ref = RefModel(D, W, S, batch=len(starts))
+    rt_, rv = ref.decode(starts, pos0, steps)
+    margins = np.array(ref.margins)
+    noise = np.abs(got_vals - rv)
+    same = got_tokens == rt_
+    print("free-running: reference tokens", rt_.T.tolist(), "| equal %d/%d | min margin %.4g | max logit noise %.4g"
+          % (same.sum(), same.size, margins.min(), noise.max()), flush=True)
+    # until the first divergence of a sequence, a token may differ only where the margin does not clear the noise
+    for b in range(len(starts)):
+        for s in range(steps):
+            if not same[s, b]:
+                assert margins[s, b] <= 8 * max(noise[: s + 1, b].max(), 1e-6), (s, b, margins[s, b], noise[: s + 1, b].max())
+                break
+    assert same[0].all() or margins[0].min() < 1e-3
+
+
+def test_tiny_model_reference_loop(orc):
+    """The reference's host loop (scalars per launch, double-buffered state) on the tiny model."""
+    D = TINY
+    W = synth_model.synth_weights(D, seed=11)
+    S = synth_model.synth_state(D, batch=1, seed=12)
+    steps, pos0 = 6, 40
+    g = model.buildModelGraph(D, 1)
+    env = runner.DecodeEnv(g, W, synth_model.device_state(S))
+    compiled = runner.compileStep(g, runner.choosePartition(g))
+    out = runner.runGraphDecode(compiled, env.resolve, 77, steps, lambda t, v, s: env.rotateState(), startPos=pos0)
+    toks = np.array(out["tokens"], np.int32)[:, None]; vals = np.array(out["logits"], np.float32)[:, None]
+    st, sv = _strict_decode(D, W, S, [77], pos0, steps, use_graph=False)
+    # the host loop and the device-resident loop run the same kernels: same tokens, same logits, bit for bit
+    assert np.array_equal(toks, st) and np.array_equal(vals.view(np.uint32), sv.view(np.uint32))
+    _free_running(D, W, S, [77], pos0, steps, toks, vals)
+    env.close()
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_tiny_model_device_loop_batch3(orc, use_graph):
+    D = TINY
+    W = synth_model.synth_weights(D, seed=11)
+    S = synth_model.synth_state(D, batch=3, seed=13)
+    toks, vals = _strict_decode(D, W, S, [77, 5, 900], 40, 6, use_graph)
+    _free_running(D, W, S, [77, 5, 900], 40, 6, toks, vals)
+
+
+def test_synthetic_qwen35_decode_step_bs1(orc):
+    """BASELINE configs[4], batch 1: 24 layers (3 GDN : 1 FA), hidden 2048, FFN 6144, vocab 151936, KV at 4096."""
+    D = SYNTH
+    print("generating weights", flush=True)
+    W = synth_model.synth_weights(D, seed=2026)
+    S = synth_model.synth_state(D, batch=1, seed=7)
+    steps, pos0, tok0 = 6, 4096, 9419          # start token of the reference's benches (bench_graph_decode.ts:77)
+    toks, vals = _strict_decode(D, W, S, [tok0], pos0, steps, use_graph=True)
+    _free_running(D, W, S, [tok0], pos0, steps, toks, vals)

@@ -140,6 +140,8 @@ def test_gemv_q4k_q8_1_decode_shapes(orc, dev, name):
     y = rt.from_device(dy, (N,), np.float32)
     ref = orc.gemv_q4k_q8_1(W, xq, N, K, acc64=True)
     _assert_rel(y, ref)
+    # every term after the integer dots is exact in double, so the f32 result equals the host's to the bit
+    assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), int((y != ref).sum())
     # run-to-run determinism (fixed reduction order, no atomics)
     rt.gemv_q4k_q8_1(dW, dxq, dy, N, K)
     assert np.array_equal(rt.from_device(dy, (N,), np.float32).view(np.uint32), y.view(np.uint32))
@@ -154,7 +156,9 @@ def test_gemv_q4k_q8_1_ragged_shapes(orc, dev, N, K):
     dW, dxq = dev.up(W), dev.up(xq)
     dy = dev.empty(N * 4)
     rt.gemv_q4k_q8_1(dW, dxq, dy, N, K)
-    _assert_rel(rt.from_device(dy, (N,), np.float32), orc.gemv_q4k_q8_1(W, xq, N, K))
+    y = rt.from_device(dy, (N,), np.float32); ref = orc.gemv_q4k_q8_1(W, xq, N, K)
+    _assert_rel(y, ref)
+    assert np.array_equal(y.view(np.uint32), ref.view(np.uint32))
     dI = dev.empty(N * (K // 32) * 4)
     rt.q4k_q8_1_subdots(dW, dxq, dI, N, K)
     assert np.array_equal(rt.from_device(dI, (N, K // 32), np.int32), orc.q4k_q8_1_subdots(W, xq, N, K))
@@ -173,6 +177,7 @@ def test_gemv_q4k_q8_1_epilogues_and_batch(orc, dev):
     rt.gemv_q4k_q8_1(dW, dxq, dy, N, K, batch=B)
     y = rt.from_device(dy, (B, N), np.float32)
     _assert_rel(y, ref)
+    assert np.array_equal(y.view(np.uint32), ref.view(np.uint32))
     # bf16 output: exactly the RNE rounding of the kernel's own f32 result
     rt.gemv_q4k_q8_1(dW, dxq, dy, N, K, batch=B, out_dtype=rt.BF16)
     yb = rt.from_device(dy, (B, N), np.uint16)

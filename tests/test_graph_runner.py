@@ -1,0 +1,95 @@
+"""Host logic without a GPU: the decode graph has the reference's shape (node count, op sequence,
+slot order per op), the runner orders it correctly, and the CPU checker runs a tiny model."""
+import numpy as np
+
+from bunker_amd import model, runner, synth_model
+from bunker_amd.model import REFERENCE, SYNTH, TINY
+
+
+def test_node_count_and_op_sequence():
+    g = model.buildModelGraph(SYNTH)
+    # 1 + 18*17 + 6*19 + 3 (src/model.ts:46-204)
+    assert len(g.nodes) == 424 == model.expected_node_count(SYNTH)
+    assert len(model.buildModelGraph(REFERENCE).nodes) == 424
+    ops = [n.op for n in g.nodes]
+    gdn_layer = ["rmsnorm", "gemm", "gemm", "conv1d_decode", "gemm", "gemm", "gdn_delta_rule", "gemm", "cast", "add",
+                 "rmsnorm", "gemm", "gemm", "swiglu", "gemm", "cast", "add"]
+    fa_layer = ["rmsnorm", "gemm", "gemm", "gemm", "qnorm", "rope", "knorm", "ropek", "fa2_attn", "gemm", "cast", "add",
+                "rmsnorm", "gemm", "gemm", "swiglu", "gemm", "cast", "add"]
+    expect = ["embed"] + (gdn_layer * 3 + fa_layer) * 6 + ["rmsnorm", "gemm", "argmax"]
+    assert ops == expect
+
+
+def test_slot_order_per_op():
+    g = model.buildModelGraph(SYNTH)
+    plans = {p.group[0].op: p for p in runner.compilePartition(g, runner.choosePartition(g))}
+    names = lambda op: [a.split("_", 1)[1] if a.startswith("n") and a[1].isdigit() else a for a in plans[op].args]
+    assert names("embed") == ["embed.weight", "token_id", "out"]
+    assert names("argmax") == ["out", "val", "idx"]
+    assert [a.split(".")[-1] for a in names("fa2_attn")] == ["out", "out", "out", "out", "kv_k_in", "kv_v_in", "pos", "out",
+                                                              "kv_k_new", "kv_v_new"]
+    assert names("rope")[1:] == ["rope_cos", "rope_sin", "pos"] and len(plans["rope"].args) == 4
+    gd = names("gdn_delta_rule")
+    assert [a.split(".")[-1] for a in gd] == ["out", "out", "A_log", "dt_bias", "out", "out", "weight", "s_state_in", "out",
+                                              "s_state_new"]
+    cv = names("conv1d_decode")
+    assert [a.split(".")[-1] for a in cv] == ["out", "conv_state_in", "weight", "out", "conv_state_new"]
+    # residual adds: attention side is add(cast, h), MLP side is add(h, cast) (src/model.ts:113-117, 184-188)
+    adds = [n for n in g.nodes if n.op == "add"]
+    first, second = adds[0], adds[1]
+    assert g.t(first.inputs[0].tensorName).producer.op == "cast"
+    assert g.t(second.inputs[1].tensorName).producer.op == "cast"
+
+
+def test_specs_carry_the_baked_constants():
+    g = model.buildModelGraph(SYNTH, batch=4)
+    specs = {n.op: runner.node_spec(n, 4, True) for n in g.nodes}
+    assert specs["embed"] == "embed H=2048 VOCAB=151936 batch=4 ids_dev=1"
+    assert specs["fa2_attn"] == "fa2_attn HD=256 NH=16 NKV=2 MAX_LEN=4352 batch=4 pos_dev=1"
+    qkv = next(n for n in g.nodes if n.op == "gemm")
+    assert runner.node_spec(qkv) == "gemm N=6144 K=2048 cast=1"
+
+
+def test_topo_order_respects_dependencies_and_in_place_rope():
+    g = model.buildModelGraph(TINY)
+    # scramble the partition: the order must come from the dependencies alone
+    part = runner.choosePartition(g)[::-1]
+    order = [grp[0] for grp in runner.topoOrder(g, part)]
+    posn = {n.id: i for i, n in enumerate(order)}
+    for n in g.nodes:
+        for d in g.deps()[n.id]:
+            assert posn[d] < posn[n.id]
+    for n in g.nodes:
+        if n.op in ("rope", "ropek"):
+            fa = next(c for c in g.t(n.inputs[0].tensorName).consumers if c.op == "fa2_attn")
+            assert posn[n.id] < posn[fa.id]
+
+
+def test_state_keys_and_bytes():
+    assert runner.state_key("n12_model.layers.0.conv_state_new") == "model.layers.0.conv_state"
+    assert runner.state_key("model.layers.3.kv_k_in") == "model.layers.3.kv_k"
+    g = model.buildModelGraph(SYNTH)
+    assert runner.tensor_bytes(g.t("lm_head.weight")) == 175030272
+    assert runner.tensor_bytes(g.t("model.layers.0.s_state_in")) == 16 * 128 * 128 * 4
+    total_q4k = sum(runner.tensor_bytes(t) for t in g.tensors.values() if t.type.dtype == "q4_k")
+    assert 0.95e9 < total_q4k < 1.05e9          # ~990 MB of weights stream per token
+
+
+def test_reference_model_runs_on_cpu(orc):
+    from oracle.model_ref import RefModel
+    W = synth_model.synth_weights(TINY, seed=5)
+    S = synth_model.synth_state(TINY, batch=2, seed=6)
+    m = RefModel(TINY, W, S, batch=2)
+    toks, vals = m.decode([3, 700], [40, 41], steps=3)
+    assert toks.shape == (3, 2) and toks.min() >= 0 and toks.max() < TINY.VOCAB
+    m2 = RefModel(TINY, W, S, batch=2)
+    t2, v2 = m2.decode([3, 700], [40, 41], steps=3)
+    assert np.array_equal(toks, t2) and np.array_equal(vals, v2)
+    # sequences are independent: sequence 1 alone gives the same tokens
+    S1 = {k: v[1:2] for k, v in S.items()}
+    t3, _ = RefModel(TINY, W, S1, batch=1).decode([700], [41], steps=3)
+    assert np.array_equal(t3[:, 0], toks[:, 1])
+    # the cache holds the new tokens' keys at positions 40..42 of sequence 0
+    k0 = "model.layers.3.kv_k"
+    assert not np.array_equal(m.S[k0][0, 40 // 16, :, 40 % 16], S[k0][0, 40 // 16, :, 40 % 16])
+    assert np.array_equal(m.S[k0][0, 0], S[k0][0, 0])
