@@ -67,11 +67,26 @@ static int run_gemv(Kernel& k, const uint64_t* s) {
 // ---- op: gemm (the model graph's M=1 matmul, src/model.ts:71-73)
 // slots: A (bf16 [batch,K]), B (Q4_K [N,K]), out (f32, or bf16 with cast=1)
 // params: N, K, cast=0, batch=1.  A is quantized to Q8_1 into the handle's workspace first.
+// Batches of GEMM_MFMA_MIN_BATCH rows and more go to the int8 MFMA kernel (32 rows per tile), smaller
+// ones stream the weights once per row through the GEMV; mfma=0/1 in the spec forces either.
+constexpr int GEMM_MFMA_MIN_BATCH = 8;
+static int matmul_q8_1(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype, const void* res, int force) {
+  const bool mfma = force >= 0 ? force != 0 : batch >= GEMM_MFMA_MIN_BATCH;
+  if (!mfma) return launch_gemv_q4k_q8_1(W, xq, y, N, K, batch, out_dtype, res);
+  for (int b0 = 0; b0 < batch; b0 += 32) {
+    const int nb = batch - b0 < 32 ? batch - b0 : 32;
+    const size_t osz = out_dtype == DT_BF16 ? 2 : 4;
+    int rc = launch_gemm_q4k_q8_1_mfma(W, (const uint8_t*)xq + (size_t)b0 * (K / 32) * 36, (uint8_t*)y + (size_t)b0 * N * osz, N, K, nb,
+                                       out_dtype, res ? (const uint8_t*)res + (size_t)b0 * N * 2 : nullptr);
+    if (rc) return rc;
+  }
+  return BK_OK;
+}
 static int run_gemm(Kernel& k, const uint64_t* s) {
   const int N = (int)k.get("N", 0), K = (int)k.get("K", 0), batch = (int)k.get("batch", 1);
   int rc = launch_quantize_q8_1(P<void>(s[0]), DT_BF16, k.scratch, K, batch);
   if (rc) return rc;
-  return launch_gemv_q4k_q8_1(P<void>(s[1]), k.scratch, P<void>(s[2]), N, K, batch, (int)k.get("cast", 0), nullptr);
+  return matmul_q8_1(P<void>(s[1]), k.scratch, P<void>(s[2]), N, K, batch, (int)k.get("cast", 0), nullptr, (int)k.get("mfma", -1));
 }
 
 // ---- op: embed (src/model.ts:53-56)   slots: embed.weight, token_id, out
@@ -286,6 +301,10 @@ int bk_gemv_q4k_f32(uint64_t W, uint64_t x, uint64_t y, int N, int K) {
 int bk_gemv_q4k_q8_1(uint64_t W, uint64_t xq, uint64_t y, int N, int K, int batch, int out_dtype, uint64_t residual) {
   BK_NEED_INIT();
   return launch_gemv_q4k_q8_1(P<void>(W), P<void>(xq), P<void>(y), N, K, batch, out_dtype, P<void>(residual));
+}
+int bk_gemm_q4k_q8_1(uint64_t W, uint64_t xq, uint64_t y, int N, int K, int batch, int out_dtype, uint64_t residual) {
+  BK_NEED_INIT();
+  return matmul_q8_1(P<void>(W), P<void>(xq), P<void>(y), N, K, batch, out_dtype, P<void>(residual), 1);
 }
 int bk_q4k_q8_1_subdots(uint64_t W, uint64_t xq, uint64_t I, int N, int K) {
   BK_NEED_INIT();

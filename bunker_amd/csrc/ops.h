@@ -26,6 +26,10 @@ int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, i
                          int out_dtype, const void* residual);
 int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, int K);
 
+// gemm_mfma.hip
+int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
+                              const void* residual);
+
 // glue.hip
 enum : int { EW_CAST_OP = 0, EW_ADD_OP = 1, EW_SWIGLU_OP = 2 };
 int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void* out, int H, int vocab, int batch);

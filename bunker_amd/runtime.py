@@ -48,6 +48,7 @@ _SIGS = {
     "bk_quantize_q8_1": [u64, i32, u64, i32, i32],
     "bk_gemv_q4k_f32": [u64, u64, u64, i32, i32],
     "bk_gemv_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
+    "bk_gemm_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
     "bk_q4k_q8_1_subdots": [u64, u64, u64, i32, i32],
     "bk_dequant_legacy_i8": [u64, u64, i64], "bk_q4k_nibbles": [u64, u64, i64],
     "bk_q4k_dequant_f32": [u64, u64, i64],
@@ -290,6 +291,10 @@ def gemv_q4k_f32(W: int, x: int, y: int, N: int, K: int) -> None:
 def gemv_q4k_q8_1(W: int, xq: int, y: int, N: int, K: int, batch: int = 1, out_dtype: int = F32,
                   residual: int = 0) -> None:
     _check(cu().bk_gemv_q4k_q8_1(W, xq, y, N, K, batch, out_dtype, residual), "bk_gemv_q4k_q8_1")
+
+
+def gemm_q4k_q8_1(W: int, xq: int, y: int, N: int, K: int, batch: int, out_dtype: int = F32, residual: int = 0) -> None:
+    _check(cu().bk_gemm_q4k_q8_1(W, xq, y, N, K, batch, out_dtype, residual), "bk_gemm_q4k_q8_1")
 
 
 def q4k_q8_1_subdots(W: int, xq: int, I: int, N: int, K: int) -> None:

@@ -95,6 +95,14 @@ BK_API int bk_gemv_q4k_f32(uint64_t W, uint64_t x, uint64_t y, int N, int K);
 BK_API int bk_gemv_q4k_q8_1(uint64_t W, uint64_t xq, uint64_t y, int N, int K, int batch,
                      int out_dtype, uint64_t residual);
 
+/* The same product for a batch of activation rows on the int8 matrix cores
+ * (v_mfma_i32_32x32x32_i8: one 32-element sub-block of K per instruction, 32 batch
+ * rows x 32 weight rows per tile); precedent: int8MatmulTTIR, src/kernel.ts:397-417,
+ * with the post-scale of experiments/q4k_q81_final.ts:214-217.  Arguments as
+ * bk_gemv_q4k_q8_1; returns the same bits as that function for every batch row. */
+BK_API int bk_gemm_q4k_q8_1(uint64_t W, uint64_t xq, uint64_t y, int N, int K, int batch,
+                            int out_dtype, uint64_t residual);
+
 /* Exact int32 sub-block dots I[N, K/32] of the same product (parity hook). */
 BK_API int bk_q4k_q8_1_subdots(uint64_t W, uint64_t xq, uint64_t I, int N, int K);
 

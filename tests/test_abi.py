@@ -17,7 +17,7 @@ def _lib_or_skip():
 def test_header_symbols_are_exported():
     lib = _lib_or_skip()
     names = rt.declared_symbols()
-    assert len(names) >= 32 and len(set(names)) == len(names)
+    assert len(names) >= 37 and len(set(names)) == len(names)
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
     # the Python binding table covers the header exactly

@@ -28,29 +28,32 @@ def _fa_layers(D):
     return [l for l in range(D.NL) if D.is_full_attention(l)]
 
 
-def _strict_decode(D, W, S, starts, pos0, steps, use_graph):
-    """GPU DeviceLoop one token at a time against the checker continued from the GPU's attention outputs."""
-    from oracle import oracle as orc
+def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None):
+    """GPU DeviceLoop one token at a time against the checker continued from the GPU's attention outputs.
+
+    check: the sequences of the batch the checker recomputes (all by default; sequences are independent)."""
     from oracle.model_ref import RefModel
     B = len(starts)
+    check = list(range(B)) if check is None else list(check)
     g = model.buildModelGraph(D, B)
     env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
     loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=use_graph)
     fa_nodes = [n for n in g.nodes if n.op == "fa2_attn"]
     logits_name = next(n for n in g.nodes if n.op == "argmax").inputs[0].tensorName
-    ref = RefModel(D, W, S, batch=B)
-    toks = np.asarray(starts, np.int32); pos = np.full(B, pos0, np.int32)
+    ref = RefModel(D, W, {k: np.asarray(v)[check] for k, v in S.items()}, batch=len(check))
+    toks = np.asarray(starts, np.int32)[check]; pos = np.full(len(check), pos0, np.int32)
     for step in range(steps):
         loop.step(1)
         rt.cuSync()
-        inj = {l: rt.from_device(env.resolve(n.outputs[0].tensorName), (B, D.NH * D.HD), np.uint16)
+        inj = {l: rt.from_device(env.resolve(n.outputs[0].tensorName), (B, D.NH * D.HD), np.uint16)[check]
                for l, n in zip(_fa_layers(D), fa_nodes)}
-        glogits = rt.from_device(env.resolve(logits_name), (B, D.VOCAB), np.float32)
+        glogits = rt.from_device(env.resolve(logits_name), (B, D.VOCAB), np.float32)[check]
         idx, val, rlogits = ref.step(toks, pos, attn_override=inj)
         gt, gv = loop.tokens()
         assert np.array_equal(glogits.view(np.uint32), rlogits.view(np.uint32)), \
             f"step {step}: {int((glogits != rlogits).sum())} logits differ, worst {np.abs(glogits - rlogits).max():.3e}"
-        assert np.array_equal(gt[step], idx) and np.array_equal(gv[step].view(np.uint32), val.view(np.uint32)), (step, gt[step], idx)
+        assert np.array_equal(gt[step][check], idx) and np.array_equal(gv[step][check].view(np.uint32), val.view(np.uint32)), \
+            (step, gt[step], idx)
         toks, pos = idx, pos + 1
     print("strict: tokens", loop.tokens()[0].T.tolist(), "max attention |gpu-ref| %.3g" % max(ref.attn_err), flush=True)
     assert max(ref.attn_err) <= 2e-2
@@ -58,14 +61,14 @@ def _strict_decode(D, W, S, starts, pos0, steps, use_graph):
     for l in range(D.NL):
         p = f"model.layers.{l}"
         if not D.is_full_attention(l):
-            Sg = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32)
+            Sg = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32)[check]
             assert np.array_equal(Sg.view(np.uint32), ref.S[f"{p}.s_state"].view(np.uint32)), p
-            cg = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)
+            cg = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)[check]
             assert np.array_equal(cg, ref.S[f"{p}.conv_state"]), p
         else:
-            kg = env.read_state(f"{p}.kv_k", ref.S[f"{p}.kv_k"].shape, np.uint16)
+            kg = env.read_state(f"{p}.kv_k", (B,) + ref.S[f"{p}.kv_k"].shape[1:], np.uint16)[check]
             assert np.array_equal(kg, ref.S[f"{p}.kv_k"]), p
-            vg = env.read_state(f"{p}.kv_v", (B, D.MAX_LEN // 16, D.NKV, D.HD, 16), np.uint16).swapaxes(-1, -2)
+            vg = env.read_state(f"{p}.kv_v", (B, D.MAX_LEN // 16, D.NKV, D.HD, 16), np.uint16)[check].swapaxes(-1, -2)
             assert np.array_equal(vg, ref.S[f"{p}.kv_v"]), p
     env.close()
     return loop.tokens()
@@ -125,3 +128,26 @@ def test_synthetic_qwen35_decode_step_bs1(orc):
     steps, pos0, tok0 = 6, 4096, 9419          # start token of the reference's benches (bench_graph_decode.ts:77)
     toks, vals = _strict_decode(D, W, S, [tok0], pos0, steps, use_graph=True)
     _free_running(D, W, S, [tok0], pos0, steps, toks, vals)
+
+
+def test_tiny_model_batch32_mfma_path(orc):
+    """Batch 32 sends every matmul through the int8 MFMA kernel; results stay equal to the checker's."""
+    D = TINY
+    W = synth_model.synth_weights(D, seed=11)
+    S = synth_model.synth_state(D, batch=32, seed=14)
+    starts = [(37 * i + 5) % D.VOCAB for i in range(32)]
+    toks, vals = _strict_decode(D, W, S, starts, 40, 4, use_graph=True)
+    # a sequence decodes to the same tokens alone (GEMV path) as inside the batch (MFMA path)
+    S1 = {k: np.asarray(v)[7:8] for k, v in S.items()}
+    t1, v1 = _strict_decode(D, W, S1, [starts[7]], 40, 4, use_graph=False)
+    assert np.array_equal(t1[:, 0], toks[:, 7]) and np.array_equal(v1[:, 0].view(np.uint32), vals[:, 7].view(np.uint32))
+
+
+def test_synthetic_qwen35_decode_step_bs32(orc):
+    """BASELINE configs[4], batch 32: 32 different start tokens and states, int8 MFMA matmuls; three of
+    the sequences are recomputed by the checker."""
+    D = SYNTH
+    W = synth_model.synth_weights(D, seed=2026)
+    S = synth_model.synth_state(D, batch=32, seed=8, share_kv_across_batch=True)
+    starts = [(9419 + 4099 * i) % D.VOCAB for i in range(32)]
+    _strict_decode(D, W, S, starts, 4096, 2, use_graph=True, check=[0, 13, 31])

@@ -248,3 +248,28 @@ def test_gemm_op_launch_surface(orc, dev):
         rt.compileAndLoad("gemm N=16 K=100")
     with pytest.raises(rt.BunkerError, match="multiple of 256"):
         rt.gemv_q4k_q8_1(1 << 20, 1 << 20, 1 << 20, 16, 100)
+
+
+@pytest.mark.parametrize("N,K,B", [(6144, 2048, 32), (2048, 6144, 32), (16, 2048, 32), (100, 768, 7), (2048, 4096, 17),
+                                   (4096, 2048, 40)])
+def test_gemm_mfma_equals_gemv_and_oracle(orc, dev, N, K, B):
+    """Batched int8-MFMA matmul: same bits as the GEMV path and as the host loop in double, for every batch row."""
+    print(f"gemm mfma N={N} K={K} B={B}", flush=True)
+    g = synth.rng(700 + N + K + B)
+    W = synth.q4k_random(g, N, K)
+    x = g.standard_normal((B, K)).astype(np.float32)
+    x[0] = 0.0                                              # an all-zero activation row
+    xq = np.stack([orc.pack_q8_1(r) for r in x])
+    res = synth.f32_to_bf16(g.standard_normal((B, N)).astype(np.float32))
+    dW, dxq, dres = dev.up(W), dev.up(xq), dev.up(res)
+    dy, dy2 = dev.empty(B * N * 4), dev.empty(B * N * 4)
+    rt.gemm_q4k_q8_1(dW, dxq, dy, N, K, B)
+    y = rt.from_device(dy, (B, N), np.float32)
+    ref = np.stack([orc.gemv_q4k_q8_1(W, xq[b], N, K) for b in range(B)])
+    _assert_rel(y, ref)
+    assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), int((y != ref).sum())
+    rt.gemv_q4k_q8_1(dW, dxq, dy2, N, K, batch=B)
+    assert np.array_equal(rt.from_device(dy2, (B, N), np.float32).view(np.uint32), y.view(np.uint32))
+    rt.gemm_q4k_q8_1(dW, dxq, dy, N, K, B, out_dtype=rt.BF16, residual=dres)
+    ya = rt.from_device(dy, (B, N), np.uint16)
+    assert np.array_equal(ya, orc.add_bf16(synth.f32_to_bf16(y).ravel(), res.ravel()).reshape(B, N))
