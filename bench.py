@@ -12,6 +12,11 @@ The timed region holds exactly K steps; launches are grouped by shape with a HIP
 between groups (recorded on the library's stream), which gives each kernel's average
 launch duration from the same region that `value` is taken from.
 
+Further sections, reported under "decode" and "kernels" of the same line: greedy decode of the
+synthetic Qwen3.5-style model (BASELINE configs[4]) at batch 1 and 32 in tok/s against the
+byte floor of one step, and the gated-DeltaNet step (configs[2]) and the paged decode attention
+(configs[3]) in algorithmic GB/s.  `--sections gemv` runs the headline part alone.
+
 Prints ONE JSON line.  `python bench.py --gpus 1 --steps 200 --warmup 20`.
 """
 from __future__ import annotations
@@ -63,15 +68,141 @@ def cpu_baseline(seconds_target=12.0):
                       f"{dt:.1f} s on {threads} OpenMP threads of the host CPU"}
 
 
+def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16):
+    """tok/s of the full synthetic decode step at batch 1 and 32 (device-resident loop, HIP graph replay)."""
+    from bunker_amd import model, runner, synth_model
+
+    D = model.SYNTH
+    W = synth_model.synth_weights(D, seed=2026)
+    out = {}
+    dev_w = None
+    envs = []
+    weight_bytes = sum(v.nbytes for k, v in W.items() if v.dtype == np.uint8)
+    for B, steps in ((1, steps_bs1), (32, steps_bs32)):
+        S = synth_model.device_state(synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True))
+        g = model.buildModelGraph(D, B)
+        env = runner.DecodeEnv(g, W, S, inplace_state=True, device_weights=dev_w)
+        envs.append(env)
+        dev_w = dev_w or env.weight_ptrs()
+        starts = [(9419 + 4099 * i) % D.VOCAB for i in range(B)]
+        warm = 3
+        loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph)
+        loop.step(warm)
+        rt.cuSync()
+        e0, e1 = rt.Event(), rt.Event()
+        t0 = time.perf_counter()
+        e0.record()
+        loop.step(steps)
+        e1.record()
+        rt.cuSync()
+        wall = time.perf_counter() - t0
+        ms = e0.elapsed_ms(e1) / steps
+        toks, _ = loop.tokens()
+        # bytes one step must move: every Q4_K weight once, GDN state read+write, the KV prefix of the FA layers
+        n_gdn = sum(1 for l in range(D.NL) if not D.is_full_attention(l))
+        n_fa = D.NL - n_gdn
+        state_bytes = B * n_gdn * (2 * D.LVH * D.LKD * D.LVD * 4) + B * n_fa * (2 * D.NKV * 4097 * D.HD * 2)
+        floor_us = (weight_bytes + state_bytes) / 8e12 * 1e6
+        out[f"bs{B}"] = {"tok_per_s": round(B / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
+                         "wall_ms_per_step": round(wall * 1e3 / steps, 4), "steps": steps,
+                         "launch": "hip graph replay" if use_graph else "eager", "kernels_per_step": len(loop.launches), "step_bytes": weight_bytes + state_bytes,
+                         "hbm_floor_us": round(floor_us, 1), "frac_of_floor": round(floor_us / (ms * 1e3), 4),
+                         "first_tokens": toks[:4, 0].tolist()}
+    for env in envs:
+        env.close()
+    return out
+
+
+def _time_launches(rt, enqueue, use_graph):
+    """Microseconds for everything `enqueue` launches, by HIP events on the library's stream."""
+    e0, e1 = rt.Event(), rt.Event()
+    if use_graph:
+        with rt.Graph() as gr:
+            enqueue()
+        rt.cuSync()
+        e0.record(); gr.launch(); e1.record()
+    else:
+        rt.cuSync()
+        e0.record(); enqueue(); e1.record()
+    rt.cuSync()
+    return e0.elapsed_ms(e1) * 1e3
+
+
+def bench_kernels(rt, synth, use_graph=True, iters=50):
+    """Gated-DeltaNet step (configs[2]) and paged decode attention (configs[3]) in algorithmic GB/s."""
+    g = synth.rng(5)
+    res = {}
+    bf = synth.f32_to_bf16
+    for B in (1, 8):
+        Hg = 32
+        ROT = max(2, 600 // (B * Hg * 131072 // (1 << 20) + 1))      # rotate states through > 512 MiB
+        ROT = min(ROT, 140)
+        S = (g.standard_normal((B, Hg, 128, 128), dtype=np.float32) * np.float32(0.02))
+        dS = [rt.to_device(S) for _ in range(ROT)]
+        q = rt.to_device(bf(g.standard_normal((B, Hg, 128), dtype=np.float32) / np.float32(11.3)))
+        k = rt.to_device(bf(g.standard_normal((B, Hg, 128), dtype=np.float32) / np.float32(11.3)))
+        v = rt.to_device(bf(g.standard_normal((B, Hg, 128), dtype=np.float32)))
+        gl = rt.to_device((-np.log1p(np.exp(g.standard_normal((B, Hg)))) * 0.1).astype(np.float32))
+        beta = rt.to_device((1 / (1 + np.exp(-g.standard_normal((B, Hg))))).astype(np.float32))
+        dout = rt.cuAlloc(B * Hg * 128 * 2)
+        for i in range(5):
+            rt.gdn_core(q, k, v, gl, beta, dS[i % ROT], dout, dS[i % ROT], Hg, B)
+        def run_gdn():
+            for i in range(iters):
+                rt.gdn_core(q, k, v, gl, beta, dS[i % ROT], dout, dS[i % ROT], Hg, B)
+
+        us = _time_launches(rt, run_gdn, use_graph) / iters
+        nbytes = B * Hg * (2 * 128 * 128 * 4 + 3 * 128 * 2 + 128 * 2 + 8)
+        res[f"gdn_step_b{B}"] = {"us": round(us, 3), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                                 "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        for p in dS + [q, k, v, gl, beta, dout]:
+            rt.cuFree(p)
+    for B, L in ((1, 4096), (8, 4096), (1, 32768), (8, 32768)):
+        NH, NKV, HD = 16, 2, 256
+        ppseq = L // 16
+        ctx = g.integers(L // 2, L + 1, B).astype(np.int32)
+        bt = g.permutation(B * ppseq).astype(np.int32).reshape(B, ppseq)
+        page = bf(g.standard_normal((64, NKV, 16, HD), dtype=np.float32))
+        reps = (B * ppseq + 63) // 64
+        cache = np.tile(page, (reps, 1, 1, 1))[: B * ppseq]
+        ROT = max(2, min(8, int(600e6 // (2 * cache.nbytes)) + 1))
+        kcs = [rt.to_device(cache) for _ in range(ROT)]
+        vcs = [rt.to_device(cache) for _ in range(ROT)]
+        dq = rt.to_device(bf(g.standard_normal((B, NH, HD), dtype=np.float32)))
+        dbt, dctx = rt.to_device(bt), rt.to_device(ctx)
+        dout, dlse = rt.cuAlloc(B * NH * HD * 2), rt.cuAlloc(B * NH * 4)
+        splits, ws = rt.attn_plan(B, NKV, L)
+        dws = rt.cuAlloc(ws) if ws else 0
+
+        def run(i):
+            rt.attn_decode(dq, kcs[i % ROT], vcs[i % ROT], dbt, ppseq, dctx, L, dout, dlse, B, NH, NKV, HD, 16, splits, dws, ws)
+
+        for i in range(3):
+            run(i)
+        us = _time_launches(rt, lambda: [run(i) for i in range(iters)], use_graph) / iters
+        nbytes = int(sum(2 * NKV * int(c) * HD * 2 for c in ctx) + B * NH * HD * 2 * 2 + B * NH * 4)
+        res[f"attn_decode_b{B}_L{L}"] = {"us": round(us, 3), "bytes": nbytes, "splits": splits,
+                                         "GBps": round(nbytes / us / 1e3, 1),
+                                         "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        for p in kcs + vcs + [dq, dbt, dctx, dout, dlse] + ([dws] if dws else []):
+            rt.cuFree(p)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
-                    help="graph: each shape's K launches are replayed from one HIP graph; "
-                         "stream: K individual launches from Python")
+    ap.add_argument("--sections", default="gemv,decode,kernels",
+                    help="comma list of gemv (headline, always on), decode, kernels")
+    ap.add_argument("--mode", choices=["graph", "stream"], default="stream",
+                    help="GEMV section. stream: K individual launches per shape, queued back to back; "
+                         "graph: the K launches replayed from one HIP graph")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="decode and kernels sections launch eagerly instead of replaying HIP graphs "
+                         "(rocprofv3 cannot trace graph launches on this ROCm)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives, no sharding).", file=sys.stderr)
@@ -174,6 +305,14 @@ def main():
         "per_shape": per_shape,
         "roofline": roofline,
     }
+    for r in sets:
+        for p in r.values():
+            rt.cuFree(p)
+    sections = set(args.sections.split(","))
+    if "decode" in sections:
+        out["decode"] = bench_decode(rt, synth, use_graph=not args.no_graph)
+    if "kernels" in sections:
+        out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

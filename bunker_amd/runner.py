@@ -209,7 +209,8 @@ class DecodeEnv:
     which the kernels allow: every thread rewrites only what it read).
     """
 
-    def __init__(self, graph: Graph, weights: dict, state: dict, inplace_state: bool = False):
+    def __init__(self, graph: Graph, weights: dict, state: dict, inplace_state: bool = False,
+                 device_weights: dict | None = None):
         self.graph = graph
         self.inplace = inplace_state
         self.ptr: dict[str, int] = {}
@@ -221,6 +222,9 @@ class DecodeEnv:
             if t.role == "scalar":
                 continue
             if t.role == "weight":
+                if device_weights is not None and name in device_weights:
+                    self.ptr[name] = device_weights[name]       # already resident; owned by the caller
+                    continue
                 if name not in weights:
                     raise KeyError(f"DecodeEnv: no weight for '{name}'")
                 arr = np.ascontiguousarray(weights[name])
@@ -250,6 +254,10 @@ class DecodeEnv:
     def _own(self, p):
         self._owned.append(p)
         return p
+
+    def weight_ptrs(self) -> dict:
+        """Device pointers of the weights, to share them with another DecodeEnv (device_weights=...)."""
+        return {n: p for n, p in self.ptr.items() if self.graph.tensors[n].role == "weight"}
 
     def resolve(self, name: str) -> int:
         t = self.graph.t(name)
