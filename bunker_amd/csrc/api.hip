@@ -241,6 +241,20 @@ using namespace bk;
 
 extern "C" {
 
+// Tuning hook for experiments: "gemv_rpi" (1, 2, 4, 8), "gemv_cap" (workgroups per CU).
+int bk_tune_set(const char* key, int value) {
+  BK_REQUIRE(key, "bk_tune_set: null key");
+  if (!strcmp(key, "gemv_rpi")) bk::g_tune_rpi = value;
+  else if (!strcmp(key, "gemv_cap")) bk::g_tune_cap = value;
+  else if (!strcmp(key, "gemv_impl")) bk::g_tune_gemv_impl = value;
+  else if (!strcmp(key, "gemv_ks_rows")) bk::g_tune_ks_rows = value;
+  else if (!strcmp(key, "memread_unroll")) bk::g_tune_mr_unroll = value;
+  else if (!strcmp(key, "memread_cap")) bk::g_tune_mr_cap = value;
+  else if (!strcmp(key, "memread_nt")) bk::g_tune_mr_nt = value;
+  else return set_error(BK_ERR_ARG, "bk_tune_set: unknown key '%s'", key);
+  return BK_OK;
+}
+
 int bk_kernel_create(const char* spec) {
   BK_NEED_INIT();
   BK_REQUIRE(spec && *spec, "bk_kernel_create: empty spec");
@@ -290,6 +304,14 @@ int bk_kernel_describe(int kernel, char* buf, int cap) {
   return BK_OK;
 }
 
+int bk_memread(uint64_t src, int64_t bytes, uint64_t sink) {
+  BK_NEED_INIT();
+  return launch_memread(P<void>(src), bytes, P<void>(sink));
+}
+int bk_memcopy(uint64_t src, uint64_t dst, int64_t bytes) {
+  BK_NEED_INIT();
+  return launch_memcopy(P<void>(src), P<void>(dst), bytes);
+}
 int bk_quantize_q8_1(uint64_t x, int x_dtype, uint64_t out, int K, int batch) {
   BK_NEED_INIT();
   return launch_quantize_q8_1(P<void>(x), x_dtype, P<void>(out), K, batch);

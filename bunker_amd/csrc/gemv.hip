@@ -22,7 +22,6 @@
 namespace bk {
 
 constexpr int GEMV_WAVES = 4;           // waves per workgroup
-constexpr int GEMV_RPI = 4;             // rows in flight per wave (independent loads)
 
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
   return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
@@ -125,8 +124,9 @@ __device__ __forceinline__ void store_out(void* __restrict__ y, const uint16_t* 
   }
 }
 
-// NR = number of 64-slot rounds per row (K = 2048*NR when the row fills every round).
-template <int NR, int EPI>
+// NR = number of 64-slot rounds per row (K = 2048*NR when the row fills every round);
+// RPI = rows a wave keeps in flight (independent loads issued before any is consumed).
+template <int NR, int EPI, int RPI>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
     const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq_all, void* __restrict__ y,
     const uint16_t* __restrict__ res, int N, int nb) {
@@ -149,10 +149,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
     boff[r] = (active ? blk : 0) * 144;
   }
 
-  for (int row0 = wave * GEMV_RPI; row0 < N; row0 += nwaves * GEMV_RPI) {
-    uint4 hdr[GEMV_RPI][NR], q[GEMV_RPI][NR];
+  for (int row0 = wave * RPI; row0 < N; row0 += nwaves * RPI) {
+    uint4 hdr[RPI][NR], q[RPI][NR];
 #pragma unroll
-    for (int i = 0; i < GEMV_RPI; i++) {
+    for (int i = 0; i < RPI; i++) {
       const int row = min(row0 + i, N - 1);
       const uint8_t* rp = W + (int64_t)row * row_bytes;
 #pragma unroll
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
       }
     }
 #pragma unroll
-    for (int i = 0; i < GEMV_RPI; i++) {
+    for (int i = 0; i < RPI; i++) {
       double acc = 0.0;
 #pragma unroll
       for (int r = 0; r < NR; r++) {
@@ -239,22 +239,35 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
   }
 }
 
+int g_tune_gemv_impl = 0;               // 1: eight-rows-per-wave layout (gemv8.hip), 0: one row per wave round
+int g_tune_rpi = 4, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows in flight per wave, workgroups per CU
+
 static int gemv_grid(int N, int rows_per_wg) {
   int wgs = (N + rows_per_wg - 1) / rows_per_wg;
-  const int cap = num_cus() * 8;
+  const int cap = num_cus() * g_tune_cap;
   return wgs < cap ? wgs : cap;
+}
+
+template <int NR, int EPI>
+static void launch_q8_1_rpi(dim3 block, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int nb, int batch) {
+  const int rpi = g_tune_rpi;
+  dim3 grid(gemv_grid(N, GEMV_WAVES * rpi), batch);
+  if (rpi == 1) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 1>), grid, block, 0, stream(), w, x, y, r, N, nb);
+  else if (rpi == 2) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 2>), grid, block, 0, stream(), w, x, y, r, N, nb);
+  else if (rpi == 8 && NR == 1) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, (NR == 1 ? 8 : 4)>), grid, block, 0, stream(), w, x, y, r, N, nb);
+  else { grid.x = gemv_grid(N, GEMV_WAVES * 4); hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 4>), grid, block, 0, stream(), w, x, y, r, N, nb); }
 }
 
 template <int EPI>
 static void launch_q8_1_variant(const void* W, const void* xq, void* y, const void* res, int N, int nb, int batch) {
   const int rounds = (nb + 7) / 8;
   dim3 block(GEMV_WAVES * 64);
-  dim3 grid(gemv_grid(N, GEMV_WAVES * GEMV_RPI), batch);
+  dim3 grid(1, batch);
   const uint8_t* w = (const uint8_t*)W; const uint8_t* x = (const uint8_t*)xq; const uint16_t* r = (const uint16_t*)res;
   switch (rounds) {
-    case 1: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<1, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
-    case 2: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<2, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
-    case 3: hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<3, EPI>), grid, block, 0, stream(), w, x, y, r, N, nb); break;
+    case 1: launch_q8_1_rpi<1, EPI>(block, w, x, y, r, N, nb, batch); break;
+    case 2: launch_q8_1_rpi<2, EPI>(block, w, x, y, r, N, nb, batch); break;
+    case 3: launch_q8_1_rpi<3, EPI>(block, w, x, y, r, N, nb, batch); break;
     default:
       grid.x = gemv_grid(N, GEMV_WAVES);
       hipLaunchKernelGGL((gemv_q4k_q8_1_generic_kernel<EPI>), grid, block, 0, stream(), w, x, y, r, N, nb);
@@ -269,6 +282,11 @@ int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, i
   BK_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gemv_q4k_q8_1: out_dtype must be 0 (f32) or 1 (bf16)");
   BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemv_q4k_q8_1: a residual needs bf16 output");
   BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "gemv_q4k_q8_1: W must be 16-byte and xq 4-byte aligned");
+  if (g_tune_gemv_impl == 1) {
+    const int epi = out_dtype == DT_F32 ? 0 : (residual ? 2 : 1);
+    const void* Ws[1] = {W}; void* outs[1] = {y}; const void* rs[1] = {residual};
+    return launch_gemv_group(xq, K, batch, 1, Ws, outs, rs, &N, &epi);
+  }
   const int nb = K / 256;
   if (out_dtype == DT_F32) launch_q8_1_variant<EPI_F32>(W, xq, y, nullptr, N, nb, batch);
   else if (!residual) launch_q8_1_variant<EPI_BF16>(W, xq, y, nullptr, N, nb, batch);

@@ -156,4 +156,64 @@ static int launch_q4k_unpack(const void* blocks, void* out, int64_t nblocks, boo
 int launch_q4k_nibbles(const void* blocks, void* out, int64_t nblocks) { return launch_q4k_unpack(blocks, out, nblocks, false); }
 int launch_q4k_dequant_f32(const void* blocks, void* out, int64_t nblocks) { return launch_q4k_unpack(blocks, out, nblocks, true); }
 
+// ---------------------------------------------------------------- calibration kernels
+// Plain streaming read / copy of a buffer with the access pattern of the GEMV (16 bytes per
+// lane, several loads in flight): what the memory system gives a kernel that does nothing else.
+// Used to calibrate counters and to put the GEMV's GB/s next to an achievable ceiling.
+template <int U, bool NT>
+__global__ __launch_bounds__(256) void memread_kernel(const uint4* __restrict__ p, int64_t n16, uint32_t* __restrict__ sink) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  uint32_t acc = 0;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + (U - 1) * stride < n16; i += U * stride) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      if (NT) {
+        typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+        const u32x4_t t = __builtin_nontemporal_load((const u32x4_t*)(p + i + u * stride));
+        v[u] = make_uint4(t.x, t.y, t.z, t.w);
+      } else {
+        v[u] = p[i + u * stride];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < n16; i += stride) { const uint4 a = p[i]; acc ^= a.x ^ a.y ^ a.z ^ a.w; }
+  if (acc == 0x9e3779b9u) sink[0] = acc;       // practically never true: keeps the loads alive
+}
+__global__ __launch_bounds__(256) void memcopy_kernel(const uint4* __restrict__ p, uint4* __restrict__ q, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) q[i] = p[i];
+}
+
+int g_tune_mr_unroll = 4, g_tune_mr_cap = 8, g_tune_mr_nt = 0;
+
+int launch_memread(const void* src, int64_t bytes, void* sink) {
+  BK_REQUIRE(src && sink && bytes >= 16 && bytes % 16 == 0, "memread: bad arguments");
+  const int64_t n16 = bytes / 16;
+  const int U = g_tune_mr_unroll;
+  int64_t wgs = (n16 + 256 * U - 1) / (256 * U);
+  if (wgs > (int64_t)num_cus() * g_tune_mr_cap) wgs = (int64_t)num_cus() * g_tune_mr_cap;
+  dim3 grid((unsigned)wgs), block(256);
+  const uint4* p = (const uint4*)src; uint32_t* sk = (uint32_t*)sink;
+  const bool nt = g_tune_mr_nt != 0;
+#define MR(UU) do { if (nt) hipLaunchKernelGGL((memread_kernel<UU, true>), grid, block, 0, stream(), p, n16, sk); \
+                    else hipLaunchKernelGGL((memread_kernel<UU, false>), grid, block, 0, stream(), p, n16, sk); } while (0)
+  if (U == 1) MR(1); else if (U == 2) MR(2); else if (U == 8) MR(8); else if (U == 16) MR(16); else MR(4);
+#undef MR
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+int launch_memcopy(const void* src, void* dst, int64_t bytes) {
+  BK_REQUIRE(src && dst && bytes >= 16 && bytes % 16 == 0, "memcopy: bad arguments");
+  const int64_t n16 = bytes / 16;
+  int64_t wgs = (n16 + 255) / 256;
+  if (wgs > num_cus() * 16) wgs = num_cus() * 16;
+  hipLaunchKernelGGL(memcopy_kernel, dim3((unsigned)wgs), dim3(256), 0, stream(), (const uint4*)src, (uint4*)dst, n16);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
 }  // namespace bk

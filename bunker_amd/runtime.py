@@ -43,8 +43,10 @@ _SIGS = {
     "bk_prof_enable": [i32], "bk_prof_reset": [], "bk_prof_report": [C.c_char_p, i32],
     "bk_capture_begin": [], "bk_capture_end": [C.POINTER(u64)], "bk_graph_launch": [u64],
     "bk_graph_destroy": [u64],
+    "bk_tune_set": [C.c_char_p, i32],
     "bk_kernel_create": [C.c_char_p], "bk_launch": [i32, C.POINTER(u64), i32],
     "bk_kernel_describe": [i32, C.c_char_p, i32],
+    "bk_memread": [u64, i64, u64], "bk_memcopy": [u64, u64, i64],
     "bk_quantize_q8_1": [u64, i32, u64, i32, i32],
     "bk_gemv_q4k_f32": [u64, u64, u64, i32, i32],
     "bk_gemv_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
@@ -201,6 +203,10 @@ def cuLaunch(k: LoadedKernel, grid: Sequence[int], block: Sequence[int], args: S
     return cu().bk_launch(k.fn, slots, n)
 
 
+def tune_set(key: str, value: int) -> None:
+    _check(cu().bk_tune_set(key.encode(), int(value)), "bk_tune_set")
+
+
 def last_error() -> str:
     return load_library().bk_last_error().decode("utf-8", "replace")
 
@@ -278,6 +284,14 @@ class Graph:
 
 # ---------------------------------------------------------------- typed entry points
 F32, BF16 = 0, 1
+
+
+def memread(src: int, nbytes: int, sink: int) -> None:
+    _check(cu().bk_memread(src, nbytes, sink), "bk_memread")
+
+
+def memcopy(src: int, dst: int, nbytes: int) -> None:
+    _check(cu().bk_memcopy(src, dst, nbytes), "bk_memcopy")
 
 
 def quantize_q8_1(x: int, out: int, K: int, batch: int = 1, x_dtype: int = F32) -> None:

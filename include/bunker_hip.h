@@ -64,6 +64,9 @@ BK_API int bk_capture_end(uint64_t* graph);
 BK_API int bk_graph_launch(uint64_t graph);
 BK_API int bk_graph_destroy(uint64_t graph);
 
+/* Launch-shape knobs for experiments ("gemv_rpi", "gemv_cap"); defaults are the tuned values. */
+BK_API int bk_tune_set(const char* key, int value);
+
 /* ---- per-op launch surface: replaces compileAndLoad + cuLaunch
  * (src/ttir.ts:488-491, 321-348).  bk_kernel_create takes the op name of the
  * model graph (src/model.ts) and the constants that the reference baked into
@@ -74,6 +77,12 @@ BK_API int bk_graph_destroy(uint64_t graph);
 BK_API int bk_kernel_create(const char* spec);
 BK_API int bk_launch(int kernel, const uint64_t* slots, int nslots);
 BK_API int bk_kernel_describe(int kernel, char* buf, int cap);
+
+/* Calibration kernels: a plain streaming read (16 bytes per lane, result discarded into the
+ * 4-byte sink) and a plain copy, both of `bytes` (multiple of 16).  They give the achievable
+ * HBM rate next to the GEMV's and the scale of the FETCH_SIZE / WRITE_SIZE counters. */
+BK_API int bk_memread(uint64_t src, int64_t bytes, uint64_t sink);
+BK_API int bk_memcopy(uint64_t src, uint64_t dst, int64_t bytes);
 
 /* ---- typed entry points (C / ctypes drivers, parity tests, benchmark) ---- */
 
