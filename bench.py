@@ -287,7 +287,7 @@ def main():
     dom_bytes = sum(per_shape[n]["bytes"] for n in dom) / len(dom)
     dom_us = sum(per_shape[n]["us_per_launch"] for n in dom) / len(dom)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemv_q4k_q8_1_kernel<1,0,4>", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": "gemv_q4k_q8_1_lds_kernel<1,0,4>", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": None}
 
@@ -295,7 +295,7 @@ def main():
         "metric": "Q4_K GEMV HBM GB/s (% of peak); synthetic Qwen3.5 decode tok/s at bs=1/32",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "int8xint4->int32 dots, f32 accumulate", "data": "synthetic",
+        "vs_baseline": None, "dtype": "u4 x int8 -> int32 dots, f64 fold, f32 out", "data": "synthetic",
         "config": {"workload": "Q4_K x Q8_1 GEMV, batch 1, decode shapes qkv/gate_up/down/lm_head "
                                "(BASELINE configs[1]); one step = one launch of each shape",
                    "weight_rotation_MB": round(ROTATION * sum(N * K * 144 // 256 for _, N, K in SHAPES) / 1e6),

@@ -64,7 +64,7 @@ constexpr int DPP_PAIR_ODD = 0xF5;
 // Activation slice of one slot, Q8_1 layout (int8 q[32] @0, fp16 d @32, fp16 s @34).
 struct XQ {
   uint32_t lo[4], hi[4];   // 16 int8 of sub-block 2g and of sub-block 2g+1
-  float d8c, s8c;          // d and s of sub-block c (for the lane's share of scales / mins)
+  float d8c, s8c;          // d and s of sub-block c (the sub-block this lane folds)
 };
 
 __device__ __forceinline__ void load_xq(XQ& x, const uint8_t* __restrict__ xq, int blk, int c, bool active) {
@@ -84,16 +84,17 @@ __device__ __forceinline__ void load_xq(XQ& x, const uint8_t* __restrict__ xq, i
   x.s8c = half_to_f32((uint16_t)(ds >> 16));
 }
 
-// One slot's contribution to a row (double); I0/I1 are the exact int32
-// half-sub-block dots (low / high nibbles).
+// One slot's contribution to a row (double).  I0/I1 are the exact int32 half-sub-block dots
+// (low / high nibbles).  The two lanes of a pair (c even, c odd) hold the two 16-element halves of
+// sub-blocks 2g and 2g+1: they add them up, and lane c then owns the whole sub-block c and folds
+// it with its own scale, so no scale has to travel between lanes:
+//   term = (d * d8_c) * (sc_c * I_c) - (dmin * s8_c) * m_c        every product exact in double
 __device__ __forceinline__ double slot_dot(const uint4& hdr, const uint4& q, const XQ& x, const ScaleSel& sel,
-                                          int& I0, int& I1) {
+                                          int& I0, int& I1, bool odd) {
   const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu));
   const float dmin = half_to_f32((uint16_t)(hdr.x >> 16));
   uint32_t sc, m;
   lane_scale_min(sel, hdr.y, hdr.z, hdr.w, sc, m);
-  const double fsc = (double)(d * x.d8c) * (double)sc;      // d*d8c: 11 x 11 significand bits, exact in f32
-  const double fm = (double)(dmin * x.s8c) * (double)m;
   int a = 0, b = 0;
   a = sdot4(q.x & 0x0f0f0f0fu, x.lo[0], a);
   b = sdot4((q.x >> 4) & 0x0f0f0f0fu, x.hi[0], b);
@@ -104,9 +105,36 @@ __device__ __forceinline__ double slot_dot(const uint4& hdr, const uint4& q, con
   a = sdot4(q.w & 0x0f0f0f0fu, x.lo[3], a);
   b = sdot4((q.w >> 4) & 0x0f0f0f0fu, x.hi[3], b);
   I0 = a; I1 = b;
-  const double f0 = dpp_f64<DPP_PAIR_EVEN>(fsc);   // combined scale of sub-block 2g
-  const double f1 = dpp_f64<DPP_PAIR_ODD>(fsc);    // combined scale of sub-block 2g+1
-  return fma(f0, (double)a, fma(f1, (double)b, -fm));
+  const int s0 = a + dpp_i32<DPP_QUAD_XOR1>(a);          // whole sub-block 2g
+  const int s1 = b + dpp_i32<DPP_QUAD_XOR1>(b);          // whole sub-block 2g+1
+  const int p = __mul24((int)sc, odd ? s1 : s0);         // 6 x 17 bits: exact
+  const double t = (double)(dmin * x.s8c) * (double)m;   // 11 x 11 bits exact in f32, then exact in double
+  return fma((double)(d * x.d8c), (double)p, -t);
+}
+
+// Sum of four per-lane doubles (four rows) over the 64 lanes with shared steps: after two
+// exchange-and-halve steps a lane carries one row, row(lane) = 2*(lane & 1) + ((lane >> 1) & 1),
+// and the remaining steps keep lane mod 4.  Every lane ends with the total of its row.
+__device__ __forceinline__ double wave_sum4_f64(double a0, double a1, double a2, double a3, int lane) {
+  const bool o1 = lane & 1, o2 = lane & 2;
+  // step 1 (partner lane ^ 1): even lanes keep rows 0,1 and give away rows 2,3
+  const double k0 = o1 ? a2 : a0, k1 = o1 ? a3 : a1, g0 = o1 ? a0 : a2, g1 = o1 ? a1 : a3;
+  const double b0 = k0 + dpp_f64<DPP_QUAD_XOR1>(g0), b1 = k1 + dpp_f64<DPP_QUAD_XOR1>(g1);
+  // step 2 (partner lane ^ 2): lanes with bit 1 clear keep the first of their two rows
+  const double k = o2 ? b1 : b0, g = o2 ? b0 : b1;
+  double v = k + dpp_f64<DPP_QUAD_XOR2>(g);
+  v += dpp_f64<0x124>(v);      // row_ror:4  (lane i gets lane (i+4) mod 16 of its row of 16)
+  v += dpp_f64<0x128>(v);      // row_ror:8
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+// Weights are read once: nontemporal loads keep them from displacing the activation in the caches.
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_nt;
+__device__ __forceinline__ uint4 load_w16(const uint8_t* p) {
+  const u32x4_nt t = __builtin_nontemporal_load((const u32x4_nt*)p);
+  return make_uint4(t.x, t.y, t.z, t.w);
 }
 
 enum : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_BF16_ADD = 2 };
@@ -124,8 +152,54 @@ __device__ __forceinline__ void store_out(void* __restrict__ y, const uint16_t* 
   }
 }
 
+template <int NR, int RPI>
+struct RowTile {
+  uint4 hdr[RPI][NR], q[RPI][NR];
+};
+
+template <int NR, int RPI>
+__device__ __forceinline__ void load_rows(RowTile<NR, RPI>& t, const uint8_t* __restrict__ W, int64_t row_bytes, int row0, int N,
+                                          const int (&boff)[NR], int c) {
+#pragma unroll
+  for (int i = 0; i < RPI; i++) {
+    const int row = min(row0 + i, N - 1);     // rows past the end re-read the last row; their results are dropped
+    const uint8_t* rp = W + (int64_t)row * row_bytes;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      t.hdr[i][r] = load_w16(rp + boff[r]);
+      t.q[i][r] = load_w16(rp + boff[r] + 16 + 16 * c);
+    }
+  }
+}
+
+template <int NR, int EPI, int RPI>
+__device__ __forceinline__ void fold_rows(const RowTile<NR, RPI>& t, const XQ (&x)[NR], const ScaleSel& sel, bool odd, int lane,
+                                          void* __restrict__ y, const uint16_t* __restrict__ res, int64_t ybase, int row0, int N) {
+  double acc[RPI];
+#pragma unroll
+  for (int i = 0; i < RPI; i++) {
+    acc[i] = 0.0;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      int I0, I1;
+      acc[i] += slot_dot(t.hdr[i][r], t.q[i][r], x[r], sel, I0, I1, odd);
+    }
+  }
+  if (RPI == 4) {
+    const double tot = wave_sum4_f64(acc[0], acc[1], acc[2], acc[3], lane);
+    const int row = row0 + 2 * (lane & 1) + ((lane >> 1) & 1);
+    if (lane < 4 && row < N) store_out<EPI>(y, res, ybase + row, (float)tot);
+  } else {
+#pragma unroll
+    for (int i = 0; i < RPI; i++) {
+      const float tot = (float)wave_sum_f64(acc[i]);
+      if (lane == 0 && row0 + i < N) store_out<EPI>(y, res, ybase + row0 + i, tot);
+    }
+  }
+}
+
 // NR = number of 64-slot rounds per row (K = 2048*NR when the row fills every round);
-// RPI = rows a wave keeps in flight (independent loads issued before any is consumed).
+// RPI = rows a wave handles per step (all their loads are issued before any is consumed).
 template <int NR, int EPI, int RPI>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
     const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq_all, void* __restrict__ y,
@@ -138,40 +212,116 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_kernel(
   const int c = lane & 7;
   const ScaleSel sel = make_scale_sel(c);
   const int64_t row_bytes = (int64_t)nb * 144;
+  const int64_t ybase = (int64_t)bidx * N;
+  const bool odd = c & 1;
+  const int step = nwaves * RPI;
+  int row0 = wave * RPI;
 
-  XQ x[NR];
   int boff[NR];   // byte offset of the slot's block inside a row
 #pragma unroll
   for (int r = 0; r < NR; r++) {
     const int blk = r * 8 + (lane >> 3);
-    const bool active = blk < nb;
-    load_xq(x[r], xq, blk, c, active);
-    boff[r] = (active ? blk : 0) * 144;
+    boff[r] = (blk < nb ? blk : 0) * 144;
+  }
+  RowTile<NR, RPI> t0;
+  XQ x[NR];
+#pragma unroll
+  for (int r = 0; r < NR; r++) {
+    const int blk = r * 8 + (lane >> 3);
+    load_xq(x[r], xq, blk, c, blk < nb);
   }
 
-  for (int row0 = wave * RPI; row0 < N; row0 += nwaves * RPI) {
-    uint4 hdr[RPI][NR], q[RPI][NR];
+  for (; row0 < N; row0 += step) {
+    load_rows<NR, RPI>(t0, W, row_bytes, row0, N, boff, c);
+    fold_rows<NR, EPI, RPI>(t0, x, sel, odd, lane, y, res, ybase, row0, N);
+  }
+}
+
+// ---------------------------------------------------------------- rows through LDS
+// Same lane mapping and arithmetic as above, but the weight bytes travel HBM -> registers ->
+// LDS -> registers: a step's RPI rows are contiguous in memory (RPI * NR * 72 pieces of 16 bytes),
+// so the wave fetches them with fully coalesced loads (lane l takes piece l, l + 64, ...: every
+// 128-byte line is requested exactly once and no header is fetched eight times), parks them in
+// its private LDS tile and reads headers and nibble chunks back in the (block, chunk) mapping.
+// The loads of the next step are in flight while the current step is folded.
+template <int NR, int RPI>
+struct StageRegs {
+  static constexpr int PIECES = RPI * NR * 72;
+  static constexpr int LOADS = (PIECES + 63) / 64;
+  uint4 v[LOADS];
+};
+
+template <int NR, int RPI>
+__device__ __forceinline__ void stage_load(StageRegs<NR, RPI>& g, const uint8_t* __restrict__ W, int64_t tile_off,
+                                           int64_t last_piece_off, int lane) {
+#pragma unroll
+  for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
+    const int piece = lane + 64 * u;
+    if (piece < StageRegs<NR, RPI>::PIECES) {
+      const int64_t off = tile_off + (int64_t)piece * 16;
+      g.v[u] = load_w16(W + (off < last_piece_off ? off : last_piece_off));   // past the matrix: re-read its last piece
+    }
+  }
+}
+
+template <int NR, int RPI>
+__device__ __forceinline__ void stage_park(const StageRegs<NR, RPI>& g, uint4* __restrict__ tile, int lane) {
+#pragma unroll
+  for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
+    const int piece = lane + 64 * u;
+    if (piece < StageRegs<NR, RPI>::PIECES) tile[piece] = g.v[u];
+  }
+}
+
+template <int NR, int EPI, int RPI>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_lds_kernel(
+    const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq_all, void* __restrict__ y,
+    const uint16_t* __restrict__ res, int N) {
+  constexpr int PIECES = RPI * NR * 72;
+  __shared__ uint4 tiles[GEMV_WAVES][PIECES];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int wave = blockIdx.x * GEMV_WAVES + wv;
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int bidx = blockIdx.y;
+  constexpr int nb = NR * 8;
+  const uint8_t* xq = xq_all + (int64_t)bidx * nb * 8 * 36;
+  const int c = lane & 7, b = lane >> 3;
+  const ScaleSel sel = make_scale_sel(c);
+  constexpr int64_t row_bytes = (int64_t)nb * 144;
+  const int64_t last_piece_off = (int64_t)N * row_bytes - 16;
+  const int64_t ybase = (int64_t)bidx * N;
+  const bool odd = c & 1;
+  const int step = nwaves * RPI;
+  int row0 = wave * RPI;
+  uint4* tile = tiles[wv];
+
+  StageRegs<NR, RPI> g;
+  if (row0 < N) stage_load<NR, RPI>(g, W, (int64_t)row0 * row_bytes, last_piece_off, lane);
+
+  XQ x[NR];
+#pragma unroll
+  for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, true);
+
+  while (row0 < N) {
+    stage_park<NR, RPI>(g, tile, lane);
+    if (row0 + step < N) stage_load<NR, RPI>(g, W, (int64_t)(row0 + step) * row_bytes, last_piece_off, lane);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    RowTile<NR, RPI> t;
 #pragma unroll
     for (int i = 0; i < RPI; i++) {
-      const int row = min(row0 + i, N - 1);
-      const uint8_t* rp = W + (int64_t)row * row_bytes;
 #pragma unroll
       for (int r = 0; r < NR; r++) {
-        hdr[i][r] = *(const uint4*)(rp + boff[r]);
-        q[i][r] = *(const uint4*)(rp + boff[r] + 16 + 16 * c);
+        const int blk = (i * NR + r) * 72 + b * 9;       // piece index of the block header
+        t.hdr[i][r] = tile[blk];
+        t.q[i][r] = tile[blk + 1 + c];
       }
     }
-#pragma unroll
-    for (int i = 0; i < RPI; i++) {
-      double acc = 0.0;
-#pragma unroll
-      for (int r = 0; r < NR; r++) {
-        int I0, I1;
-        acc += slot_dot(hdr[i][r], q[i][r], x[r], sel, I0, I1);
-      }
-      const float tot = (float)wave_sum_f64(acc);
-      if (lane == 0 && row0 + i < N) store_out<EPI>(y, res, (int64_t)bidx * N + row0 + i, tot);
-    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                     // every lane has read its pieces before the tile is overwritten
+    fold_rows<NR, EPI, RPI>(t, x, sel, odd, lane, y, res, ybase, row0, N);
+    row0 += step;
   }
 }
 
@@ -202,7 +352,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_generic_kernel(
       const uint4 hdr = *(const uint4*)(rp + bo);
       const uint4 q = *(const uint4*)(rp + bo + 16 + 16 * c);
       int I0, I1;
-      acc += slot_dot(hdr, q, x, sel, I0, I1);
+      acc += slot_dot(hdr, q, x, sel, I0, I1, c & 1);
     }
     const float tot = (float)wave_sum_f64(acc);
     if (lane == 0) store_out<EPI>(y, res, (int64_t)bidx * N + row, tot);
@@ -231,7 +381,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
       const uint4 hdr = *(const uint4*)(rp + bo);
       const uint4 q = *(const uint4*)(rp + bo + 16 + 16 * c);
       int I0, I1;
-      (void)slot_dot(hdr, q, x, sel, I0, I1);
+      (void)slot_dot(hdr, q, x, sel, I0, I1, c & 1);
       const int s0 = I0 + dpp_i32<DPP_QUAD_XOR1>(I0);
       const int s1 = I1 + dpp_i32<DPP_QUAD_XOR1>(I1);
       if (active) I[(int64_t)row * nb * 8 + blk * 8 + c] = (c & 1) ? s1 : s0;
@@ -239,8 +389,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
   }
 }
 
-int g_tune_gemv_impl = 0;               // 1: eight-rows-per-wave layout (gemv8.hip), 0: one row per wave round
-int g_tune_rpi = 4, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows in flight per wave, workgroups per CU
+int g_tune_gemv_impl = 2;               // 2: rows staged through LDS when K is a multiple of 2048 (else as 0), 1: eight-rows-per-wave
+                                        // layout (gemv8.hip), 0: direct loads in the (block, chunk) mapping
+int g_tune_rpi = 4, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows per wave step, workgroups per CU
 
 static int gemv_grid(int N, int rows_per_wg) {
   int wgs = (N + rows_per_wg - 1) / rows_per_wg;
@@ -254,8 +405,15 @@ static void launch_q8_1_rpi(dim3 block, const uint8_t* w, const uint8_t* x, void
   dim3 grid(gemv_grid(N, GEMV_WAVES * rpi), batch);
   if (rpi == 1) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 1>), grid, block, 0, stream(), w, x, y, r, N, nb);
   else if (rpi == 2) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 2>), grid, block, 0, stream(), w, x, y, r, N, nb);
-  else if (rpi == 8 && NR == 1) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, (NR == 1 ? 8 : 4)>), grid, block, 0, stream(), w, x, y, r, N, nb);
   else { grid.x = gemv_grid(N, GEMV_WAVES * 4); hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 4>), grid, block, 0, stream(), w, x, y, r, N, nb); }
+}
+
+template <int NR, int EPI>
+static void launch_q8_1_lds(dim3 block, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int batch) {
+  const int rpi = NR == 1 ? (g_tune_rpi == 2 ? 2 : 4) : 2;
+  dim3 grid(gemv_grid(N, GEMV_WAVES * rpi), batch);
+  if (NR == 1 && rpi == 4) hipLaunchKernelGGL((gemv_q4k_q8_1_lds_kernel<NR, EPI, (NR == 1 ? 4 : 2)>), grid, block, 0, stream(), w, x, y, r, N);
+  else hipLaunchKernelGGL((gemv_q4k_q8_1_lds_kernel<NR, EPI, 2>), grid, block, 0, stream(), w, x, y, r, N);
 }
 
 template <int EPI>
@@ -265,9 +423,12 @@ static void launch_q8_1_variant(const void* W, const void* xq, void* y, const vo
   dim3 grid(1, batch);
   const uint8_t* w = (const uint8_t*)W; const uint8_t* x = (const uint8_t*)xq; const uint16_t* r = (const uint16_t*)res;
   switch (rounds) {
-    case 1: launch_q8_1_rpi<1, EPI>(block, w, x, y, r, N, nb, batch); break;
-    case 2: launch_q8_1_rpi<2, EPI>(block, w, x, y, r, N, nb, batch); break;
-    case 3: launch_q8_1_rpi<3, EPI>(block, w, x, y, r, N, nb, batch); break;
+    case 1: if (g_tune_gemv_impl == 2 && nb == 8) launch_q8_1_lds<1, EPI>(block, w, x, y, r, N, batch); else launch_q8_1_rpi<1, EPI>(block, w, x, y, r, N, nb, batch);
+      break;
+    case 2: if (g_tune_gemv_impl == 2 && nb == 16) launch_q8_1_lds<2, EPI>(block, w, x, y, r, N, batch); else launch_q8_1_rpi<2, EPI>(block, w, x, y, r, N, nb, batch);
+      break;
+    case 3: if (g_tune_gemv_impl == 2 && nb == 24) launch_q8_1_lds<3, EPI>(block, w, x, y, r, N, batch); else launch_q8_1_rpi<3, EPI>(block, w, x, y, r, N, nb, batch);
+      break;
     default:
       grid.x = gemv_grid(N, GEMV_WAVES);
       hipLaunchKernelGGL((gemv_q4k_q8_1_generic_kernel<EPI>), grid, block, 0, stream(), w, x, y, r, N, nb);
