@@ -89,6 +89,71 @@ static int run_gemm(Kernel& k, const uint64_t* s) {
   return matmul_q8_1(P<void>(s[1]), k.scratch, P<void>(s[2]), N, K, batch, (int)k.get("cast", 0), nullptr, (int)k.get("mfma", -1));
 }
 
+// ---- op: gemv_fused — rmsnorm / quantize + up to four matmuls over one activation + their cast / add / swiglu
+// consumers (src/model.ts:65-73, 161-191 as one launch; the node-by-node result to the bit).
+// params: K, pro (0: x is Q8_1, 1: x is bf16, 2: x is bf16 and goes through rmsnorm with norm_w first),
+//         G matrices with N<i>, epi<i> (0: f32, 1: bf16, 2: bf16(bf16(y) + residual)), swiglu=0|1 (G=2: gate, up), batch=1
+// slots:  x, [norm_w if pro=2], then per matrix: W, [residual if epi=2], out      (swiglu: x, [norm_w], Wg, Wu, out)
+// Shapes outside the fused kernel (K not 2048/4096/6144, batch >= 8) run as rmsnorm/quantize, matmuls, swiglu.
+static int run_gemv_fused(Kernel& k, const uint64_t* s) {
+  const int K = (int)k.get("K", 0), pro = (int)k.get("pro", 0), G = (int)k.get("G", 1), batch = (int)k.get("batch", 1);
+  const bool swiglu = k.get("swiglu", 0) != 0;
+  int si = 0;
+  const void* x = P<void>(s[si++]);
+  const void* nw = pro == 2 ? P<void>(s[si++]) : nullptr;
+  const void* W[4] = {}; void* out[4] = {}; const void* res[4] = {}; int N[4] = {}, epi[4] = {};
+  char key[16];
+  for (int i = 0; i < G; i++) {
+    snprintf(key, sizeof key, "N%d", i); N[i] = (int)k.get(key, 0);
+    snprintf(key, sizeof key, "epi%d", i); epi[i] = (int)k.get(key, 0);
+    W[i] = P<void>(s[si++]);
+    if (swiglu) continue;
+    if (epi[i] == 2) res[i] = P<void>(s[si++]);
+    out[i] = P<void>(s[si++]);
+  }
+  if (swiglu) out[0] = P<void>(s[si++]);
+  if (gemv_fused_fast_path(K, batch, swiglu)) return launch_gemv_fused(pro, x, nw, K, batch, G, W, out, res, N, epi, swiglu);
+  int rc;
+  const void* xq = x;
+  if (pro == 2) { if ((rc = launch_rmsnorm(x, nw, nullptr, k.scratch, K, batch))) return rc; xq = k.scratch; }
+  else if (pro == 1) { if ((rc = launch_quantize_q8_1(x, DT_BF16, k.scratch, K, batch))) return rc; xq = k.scratch; }
+  if (swiglu) {
+    float* g = (float*)((uint8_t*)k.scratch + (size_t)batch * (K / 32) * 36);
+    float* u = g + (size_t)batch * N[0];
+    if ((rc = matmul_q8_1(W[0], xq, g, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
+    if ((rc = matmul_q8_1(W[1], xq, u, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
+    return launch_elementwise(EW_SWIGLU_OP, g, u, out[0], (int64_t)batch * N[0]);
+  }
+  for (int i = 0; i < G; i++)
+    if ((rc = matmul_q8_1(W[i], xq, out[i], N[i], K, batch, epi[i] == 0 ? DT_F32 : DT_BF16, res[i], -1))) return rc;
+  return BK_OK;
+}
+static int build_gemv_fused(Kernel& k) {
+  int rc;
+  if ((rc = need(k, "K")) || (rc = need(k, "N0"))) return rc;
+  const int64_t K = k.get("K", 0), pro = k.get("pro", 0), G = k.get("G", 1), batch = k.get("batch", 1);
+  const bool swiglu = k.get("swiglu", 0) != 0;
+  BK_REQUIRE(K > 0 && K % 256 == 0, "gemv_fused: K=%lld must be a positive multiple of 256", (long long)K);
+  BK_REQUIRE(pro >= 0 && pro <= 2 && G >= 1 && G <= 4 && batch >= 1 && batch <= 4096, "gemv_fused: bad pro/G/batch");
+  BK_REQUIRE(!swiglu || G == 2, "gemv_fused: swiglu needs G=2 (gate, up)");
+  int nslots = 1 + (pro == 2 ? 1 : 0);
+  char key[16];
+  for (int i = 0; i < G; i++) {
+    snprintf(key, sizeof key, "N%d", i);
+    BK_REQUIRE(k.get(key, 0) > 0, "gemv_fused: missing or bad %s", key);
+    BK_REQUIRE(!swiglu || k.get(key, 0) == k.get("N0", 0), "gemv_fused: gate and up must have the same N");
+    BK_REQUIRE(!swiglu || k.get(key, 0) % 4 == 0, "gemv_fused: swiglu needs N to be a multiple of 4");
+    snprintf(key, sizeof key, "epi%d", i);
+    const int64_t e = k.get(key, 0);
+    BK_REQUIRE(e >= 0 && e <= 2, "gemv_fused: bad %s", key);
+    nslots += swiglu ? 1 : (e == 2 ? 3 : 2);
+  }
+  if (swiglu) nslots += 1;
+  if ((rc = alloc_scratch(k, (size_t)(batch * (K / 32) * 36) + (swiglu ? (size_t)(2 * batch * k.get("N0", 0) * 4) : 0)))) return rc;
+  k.run = run_gemv_fused; k.nslots = nslots;
+  return BK_OK;
+}
+
 // ---- op: embed (src/model.ts:53-56)   slots: embed.weight, token_id, out
 // params: H, VOCAB, batch=1, ids_dev=0 (1: slot 1 is a device pointer to int32 [batch])
 static int run_embed(Kernel& k, const uint64_t* s) {
@@ -216,6 +281,7 @@ static int build_kernel(Kernel& k) {
     k.run = run_argmax; k.nslots = 3;
     return BK_OK;
   }
+  if (k.op == "gemv_fused") return build_gemv_fused(k);
   if (k.op == "quantize_q8_1") {
     if ((rc = need(k, "K"))) return rc;
     k.run = run_quantize; k.nslots = 2;

@@ -152,5 +152,48 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
   return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 
+// Q8_1 of one 32-element block held by four consecutive lanes (8 values each, already rounded to
+// the activation's storage type).  bench/bench.ts:53-72: d = amax/127 and the quotient in double,
+// round half toward +infinity, s = trunc16(float(sum(q) * d)) with the unrounded d.  Returns the
+// lane's 8 int8 in pk[0..1] and the packed (d, s) halves, the same in all four lanes.
+__device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk)[2]) {
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(f[j]));
+  amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
+  amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
+  const double d = (double)amax / 127.0, div = d != 0.0 ? d : 1.0;
+  int sum = 0;
+  pk[0] = 0; pk[1] = 0;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const double qd = (double)f[j] / div;
+    double r = floor(qd);
+    if (qd - r >= 0.5) r += 1.0;
+    int q = (int)r;
+    sum += q;
+    q = q < -128 ? -128 : (q > 127 ? 127 : q);
+    pk[j >> 2] |= (uint32_t)(q & 0xff) << (8 * (j & 3));
+  }
+  sum += dpp_i32<DPP_QUAD_XOR1>(sum);
+  sum += dpp_i32<DPP_QUAD_XOR2>(sum);
+  return (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);
+}
+
+// Block-wide sum in double for blockDim.x = 64 * NW; every thread gets the total.
+template <int NW>
+__device__ __forceinline__ double block_sum_f64(double v, double* lds) {
+  v = wave_sum_f64(v);
+  if (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) lds[w] = v;
+  __syncthreads();
+  double t = 0.0;
+#pragma unroll
+  for (int i = 0; i < NW; i++) t += lds[i];
+  __syncthreads();
+  return t;
+}
+
 #endif  // __HIPCC__
 }  // namespace bk

@@ -1,0 +1,275 @@
+// Q4_K x Q8_1 GEMV with the surrounding glue folded in: one launch serves
+//   [RMSNorm | bf16 -> Q8_1 | Q8_1 as given]  ->  up to four matrices over the same activation
+//   ->  per matrix: f32 | bf16 | bf16(bf16(y) + residual)      or, for a (gate, up) pair, SwiGLU.
+//
+// Prologue.  Every workgroup prepares the activation row itself: 256 threads x 8 elements per
+// pass, the sum of squares in double through the same block reduction as the stand-alone
+// RMSNorm kernel, the Q8_1 blocks by groups of four lanes.  The quantized row lives in LDS in
+// the Q8_1 byte layout; each lane then takes its slice into registers as the plain GEMV does.
+// The first weight loads are requested before the prologue, so its latency hides behind them.
+//
+// Rows.  As in the LDS-staged GEMV: a wave step fetches RPI contiguous rows with coalesced
+// 16-byte loads, parks them in the wave's LDS tile and reads them back in the (block, chunk)
+// mapping.  The matrices of a launch are laid end to end in "step" space; a step belongs to
+// exactly one matrix.  For SwiGLU a step holds RPI/2 rows of the gate matrix and the same rows
+// of the up matrix, so that the lanes that end up with g and u of one output row are neighbours.
+//
+// Arithmetic is that of gemv.hip and glue.hip, operation for operation, so a fused launch gives
+// the bits of the node-by-node sequence rmsnorm -> gemm [-> cast -> add | -> swiglu].
+#include "gemv_tile.h"
+
+namespace bk {
+
+enum : int { PRO_Q8 = 0, PRO_BF16 = 1, PRO_RMSNORM = 2 };
+
+struct FusedGroup {
+  const uint8_t* W;
+  void* out;
+  const uint16_t* res;
+  int N, epi;
+};
+struct FusedArgs {
+  FusedGroup g[4];
+  int step_first[5];     // first step of each matrix; step_first[i >= ngroups] = total steps
+  int ngroups;
+  const void* x;         // PRO_Q8: Q8_1 [batch, K/32 blocks]; else bf16 [batch, K]
+  const uint16_t* norm_w;
+};
+
+// What a step needs to know about its matrix (all wave-uniform).
+struct StepSel {
+  const uint8_t* W;
+  void* out;
+  const uint16_t* res;
+  int N, epi, row0;
+};
+
+template <int ROWS_PER_STEP>
+__device__ __forceinline__ StepSel select_step(const FusedArgs& A, int s) {
+  const bool s1 = s >= A.step_first[1], s2 = s >= A.step_first[2], s3 = s >= A.step_first[3];
+  StepSel r;
+  r.W = s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
+  r.out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
+  r.res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
+  r.N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
+  r.epi = s3 ? A.g[3].epi : s2 ? A.g[2].epi : s1 ? A.g[1].epi : A.g[0].epi;
+  r.row0 = (s - (s3 ? A.step_first[3] : s2 ? A.step_first[2] : s1 ? A.step_first[1] : 0)) * ROWS_PER_STEP;
+  return r;
+}
+
+// ---- prologue: activation row -> Q8_1 in LDS (36-byte blocks)
+template <int PRO>
+__device__ __forceinline__ void stage_activation(const uint16_t* __restrict__ xr, const uint16_t* __restrict__ w, int K,
+                                                 uint8_t* lds_xq, double* lds_red) {
+  float rstd = 0.0f;
+  if (PRO == PRO_RMSNORM) {
+    double ss = 0.0;
+    for (int i = threadIdx.x * 8; i < K; i += 256 * 8) {
+      const uint4 v = *(const uint4*)(xr + i);
+      const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
+        ss += (double)(a * a) + (double)(b * b);
+      }
+    }
+    ss = block_sum_f64<4>(ss, lds_red);
+    rstd = rsqrt_f64(ss / (double)K + 1e-6);
+  }
+  for (int i = threadIdx.x * 8; i < K; i += 256 * 8) {
+    const uint4 v = *(const uint4*)(xr + i);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+    if (PRO == PRO_RMSNORM) {
+      const uint4 wv = *(const uint4*)(w + i);
+      const uint32_t uw[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
+        const float wa = __uint_as_float(uw[j] << 16), wb = __uint_as_float(uw[j] & 0xffff0000u);
+        f[2 * j] = bf16_to_f32(f32_to_bf16(__fmul_rn(__fmul_rn(a, rstd), __fadd_rn(1.0f, wa))));
+        f[2 * j + 1] = bf16_to_f32(f32_to_bf16(__fmul_rn(__fmul_rn(b, rstd), __fadd_rn(1.0f, wb))));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        f[2 * j] = __uint_as_float(u[j] << 16);
+        f[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+      }
+    }
+    uint32_t pk[2];
+    const uint32_t ds = quad_q8_1(f, pk);
+    uint8_t* ob = lds_xq + (i / 32) * 36;
+    uint32_t* oq = (uint32_t*)(ob + (i & 31));
+    oq[0] = pk[0]; oq[1] = pk[1];
+    if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+  }
+  __syncthreads();
+}
+
+// ---- weight rows of one step: coalesced 16-byte pieces; with SWIGLU the second half of the tile
+// comes from the up matrix (same rows)
+template <int NR, int RPI, bool SWIGLU>
+__device__ __forceinline__ void fused_stage_load(StageRegs<NR, RPI>& g, const uint8_t* __restrict__ W0,
+                                                 const uint8_t* __restrict__ W1, int row0, int N, int lane) {
+  constexpr int PIECES = StageRegs<NR, RPI>::PIECES;
+  constexpr int64_t row_bytes = (int64_t)NR * 8 * 144;
+  const int64_t last = (int64_t)N * row_bytes - 16;
+  const int64_t base = (int64_t)row0 * row_bytes;
+#pragma unroll
+  for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
+    const int piece = lane + 64 * u;
+    if (piece < PIECES) {
+      const bool second = SWIGLU && piece >= PIECES / 2;
+      const int64_t off = base + (int64_t)(second ? piece - PIECES / 2 : piece) * 16;
+      const uint8_t* W = second ? W1 : W0;
+      g.v[u] = load_w16(W + (off < last ? off : last));     // past the matrix: re-read its last piece
+    }
+  }
+}
+
+template <int NR, int RPI, int PRO, bool SWIGLU>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A) {
+  constexpr int PIECES = RPI * NR * 72;
+  constexpr int K = NR * 2048;
+  constexpr int ROWS_PER_STEP = SWIGLU ? RPI / 2 : RPI;
+  __shared__ uint4 tiles[GEMV_WAVES][PIECES];
+  __shared__ __align__(16) uint8_t lds_xq[PRO == PRO_Q8 ? 16 : (K / 32) * 36];
+  __shared__ double lds_red[4];
+
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int bidx = blockIdx.y;
+  const int c = lane & 7, b = lane >> 3;
+  const ScaleSel sel = make_scale_sel(c);
+  const bool odd = c & 1;
+  const int total = A.step_first[4];
+  uint4* tile = tiles[wv];
+
+  int s = blockIdx.x * GEMV_WAVES + wv;
+  StepSel cur = select_step<ROWS_PER_STEP>(A, s < total ? s : 0);
+  StageRegs<NR, RPI> g;
+  if (s < total) fused_stage_load<NR, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
+
+  XQ x[NR];
+  if (PRO == PRO_Q8) {
+    const uint8_t* xq = (const uint8_t*)A.x + (int64_t)bidx * (K / 32) * 36;
+#pragma unroll
+    for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, true);
+  } else {
+    stage_activation<PRO>((const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w, K, lds_xq, lds_red);
+#pragma unroll
+    for (int r = 0; r < NR; r++) load_xq(x[r], lds_xq, r * 8 + b, c, true);
+  }
+
+  while (s < total) {
+    stage_park<NR, RPI>(g, tile, lane);
+    const int sn = s + nwaves;
+    StepSel nxt = cur;
+    if (sn < total) {
+      nxt = select_step<ROWS_PER_STEP>(A, sn);
+      fused_stage_load<NR, RPI, SWIGLU>(g, nxt.W, A.g[1].W, nxt.row0, nxt.N, lane);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    RowTile<NR, RPI> t;
+#pragma unroll
+    for (int i = 0; i < RPI; i++) {
+#pragma unroll
+      for (int r = 0; r < NR; r++) {
+        const int blk = (i * NR + r) * 72 + b * 9;
+        t.hdr[i][r] = tile[blk];
+        t.q[i][r] = tile[blk + 1 + c];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();       // every lane has read its pieces before the tile is overwritten
+
+    const double tot = fold_rows_total<NR, RPI>(t, x, sel, odd, lane);
+    const int rl = RPI == 4 ? 2 * (lane & 1) + ((lane >> 1) & 1) : (lane & 1);     // tile row this lane holds
+    const float v = (float)tot;
+    if (SWIGLU) {
+      // tile rows: gate row0, gate row0+1, up row0, up row0+1 -> lanes 0..3 hold g0, u0, g1, u1
+      const float other = dpp_f32<DPP_QUAD_XOR1>(v);
+      const int row = cur.row0 + (lane >> 1);
+      if (lane < 4 && !(lane & 1) && row < cur.N) {
+        // src/fusion.ts:324-330: bf16((g * sigmoid(g)) * u)
+        ((uint16_t*)cur.out)[(int64_t)bidx * cur.N + row] = f32_to_bf16(__fmul_rn(__fmul_rn(v, sigmoid_f64(v)), other));
+      }
+    } else {
+      const int row = cur.row0 + rl;
+      if (lane < RPI && row < cur.N) {
+        const int64_t o = (int64_t)bidx * cur.N + row;
+        if (cur.epi == EPI_F32) store_out<EPI_F32>(cur.out, cur.res, o, v);
+        else if (cur.epi == EPI_BF16) store_out<EPI_BF16>(cur.out, cur.res, o, v);
+        else store_out<EPI_BF16_ADD>(cur.out, cur.res, o, v);
+      }
+    }
+    s = sn;
+    cur = nxt;
+  }
+}
+
+bool gemv_fused_fast_path(int K, int batch, bool swiglu) {
+  if (K <= 0 || K % 2048 != 0 || K > 6144) return false;
+  if (swiglu && K != 2048) return false;
+  return batch >= 1 && batch < 8;
+}
+
+template <int NR, int RPI, bool SWIGLU>
+static void launch_fused_pro(int pro, dim3 grid, const FusedArgs& A) {
+  const dim3 block(GEMV_WAVES * 64);
+  if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_Q8, SWIGLU>), grid, block, 0, stream(), A);
+  else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_BF16, SWIGLU>), grid, block, 0, stream(), A);
+  else hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
+}
+
+// Fast path only (gemv_fused_fast_path says whether it applies); the caller composes the same
+// result from separate kernels otherwise.
+int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
+                      void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu) {
+  BK_REQUIRE(pro == PRO_Q8 || pro == PRO_BF16 || pro == PRO_RMSNORM, "gemv_fused: bad prologue %d", pro);
+  BK_REQUIRE(x && (pro != PRO_RMSNORM || norm_w), "gemv_fused: null activation or norm weight");
+  BK_REQUIRE(gemv_fused_fast_path(K, batch, swiglu), "gemv_fused: K=%d batch=%d is outside the fused kernel's shapes", K, batch);
+  BK_REQUIRE(ngroups >= 1 && ngroups <= 4 && (!swiglu || ngroups == 2), "gemv_fused: bad number of matrices %d", ngroups);
+  BK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemv_fused: activation and norm weight must be 16-byte aligned");
+  const int NR = K / 2048, RPI = NR == 1 ? 4 : 2;
+  const int rows_per_step = swiglu ? RPI / 2 : RPI;
+  FusedArgs A{};
+  A.ngroups = ngroups; A.x = x; A.norm_w = (const uint16_t*)norm_w;
+  int steps = 0;
+  for (int i = 0; i < ngroups; i++) {
+    BK_REQUIRE(W[i] && N[i] > 0 && ((uintptr_t)W[i] & 15) == 0, "gemv_fused: matrix %d: null, misaligned or N <= 0", i);
+    A.g[i].W = (const uint8_t*)W[i];
+    A.g[i].N = N[i];
+    if (swiglu) {
+      BK_REQUIRE(N[i] == N[0], "gemv_fused: gate and up must have the same number of rows");
+      A.g[i].out = out[0]; A.g[i].res = nullptr; A.g[i].epi = EPI_BF16;
+      A.step_first[i] = 0;
+      if (i == 0) { BK_REQUIRE(out[0], "gemv_fused: null output"); steps = (N[0] + rows_per_step - 1) / rows_per_step; }
+    } else {
+      BK_REQUIRE(out[i], "gemv_fused: matrix %d: null output", i);
+      BK_REQUIRE(epi[i] == EPI_F32 || epi[i] == EPI_BF16 || epi[i] == EPI_BF16_ADD, "gemv_fused: bad epilogue %d", epi[i]);
+      BK_REQUIRE(epi[i] != EPI_BF16_ADD || res[i], "gemv_fused: the add epilogue needs a residual");
+      A.g[i].out = out[i]; A.g[i].res = (const uint16_t*)res[i]; A.g[i].epi = epi[i];
+      A.step_first[i] = steps;
+      steps += (N[i] + rows_per_step - 1) / rows_per_step;
+    }
+  }
+  for (int i = swiglu ? 1 : ngroups; i < 5; i++) A.step_first[i] = steps;
+  if (swiglu) A.step_first[0] = 0;
+  int wgs = (steps + GEMV_WAVES - 1) / GEMV_WAVES;
+  const int cap = num_cus() * g_tune_cap;
+  if (wgs > cap) wgs = cap;
+  const dim3 grid(wgs, batch);
+  if (swiglu) launch_fused_pro<1, 4, true>(pro, grid, A);
+  else if (NR == 1) launch_fused_pro<1, 4, false>(pro, grid, A);
+  else if (NR == 2) launch_fused_pro<2, 2, false>(pro, grid, A);
+  else launch_fused_pro<3, 2, false>(pro, grid, A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

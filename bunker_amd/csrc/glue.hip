@@ -6,21 +6,6 @@
 
 namespace bk {
 
-// Block-wide sum in double for blockDim.x = 64 * NW; every thread gets the total.
-template <int NW>
-__device__ __forceinline__ double block_sum_f64(double v, double* lds) {
-  v = wave_sum_f64(v);
-  if (NW == 1) return v;
-  const int w = threadIdx.x >> 6;
-  if ((threadIdx.x & 63) == 0) lds[w] = v;
-  __syncthreads();
-  double t = 0.0;
-#pragma unroll
-  for (int i = 0; i < NW; i++) t += lds[i];
-  __syncthreads();
-  return t;
-}
-
 // ---------------------------------------------------------------- embed
 // src/emitters.ts:31-45: X[b, 0:H] = E[id[b], :] (bf16 row copy).  The id is a scalar
 // argument (batch 1, as the reference passes it) or comes from an int32 device array.
@@ -84,31 +69,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     if (out) *(uint4*)(out + (int64_t)row * N + i) = make_uint4(o[0], o[1], o[2], o[3]);
     if (QUANT) {
       // Q8_1 of the bf16-rounded values: block = 4 consecutive lanes x 8 elements
-      float amax = 0.0f;
-#pragma unroll
-      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(f[j]));
-      amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
-      amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
-      const double d = (double)amax / 127.0, div = d != 0.0 ? d : 1.0;
-      int sum = 0;
-      uint32_t pk[2] = {0, 0};
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const double qd = (double)f[j] / div;
-        double r = floor(qd);
-        if (qd - r >= 0.5) r += 1.0;
-        int q = (int)r;
-        sum += q;
-        q = q < -128 ? -128 : (q > 127 ? 127 : q);
-        pk[j >> 2] |= (uint32_t)(q & 0xff) << (8 * (j & 3));
-      }
-      sum += dpp_i32<DPP_QUAD_XOR1>(sum);
-      sum += dpp_i32<DPP_QUAD_XOR2>(sum);
+      uint32_t pk[2];
+      const uint32_t ds = quad_q8_1(f, pk);
       uint8_t* ob = xq + ((int64_t)row * (N / 32) + i / 32) * 36;
       uint32_t* oq = (uint32_t*)(ob + (i & 31));
       oq[0] = pk[0]; oq[1] = pk[1];
-      if ((i & 31) == 0)
-        *(uint32_t*)(ob + 32) = (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);
+      if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
     }
   }
 }
