@@ -68,7 +68,7 @@ def cpu_baseline(seconds_target=12.0):
                       f"{dt:.1f} s on {threads} OpenMP threads of the host CPU"}
 
 
-def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16):
+def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16, fused=True):
     """tok/s of the full synthetic decode step at batch 1 and 32 (device-resident loop, HIP graph replay)."""
     from bunker_amd import model, runner, synth_model
 
@@ -86,7 +86,8 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16):
         dev_w = dev_w or env.weight_ptrs()
         starts = [(9419 + 4099 * i) % D.VOCAB for i in range(B)]
         warm = 3
-        loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph)
+        loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph,
+                                 partition=runner.fusedPartition(g) if fused else None)
         loop.step(warm)
         rt.cuSync()
         e0, e1 = rt.Event(), rt.Event()
@@ -105,7 +106,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16):
         floor_us = (weight_bytes + state_bytes) / 8e12 * 1e6
         out[f"bs{B}"] = {"tok_per_s": round(B / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
                          "wall_ms_per_step": round(wall * 1e3 / steps, 4), "steps": steps,
-                         "launch": "hip graph replay" if use_graph else "eager", "kernels_per_step": len(loop.launches), "step_bytes": weight_bytes + state_bytes,
+                         "launch": "hip graph replay" if use_graph else "eager", "launches_per_step": len(loop.launches), "partition": "fused" if fused else "node per kernel", "step_bytes": weight_bytes + state_bytes,
                          "hbm_floor_us": round(floor_us, 1), "frac_of_floor": round(floor_us / (ms * 1e3), 4),
                          "first_tokens": toks[:4, 0].tolist()}
     for env in envs:
@@ -200,6 +201,7 @@ def main():
     ap.add_argument("--mode", choices=["graph", "stream"], default="stream",
                     help="GEMV section. stream: K individual launches per shape, queued back to back; "
                          "graph: the K launches replayed from one HIP graph")
+    ap.add_argument("--unfused", action="store_true", help="decode section: one kernel per graph node (the reference's partition)")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode and kernels sections launch eagerly instead of replaying HIP graphs "
                          "(rocprofv3 cannot trace graph launches on this ROCm)")
@@ -310,7 +312,7 @@ def main():
             rt.cuFree(p)
     sections = set(args.sections.split(","))
     if "decode" in sections:
-        out["decode"] = bench_decode(rt, synth, use_graph=not args.no_graph)
+        out["decode"] = bench_decode(rt, synth, use_graph=not args.no_graph, fused=not args.unfused)
     if "kernels" in sections:
         out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
     if not args.no_cpu_baseline:

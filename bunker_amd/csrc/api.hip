@@ -190,6 +190,14 @@ static int run_gdn(Kernel& k, const uint64_t* s) {
   return launch_gdn_fused(P<void>(s[0]), P<void>(s[1]), P<float>(s[2]), P<void>(s[3]), P<float>(s[4]), P<float>(s[5]),
                           P<float>(s[6]), P<float>(s[7]), P<void>(s[8]), P<float>(s[9]), (int)k.get("LVH", 0), (int)k.get("batch", 1));
 }
+// ---- op: gdn_conv = conv1d_decode + gdn_delta_rule in one launch (the conv output never reaches memory)
+// slots: qkv, conv_state_in, conv_w, z, A_log, dt_bias, a_p, b_p, norm_w, s_state_in, out, conv_state_new, s_state_new
+// params: LVH (= number of key heads), batch=1
+static int run_gdn_conv(Kernel& k, const uint64_t* s) {
+  return launch_gdn_conv_fused(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<float>(s[4]), P<void>(s[5]),
+                               P<float>(s[6]), P<float>(s[7]), P<float>(s[8]), P<float>(s[9]), P<void>(s[10]), P<void>(s[11]),
+                               P<float>(s[12]), (int)k.get("LVH", 0), (int)k.get("batch", 1));
+}
 // ---- ops: qnorm (q-gate buffer, w, out; NH heads, input rows 2*HD apart), knorm (k, w, out; NKV heads)
 static int run_qnorm(Kernel& k, const uint64_t* s) {
   const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0);
@@ -228,6 +236,25 @@ static int run_fa2(Kernel& k, const uint64_t* s) {
                             P<uint16_t>(s[3]) + HD, (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[7]), nullptr, k.scratch, k.scratch_bytes,
                             batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
 }
+// ---- op: fa2_fused = qnorm, rope, knorm, ropek, fa2_attn of src/model.ts:126-157 as three launches
+// (norm + rotation + cache append; split attention; merge with the output gate).
+// slots: qgate (q_proj output, [q | gate] per head), k, v, q_norm.weight, k_norm.weight, rope_cos, rope_sin, pos,
+//        kv_k, kv_v, out         params: HD, NH, NKV, MAX_LEN, ROT_HALF, batch=1, pos_dev=0
+static int run_fa2_fused(Kernel& k, const uint64_t* s) {
+  const bool dev = k.get("pos_dev", 0) != 0;
+  const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0), NKV = (int)k.get("NKV", 0), batch = (int)k.get("batch", 1);
+  const int max_len = (int)k.get("MAX_LEN", 0), bt_stride = (max_len + 15) / 16, half = (int)k.get("ROT_HALF", 0);
+  const int32_t* pos_dev = dev ? P<int32_t>(s[7]) : nullptr;
+  const int pos = dev ? 0 : (int)(int32_t)s[7];
+  void* qn = k.scratch;                                              // bf16 [batch, NH, HD]
+  void* ws = (uint8_t*)k.scratch + (size_t)batch * NH * HD * 2;
+  int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
+                            pos_dev, pos, half, max_len, qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, batch, NH, NKV, HD, 16);
+  if (rc) return rc;
+  return launch_attn_decode(qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, pos_dev, pos, 1, max_len, P<uint16_t>(s[0]) + HD,
+                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - (size_t)batch * NH * HD * 2,
+                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
+}
 // ---- op: argmax (src/model.ts:198-201)   slots: logits, val, idx     params: VOCAB, batch=1
 static int run_argmax(Kernel& k, const uint64_t* s) {
   return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
@@ -247,6 +274,7 @@ static int build_kernel(Kernel& k) {
       {"rmsnorm_q8_1", run_rmsnorm_q8, 4, "N", nullptr}, {"cast", run_cast, 2, "N", nullptr},
       {"add", run_add, 3, "N", nullptr},            {"swiglu", run_swiglu, 3, "N", nullptr},
       {"conv1d_decode", run_conv1d, 5, "QKVD", nullptr}, {"gdn_delta_rule", run_gdn, 10, "LVH", nullptr},
+      {"gdn_conv", run_gdn_conv, 13, "LVH", nullptr},
       {"qnorm", run_qnorm, 3, "HD", "NH"},          {"knorm", run_knorm, 3, "HD", "NKV"},
       {"rope", run_rope, 4, "HD", "NH"},            {"ropek", run_rope, 4, "HD", "NKV"},
       {"advance", run_advance, 6, "batch", "max_steps"},
@@ -258,7 +286,7 @@ static int build_kernel(Kernel& k) {
     if (k.op == "rope" || k.op == "ropek") {
       if ((rc = need(k, "ROT_HALF")) || (rc = need(k, "MAX_LEN"))) return rc;
     }
-    if (k.op == "gdn_delta_rule")
+    if (k.op == "gdn_delta_rule" || k.op == "gdn_conv")
       BK_REQUIRE(k.get("LKD", 128) == 128 && k.get("LVD", 128) == 128, "gdn_delta_rule: dk = dv = 128 only");
     k.run = sp.run; k.nslots = sp.nslots;
     return BK_OK;
@@ -271,6 +299,17 @@ static int build_kernel(Kernel& k) {
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
     if (splits > 1 && (rc = alloc_scratch(k, attn_workspace_bytes(batch, NKV, splits)))) return rc;
     k.run = run_fa2; k.nslots = 10;
+    return BK_OK;
+  }
+  if (k.op == "fa2_fused") {
+    if ((rc = need(k, "HD")) || (rc = need(k, "NH")) || (rc = need(k, "NKV")) || (rc = need(k, "MAX_LEN")) || (rc = need(k, "ROT_HALF"))) return rc;
+    const int batch = (int)k.get("batch", 1), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
+    BK_REQUIRE(batch >= 1 && NKV >= 1 && max_len >= 1 && k.get("NH", 0) >= 1 && k.get("HD", 0) >= 1, "fa2_fused: bad batch/NH/NKV/HD/MAX_LEN");
+    int splits = (int)k.get("splits", 0);
+    if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
+    const size_t qbytes = (size_t)batch * k.get("NH", 0) * k.get("HD", 0) * 2;
+    if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(batch, NKV, splits) : 0)))) return rc;
+    k.run = run_fa2_fused; k.nslots = 11;
     return BK_OK;
   }
   if (k.op == "argmax") {
@@ -314,6 +353,7 @@ int bk_tune_set(const char* key, int value) {
   else if (!strcmp(key, "gemv_cap")) bk::g_tune_cap = value;
   else if (!strcmp(key, "gemv_impl")) bk::g_tune_gemv_impl = value;
   else if (!strcmp(key, "gemv_ks_rows")) bk::g_tune_ks_rows = value;
+  else if (!strcmp(key, "gemm_nw")) bk::g_tune_gemm_nw = value;
   else if (!strcmp(key, "memread_unroll")) bk::g_tune_mr_unroll = value;
   else if (!strcmp(key, "memread_cap")) bk::g_tune_mr_cap = value;
   else if (!strcmp(key, "memread_nt")) bk::g_tune_mr_nt = value;

@@ -269,6 +269,86 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   return BK_OK;
 }
 
+// ---------------------------------------------------------------- per-head norm + RoPE + cache append in one launch
+// qnorm -> rope, knorm -> ropek and the cache write (src/emitters.ts:123-183, 202-205) as one kernel:
+// one wavefront per (role, head, sequence).  Query heads go to `qout` (bf16 [B, NH, 256]); the
+// normalised, rotated key goes straight into its K page and the value into its V page (dim-major),
+// so neither passes through memory a second time.  Arithmetic as in the stand-alone kernels:
+//   n[i] = bf16((x[i] * rstd) * (1 + w[i])), rstd from the sum of squares in double;
+//   pairs (i, i + half), i < half: x1' = bf16(x1*c - x2*s), x2' = bf16(x2*c + x1*s).
+struct PrepArgs {
+  const uint16_t *qg, *k, *v;      // q|gate bf16 [B, NH, 2*256]; k, v bf16 [B, NKV, 256]
+  const uint16_t *qw, *kw;         // norm weights bf16 [256]
+  const float *cos_t, *sin_t;      // f32 [max_len, half]
+  const int32_t* pos_dev; int pos_scalar;
+  uint16_t *qout, *kc, *vc;
+  const int32_t* block_table; int bt_stride;
+  int NH, NKV, half;
+};
+
+__global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs A) {
+  __shared__ uint16_t sh[ATT_HD];
+  const int role = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const int pos = A.pos_dev ? A.pos_dev[b] : A.pos_scalar;
+  const int pg = pos / ATT_PAGE, slot = pos % ATT_PAGE;
+  const bool is_q = role < A.NH, is_k = !is_q && role < A.NH + A.NKV;
+  const int kvh = is_q ? 0 : (is_k ? role - A.NH : role - A.NH - A.NKV);
+  const int phys = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + pg] : b * A.bt_stride + pg;
+  const int64_t base = ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
+  if (!is_q && !is_k) {
+    const uint16_t* vp = A.v + ((int64_t)b * A.NKV + kvh) * ATT_HD;
+    for (int i = lane; i < ATT_HD; i += 64) A.vc[base + i * ATT_PAGE + slot] = vp[i];
+    return;
+  }
+  const uint16_t* xh = is_q ? A.qg + ((int64_t)b * A.NH + role) * 2 * ATT_HD : A.k + ((int64_t)b * A.NKV + kvh) * ATT_HD;
+  const uint16_t* w = is_q ? A.qw : A.kw;
+  float xv[ATT_HD / 64];
+  double ss = 0.0;
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) { xv[j] = bf16_to_f32(xh[lane + 64 * j]); ss += (double)(xv[j] * xv[j]); }
+  ss = wave_sum_f64(ss);
+  const float rstd = rsqrt_f64(ss / (double)ATT_HD + 1e-6);
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) {
+    const int i = lane + 64 * j;
+    sh[i] = f32_to_bf16(__fmul_rn(__fmul_rn(xv[j], rstd), __fadd_rn(1.0f, bf16_to_f32(w[i]))));
+  }
+  __syncthreads();
+  uint16_t* dst = is_q ? A.qout + ((int64_t)b * A.NH + role) * ATT_HD : A.kc + base + slot * ATT_HD;
+  const int half = A.half;
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) {
+    const int i = lane + 64 * j;
+    uint16_t o = sh[i];
+    if (i < 2 * half) {
+      const int i1 = i < half ? i : i - half;
+      const float x1 = bf16_to_f32(sh[i1]), x2 = bf16_to_f32(sh[i1 + half]);
+      const float c = A.cos_t[(int64_t)pos * half + i1], sn = A.sin_t[(int64_t)pos * half + i1];
+      o = i < half ? f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, sn)))
+                   : f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, sn)));
+    }
+    dst[i] = o;
+  }
+}
+
+int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
+                     const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
+                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size) {
+  BK_REQUIRE(qg && k && v && qw && kw && cos_t && sin_t && qout && kc && vc, "attn_prep: null pointer");
+  BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_prep: head_dim 256 and 16-token pages only");
+  BK_REQUIRE(batch > 0 && batch <= 65535 && NH > 0 && NKV > 0 && half > 0 && 2 * half <= HD, "attn_prep: bad shape");
+  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len && pos_scalar / ATT_PAGE < bt_stride),
+             "attn_prep: pos=%d outside the cache (max_len=%d)", pos_scalar, max_len);
+  PrepArgs A{};
+  A.qg = (const uint16_t*)qg; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v; A.qw = (const uint16_t*)qw; A.kw = (const uint16_t*)kw;
+  A.cos_t = cos_t; A.sin_t = sin_t; A.pos_dev = pos_dev; A.pos_scalar = pos_scalar;
+  A.qout = (uint16_t*)qout; A.kc = (uint16_t*)kc; A.vc = (uint16_t*)vc; A.block_table = block_table; A.bt_stride = bt_stride;
+  A.NH = NH; A.NKV = NKV; A.half = half;
+  hipLaunchKernelGGL(attn_prep_kernel, dim3(NH + 2 * NKV, batch), dim3(64), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
 // ---------------------------------------------------------------- cache append
 // The cache write of src/emitters.ts:202-205: token `pos` of every sequence gets this
 // step's k and v (bf16 [B, NKV, 256]); V goes in dim-major.

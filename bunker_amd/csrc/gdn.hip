@@ -37,10 +37,33 @@ struct GdnArgs {
   float* S_out;
   uint16_t* out;            // bf16 [B, Hg*128]
   int Hg;
+  // conv mode (src/emitters.ts:48-72 folded in): q, k, v above point into the raw qkv projection and every
+  // channel first goes through the 4-tap causal convolution + SiLU; its state rows are shifted in the same pass
+  const uint16_t* conv_st;  // bf16 [B, 3, C]
+  const uint16_t* conv_w;   // bf16 [C, 4]
+  uint16_t* conv_st_new;    // bf16 [B, 3, C], may alias conv_st
+  int C;
 };
 
-template <int CS, bool FUSED>
+// One channel of conv1d_decode: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); returns bf16(r * sigmoid(r)) and
+// writes the state rows (s1, s2, x).  The thread that reads a channel's rows is the one that rewrites them.
+__device__ __forceinline__ uint16_t conv_channel(const GdnArgs& A, int b, int ch, uint16_t xbits) {
+  const uint16_t* sb = A.conv_st + (int64_t)b * 3 * A.C;
+  const uint16_t s0 = sb[ch], s1 = sb[A.C + ch], s2 = sb[2 * A.C + ch];
+  const uint2 wv = *(const uint2*)(A.conv_w + 4 * (int64_t)ch);
+  const float w0 = __uint_as_float(wv.x << 16), w1 = __uint_as_float(wv.x & 0xffff0000u);
+  const float w2 = __uint_as_float(wv.y << 16), w3 = __uint_as_float(wv.y & 0xffff0000u);
+  // products of two bf16 values are exact in f32
+  const float r = __fadd_rn(__fadd_rn(w0 * bf16_to_f32(s0), w1 * bf16_to_f32(s1)),
+                            __fadd_rn(w2 * bf16_to_f32(s2), w3 * bf16_to_f32(xbits)));
+  uint16_t* nb = A.conv_st_new + (int64_t)b * 3 * A.C;
+  nb[ch] = s1; nb[A.C + ch] = s2; nb[2 * A.C + ch] = xbits;
+  return f32_to_bf16(__fmul_rn(r, sigmoid_f64(r)));
+}
+
+template <int CS, bool FUSED, bool CONV = false>
 __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
+  static_assert(!CONV || FUSED, "the convolution is part of the fused op only");
   constexpr int COLS = GDN_D / CS;          // v columns of this workgroup
   constexpr int VQ = COLS / 4;              // float4 column groups
   constexpr int KG = GDN_THREADS / VQ;      // k-row groups
@@ -49,6 +72,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   __shared__ float kn[GDN_D], qn[GDN_D];
   __shared__ float part[KG][COLS];
   __shared__ double red[4];
+  __shared__ __align__(8) uint16_t vsh[CONV ? GDN_D : 4];
 
   const int h = blockIdx.x, slab = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x;
@@ -70,7 +94,13 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     // threads 0..127 hold q, 128..255 hold k
     const bool isk = tid >= 128;
     const int i = tid & 127;
-    const float x = bf16_to_f32((isk ? kp : qp)[i]);
+    float x;
+    if (CONV) {
+      x = bf16_to_f32(conv_channel(A, b, (int)((isk ? kp : qp) - (A.q + (int64_t)b * A.qkv_bstride)) + i, (isk ? kp : qp)[i]));
+      if (!isk) vsh[i] = conv_channel(A, b, (int)(vp - (A.q + (int64_t)b * A.qkv_bstride)) + i, vp[i]);
+    } else {
+      x = bf16_to_f32((isk ? kp : qp)[i]);
+    }
     const double ss = wave_sum_f64((double)(x * x));       // square of a bf16 value: exact in f32
     if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
@@ -111,7 +141,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     kS.x += p.x; kS.y += p.y; kS.z += p.z; kS.w += p.w;
   }
   __syncthreads();   // part is reused for o below
-  const uint2 vv = *(const uint2*)(vp + col0);
+  const uint2 vv = CONV ? *(const uint2*)(vsh + col0) : *(const uint2*)(vp + col0);
   float4 d;
   d.x = (__uint_as_float(vv.x << 16) - kS.x) * beta;
   d.y = (__uint_as_float(vv.x & 0xffff0000u) - kS.y) * beta;
@@ -174,6 +204,25 @@ int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, co
   int rc = check_common(A, batch);
   if (rc) return rc;
   hipLaunchKernelGGL((gdn_step_kernel<1, true>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv_w, const void* z, const float* A_log,
+                          const void* dt_bias, const float* a_p, const float* b_p, const float* norm_w, const float* S_in,
+                          void* out, void* conv_st_new, float* S_out, int Hg, int batch) {
+  GdnArgs A{};
+  const int KEYDIM = Hg * GDN_D;
+  A.q = (const uint16_t*)qkv; A.k = A.q + KEYDIM; A.v = A.q + 2 * KEYDIM;
+  A.qkv_bstride = 3 * (int64_t)KEYDIM;
+  A.z = (const uint16_t*)z; A.A_log = A_log; A.dt_bias = (const uint16_t*)dt_bias; A.a_p = a_p; A.b_p = b_p; A.norm_w = norm_w;
+  A.S_in = S_in; A.S_out = S_out; A.out = (uint16_t*)out; A.Hg = Hg;
+  A.conv_st = (const uint16_t*)conv_st; A.conv_w = (const uint16_t*)conv_w; A.conv_st_new = (uint16_t*)conv_st_new; A.C = 3 * KEYDIM;
+  BK_REQUIRE(qkv && z && A_log && dt_bias && a_p && b_p && norm_w && conv_st && conv_w && conv_st_new, "gdn_conv: null pointer");
+  BK_REQUIRE(((uintptr_t)conv_w & 7) == 0, "gdn_conv: the conv weight must be 8-byte aligned");
+  int rc = check_common(A, batch);
+  if (rc) return rc;
+  hipLaunchKernelGGL((gdn_step_kernel<1, true, true>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -10,8 +10,10 @@
 // (every term exact, ~1e-16 accumulation error, one rounding to f32), so the batched
 // path returns the same bits as the batch-1 path:
 //   y[b, n] = sum_blk ( d * sum_j d8_j[b] * (sc_j * I_j) - dmin * sum_j m_j * s8_j[b] )
-// One wavefront per workgroup; the activation blocks of the current super-block are
-// staged in LDS (int8 data in MFMA operand order, scales as doubles).
+// A workgroup owns one 32 x 32 output tile; its NW wavefronts split K by super-block (wave w takes
+// blocks w, w + NW, ...) and add their double partials in wave order through LDS at the end.  The
+// int8 activation operand is read straight from the Q8_1 rows (16-byte pieces, L2-resident); only
+// the activation scales of the wave's current super-block are staged in LDS, as doubles.
 #include "ops.h"
 
 namespace bk {
@@ -24,53 +26,52 @@ enum : int { GEPI_F32 = 0, GEPI_BF16 = 1, GEPI_BF16_ADD = 2 };
 // rows of the 32x32 accumulator held by a lane: r = 0..15 -> 8*(r/4) + 4*(lane/32) + r%4
 __device__ __forceinline__ int mfma32_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
 
-template <int EPI>
-__global__ __launch_bounds__(64) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq,
-                                                                void* __restrict__ out, const uint16_t* __restrict__ res,
-                                                                int N, int nb, int B) {
-  // activation int8 data of one super-block in operand order: [j][half][b] x 16 bytes
-  __shared__ uint4 lds_q[8 * 2 * 32];
-  __shared__ double lds_d8[8][32], lds_s8[8][32];
+template <int EPI, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq,
+                                                                     void* __restrict__ out, const uint16_t* __restrict__ res,
+                                                                     int N, int nb, int B) {
+  __shared__ double lds_d8[NW][8][32], lds_s8[NW][8][32];
+  __shared__ double lds_acc[NW > 1 ? 16 * 64 : 1];
 
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = lane >> 5, col = lane & 31;
   const int n0 = blockIdx.x * 32;
   const int n = min(n0 + col, N - 1);                 // rows past N recompute row N-1 and are not stored
   const uint8_t* wrow = W + (int64_t)n * nb * 144;
   const int64_t xrow_bytes = (int64_t)nb * 8 * 36;
+  // A operand: batch row `col` (rows past B re-read row B-1; their results are not stored)
+  const uint8_t* xrow = xq + (int64_t)min(col, B - 1) * xrow_bytes + 16 * half;
 
   double acc[16];
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0;
 
-  for (int blk = 0; blk < nb; blk++) {
+  for (int blk = wave; blk < nb; blk += NW) {
     // weights of this lane's row: header + its half of every 32-byte nibble group
     const uint4 hdr = *(const uint4*)(wrow + blk * 144);
     uint4 qs[4];
 #pragma unroll
     for (int g = 0; g < 4; g++) qs[g] = *(const uint4*)(wrow + blk * 144 + 16 + 32 * g + 16 * half);
-
-    __syncthreads();   // the previous super-block's LDS contents are no longer needed
-    // stage activations: 32 rows x 8 sub-blocks = 256 Q8_1 blocks, 4 per lane
+    // activations: the lane's 16 int8 of each of the 8 sub-blocks (4-byte aligned 16-byte loads)
+    uint4 xa4[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const uint32_t* p = (const uint32_t*)(xrow + (int64_t)(blk * 8 + j) * 36);
+      xa4[j] = make_uint4(p[0], p[1], p[2], p[3]);
+    }
+    // scales of the 32 x 8 activation blocks of this super-block -> LDS of this wave, 4 per lane
+    __builtin_amdgcn_wave_barrier();     // the previous super-block's scales have been consumed by every lane
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int t = lane + 64 * i;
       const int b = t >> 3, j = t & 7;
-      uint32_t w[9];
-      if (b < B) {
-        const uint32_t* p = (const uint32_t*)(xq + (int64_t)b * xrow_bytes + (int64_t)(blk * 8 + j) * 36);
-#pragma unroll
-        for (int k = 0; k < 9; k++) w[k] = p[k];
-      } else {
-#pragma unroll
-        for (int k = 0; k < 9; k++) w[k] = 0;
-      }
-      lds_q[(j * 2 + 0) * 32 + b] = make_uint4(w[0], w[1], w[2], w[3]);
-      lds_q[(j * 2 + 1) * 32 + b] = make_uint4(w[4], w[5], w[6], w[7]);
-      lds_d8[j][b] = (double)half_to_f32((uint16_t)(w[8] & 0xffffu));
-      lds_s8[j][b] = (double)half_to_f32((uint16_t)(w[8] >> 16));
+      const uint32_t ds = *(const uint32_t*)(xq + (int64_t)min(b, B - 1) * xrow_bytes + (int64_t)(blk * 8 + j) * 36 + 32);
+      lds_d8[wave][j][b] = (double)half_to_f32((uint16_t)(ds & 0xffffu));
+      lds_s8[wave][j][b] = (double)half_to_f32((uint16_t)(ds >> 16));
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu)), dmin = half_to_f32((uint16_t)(hdr.x >> 16));
     // all eight 6-bit scales and mins of the block, four per dword
@@ -93,8 +94,7 @@ __global__ __launch_bounds__(64) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* _
       } else {
         wb = (i32x4_t){(int)(q.x & 0x0f0f0f0fu), (int)(q.y & 0x0f0f0f0fu), (int)(q.z & 0x0f0f0f0fu), (int)(q.w & 0x0f0f0f0fu)};
       }
-      const uint4 xa4 = lds_q[(j * 2 + half) * 32 + col];
-      const i32x4_t xa = (i32x4_t){(int)xa4.x, (int)xa4.y, (int)xa4.z, (int)xa4.w};
+      const i32x4_t xa = (i32x4_t){(int)xa4[j].x, (int)xa4[j].y, (int)xa4[j].z, (int)xa4[j].w};
       i32x16_t c;
 #pragma unroll
       for (int r = 0; r < 16; r++) c[r] = 0;
@@ -106,13 +106,28 @@ __global__ __launch_bounds__(64) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* _
       for (int r = 0; r < 16; r++) {
         const int b = mfma32_row(r, half);
         const int p = __mul24(sc, c[r]);                            // 6-bit x 17-bit: exact
-        sblk[r] = fma(lds_d8[j][b], (double)p, sblk[r]);
-        mblk[r] = fma(mj, lds_s8[j][b], mblk[r]);
+        sblk[r] = fma(lds_d8[wave][j][b], (double)p, sblk[r]);
+        mblk[r] = fma(mj, lds_s8[wave][j][b], mblk[r]);
       }
     }
     const double dd = (double)d, dm = (double)dmin;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] += dd * sblk[r] - dm * mblk[r];
+  }
+
+  if (NW > 1) {
+    // partial sums meet in wave order; the last wave ends up with the totals
+    for (int w = 0; w < NW; w++) {
+      if (wave == w) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          if (w > 0) acc[r] += lds_acc[r * 64 + lane];
+          if (w < NW - 1) lds_acc[r * 64 + lane] = acc[r];
+        }
+      }
+      if (w < NW - 1) __syncthreads();
+    }
+    if (wave != NW - 1) return;
   }
 
   if (n0 + col < N) {
@@ -129,6 +144,16 @@ __global__ __launch_bounds__(64) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* _
   }
 }
 
+int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
+
+template <int NW>
+static void launch_gemm_nw(int epi, dim3 grid, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int nb, int batch) {
+  const dim3 block(64 * NW);
+  if (epi == GEPI_F32) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_F32, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
+  else if (epi == GEPI_BF16) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16_ADD, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
+}
+
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
                               const void* residual) {
   BK_REQUIRE(W && xq && y, "gemm_q4k_q8_1_mfma: null pointer");
@@ -137,12 +162,22 @@ int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int
   BK_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gemm_q4k_q8_1_mfma: out_dtype must be 0 (f32) or 1 (bf16)");
   BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemm_q4k_q8_1_mfma: a residual needs bf16 output");
   BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "gemm_q4k_q8_1_mfma: W must be 16-byte and xq 4-byte aligned");
-  dim3 grid((N + 31) / 32), block(64);
+  const dim3 grid((N + 31) / 32);
   const uint8_t* w = (const uint8_t*)W; const uint8_t* x = (const uint8_t*)xq; const uint16_t* r = (const uint16_t*)residual;
   const int nb = K / 256;
-  if (out_dtype == DT_F32) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_F32>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
-  else if (!residual) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16_ADD>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
+  const int epi = out_dtype == DT_F32 ? GEPI_F32 : (residual ? GEPI_BF16_ADD : GEPI_BF16);
+  // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
+  // and two ways when the tiles alone fill the chip many times over (lm_head)
+  int nw = g_tune_gemm_nw;
+  if (nw <= 0) {
+    const int tiles = (N + 31) / 32;
+    nw = nb >= 16 ? 8 : (nb >= 4 ? 4 : (nb >= 2 ? 2 : 1));
+    if (tiles >= 8 * num_cus() && nw > 2) nw = 2;
+  }
+  if (nw >= 8) launch_gemm_nw<8>(epi, grid, w, x, y, r, N, nb, batch);
+  else if (nw >= 4) launch_gemm_nw<4>(epi, grid, w, x, y, r, N, nb, batch);
+  else if (nw >= 2) launch_gemm_nw<2>(epi, grid, w, x, y, r, N, nb, batch);
+  else launch_gemm_nw<1>(epi, grid, w, x, y, r, N, nb, batch);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

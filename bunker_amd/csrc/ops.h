@@ -41,6 +41,7 @@ int launch_gemv_group(const void* xq, int K, int batch, int ngroups, const void*
 int launch_gemv_swiglu_q8(const void* Wg, const void* Wu, const void* xq, void* act, void* act_q8, int N, int K, int batch);
 
 // gemm_mfma.hip
+extern int g_tune_gemm_nw;
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
                               const void* residual);
 
@@ -64,6 +65,9 @@ int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* 
 // gdn.hip
 int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
                      const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch);
+int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv_w, const void* z, const float* A_log,
+                          const void* dt_bias, const float* a_p, const float* b_p, const float* norm_w, const float* S_in,
+                          void* out, void* conv_st_new, float* S_out, int Hg, int batch);
 int launch_gdn_core(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* S_in,
                     void* out, float* S_out, int Hg, int batch);
 
@@ -74,6 +78,9 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
                        int NH, int NKV, int HD, int page_size, int splits);
+int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
+                     const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
+                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size);
 int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
                      const int32_t* pos_dev, int pos_scalar, int batch, int NKV, int HD, int page_size);
 

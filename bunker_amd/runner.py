@@ -35,6 +35,7 @@ class KernelPlan:
     args: list            # external tensor names, in slot order
     grid: list
     group: list
+    aux: dict = field(default_factory=dict)   # name -> bytes of buffers that exist only between fused kernels
 
 
 @dataclass
@@ -49,6 +50,91 @@ class CompiledStep:
 def choosePartition(graph: Graph, env=None, opts: dict | None = None) -> Partition:
     """Every node its own kernel (src/runner.ts:40-49)."""
     return [[n] for n in graph.nodes]
+
+
+LM_HEAD_ROWS = 32768     # matmuls with more rows keep the stand-alone norm + quantizer (its cost is paid once, not per workgroup)
+
+
+def fusedPartition(graph: Graph) -> Partition:
+    """Groups of nodes that one fused kernel (or one short kernel sequence) serves.
+
+    The counterpart of src/fusion.ts's partitioning, with the fusions that pay on this hardware:
+      rmsnorm + the matmuls that read it                      (norm and Q8_1 in the GEMV prologue)
+      rmsnorm + gate + up + swiglu                            (SwiGLU in the GEMV epilogue)
+      matmul + cast + add                                     (residual add in the GEMV epilogue)
+      conv1d_decode + gdn_delta_rule                          (the conv output stays on chip)
+      qnorm + rope + knorm + ropek + fa2_attn                 (norm, rotation and cache append in one launch)
+    A group is formed only when no tensor produced inside it (other than its declared result) is read outside.
+    """
+    taken: set = set()
+    groups: dict[int, list] = {}          # first node id -> group
+
+    def consumers(t):
+        return graph.tensors[t].consumers
+
+    def only_inside(nodes, results):
+        ids = {n.id for n in nodes}
+        for n in nodes:
+            for o in n.outputs:
+                if o.tensorName in results or graph.tensors[o.tensorName].role == "state":
+                    continue
+                if any(c.id not in ids for c in consumers(o.tensorName)):
+                    return False
+        return True
+
+    def take(nodes):
+        nodes = sorted(nodes, key=lambda n: n.id)
+        groups[nodes[0].id] = nodes
+        taken.update(n.id for n in nodes)
+
+    for n in graph.nodes:
+        if n.id in taken:
+            continue
+        if n.op == "rmsnorm":
+            cons = consumers(n.outputs[0].tensorName)
+            if cons and all(c.op == "gemm" and c.inputs[0].tensorName == n.outputs[0].tensorName for c in cons) and len(cons) <= 4:
+                if max(int(c.params["N"]) for c in cons) > LM_HEAD_ROWS:
+                    continue
+                sw = None
+                if len(cons) == 2:
+                    c0, c1 = (consumers(c.outputs[0].tensorName) for c in cons)
+                    if len(c0) == 1 and len(c1) == 1 and c0[0] is c1[0] and c0[0].op == "swiglu" and not cons[0].params.get("cast") \
+                            and int(cons[0].params["N"]) % 4 == 0:
+                        sw = c0[0]
+                nodes = [n] + list(cons) + ([sw] if sw else [])
+                results = {sw.outputs[0].tensorName} if sw else {c.outputs[0].tensorName for c in cons}
+                if only_inside(nodes, results):
+                    take(nodes)
+        elif n.op == "gemm" and not n.params.get("cast"):
+            c = consumers(n.outputs[0].tensorName)
+            if len(c) == 1 and c[0].op == "cast":
+                a = consumers(c[0].outputs[0].tensorName)
+                if len(a) == 1 and a[0].op == "add" and a[0].id not in taken:
+                    take([n, c[0], a[0]])
+        elif n.op == "conv1d_decode":
+            c = consumers(n.outputs[0].tensorName)
+            if len(c) == 1 and c[0].op == "gdn_delta_rule" and c[0].inputs[0].tensorName == n.outputs[0].tensorName:
+                take([n, c[0]])
+        elif n.op == "qnorm":
+            qn_out = n.outputs[0].tensorName
+            fa = next((c for c in consumers(qn_out) if c.op == "fa2_attn"), None)
+            rope = next((c for c in consumers(qn_out) if c.op == "rope"), None)
+            if fa is None or rope is None:
+                continue
+            kn = graph.tensors[fa.inputs[1].tensorName].producer
+            ropek = next((c for c in consumers(kn.outputs[0].tensorName) if c.op == "ropek"), None) if kn is not None and kn.op == "knorm" else None
+            if ropek is None or fa.inputs[3].tensorName != n.inputs[0].tensorName:
+                continue
+            nodes = [n, rope, kn, ropek, fa]
+            if only_inside(nodes, {fa.outputs[0].tensorName}):
+                take(nodes)
+    out = []
+    for n in graph.nodes:
+        if n.id in groups:
+            out.append(groups[n.id])
+        elif n.id not in taken:
+            out.append([n])
+    return out
 
 
 def topoOrder(graph: Graph, partition: Partition) -> Partition:
@@ -119,13 +205,85 @@ def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str
     return " ".join(parts)
 
 
+def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict) -> KernelPlan:
+    """The fused op spec and slot list for a multi-node group (see fusedPartition)."""
+    ops = tuple(n.op for n in grp)
+    bpart = f" batch={batch}" if batch != 1 else ""
+    name = "+".join(ops) + f"_{grp[0].id}"
+    if ops[0] == "rmsnorm" and ops[-1] == "swiglu":
+        norm, gate, up, sw = grp
+        N, K = int(gate.params["N"]), int(gate.params["K"])
+        spec = f"gemv_fused K={K} pro=2 G=2 swiglu=1 N0={N} N1={N}" + bpart
+        args = [norm.inputs[0].tensorName, norm.inputs[1].tensorName, gate.inputs[1].tensorName, up.inputs[1].tensorName,
+                sw.outputs[0].tensorName]
+        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+    if ops[0] == "rmsnorm" and all(o == "gemm" for o in ops[1:]) and len(ops) > 1:
+        norm, gemms = grp[0], grp[1:]
+        K = int(gemms[0].params["K"])
+        spec = f"gemv_fused K={K} pro=2 G={len(gemms)} " + " ".join(
+            f"N{i}={int(m.params['N'])} epi{i}={1 if m.params.get('cast') else 0}" for i, m in enumerate(gemms)) + bpart
+        args = [norm.inputs[0].tensorName, norm.inputs[1].tensorName]
+        for m in gemms:
+            args += [m.inputs[1].tensorName, m.outputs[0].tensorName]
+        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+    if ops == ("gemm", "cast", "add"):
+        m, c, a = grp
+        cast_out = c.outputs[0].tensorName
+        res = next(i.tensorName for i in a.inputs if i.tensorName != cast_out)
+        N, K = int(m.params["N"]), int(m.params["K"])
+        src = m.inputs[0].tensorName
+        if src in q8_of:      # the activation already exists as Q8_1 (written by a stand-alone rmsnorm_q8_1)
+            spec, first = f"gemv_fused K={K} pro=0 G=1 N0={N} epi0=2" + bpart, q8_of[src]
+        else:
+            spec, first = f"gemv_fused K={K} pro=1 G=1 N0={N} epi0=2" + bpart, src
+        return KernelPlan(spec, name, [first, m.inputs[1].tensorName, res, a.outputs[0].tensorName], [1, 1, 1], grp)
+    if ops == ("conv1d_decode", "gdn_delta_rule"):
+        cv, gd = grp
+        spec = f"gdn_conv LVH={int(gd.params['LVH'])} LKD={int(gd.params['LKD'])} LVD={int(gd.params['LVD'])}" + bpart
+        args = [cv.inputs[0].tensorName, cv.inputs[1].tensorName, cv.inputs[2].tensorName] + \
+               [i.tensorName for i in gd.inputs[1:]] + [gd.outputs[0].tensorName, cv.outputs[1].tensorName, gd.outputs[1].tensorName]
+        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+    if ops == ("qnorm", "rope", "knorm", "ropek", "fa2_attn"):
+        qn, rp, kn, rk, fa = grp
+        P = fa.params
+        spec = (f"fa2_fused HD={int(P['HD'])} NH={int(P['NH'])} NKV={int(P['NKV'])} MAX_LEN={int(P['MAX_LEN'])} "
+                f"ROT_HALF={int(rp.params['ROT_HALF'])}") + bpart + (" pos_dev=1" if device_scalars else "")
+        args = [qn.inputs[0].tensorName, kn.inputs[0].tensorName, fa.inputs[2].tensorName, qn.inputs[1].tensorName,
+                kn.inputs[1].tensorName, rp.inputs[1].tensorName, rp.inputs[2].tensorName, rp.inputs[3].tensorName,
+                fa.inputs[4].tensorName, fa.inputs[5].tensorName, fa.outputs[0].tensorName]
+        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+    raise NotImplementedError(f"no fused kernel for the group {ops}")
+
+
 def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_scalars: bool = False) -> list:
+    """One KernelPlan per group.  Single nodes keep the reference's op and slot order; in a partition that has
+    fused groups, a stand-alone rmsnorm whose readers are all matmuls also leaves its result as Q8_1 in an
+    auxiliary buffer, and those matmuls read that instead of quantizing again."""
+    fused = any(len(grp) > 1 for grp in ordered)
+    q8_of: dict[str, str] = {}
     plans = []
     for grp in ordered:
         if len(grp) != 1:
-            raise NotImplementedError("multi-node groups are produced by fusedPartition only")
+            plans.append(_group_plan(graph, grp, batch, device_scalars, q8_of))
+            continue
         n = grp[0]
         args = [i.tensorName for i in n.inputs] + [o.tensorName for o in n.outputs]
+        bpart = f" batch={batch}" if batch != 1 else ""
+        if fused and n.op == "rmsnorm":
+            out = n.outputs[0].tensorName
+            cons = graph.tensors[out].consumers
+            if cons and all(c.op == "gemm" and c.inputs[0].tensorName == out for c in cons):
+                aux = out + ".q8_1"
+                q8_of[out] = aux
+                N = int(n.params["N"])
+                plans.append(KernelPlan(f"rmsnorm_q8_1 N={N}" + bpart, f"rmsnorm_q8_1_{n.id}", args + [aux], n.grid, grp,
+                                        {aux: batch * (N // 32) * 36}))
+                continue
+        if fused and n.op == "gemm" and n.inputs[0].tensorName in q8_of:
+            N, K = int(n.params["N"]), int(n.params["K"])
+            spec = f"gemv_fused K={K} pro=0 G=1 N0={N} epi0={1 if n.params.get('cast') else 0}" + bpart
+            plans.append(KernelPlan(spec, f"gemv_{n.id}", [q8_of[n.inputs[0].tensorName], args[1], args[2]], n.grid, grp))
+            continue
         plans.append(KernelPlan(node_spec(n, batch, device_scalars), f"{n.op}_{n.id}", args, n.grid, grp))
     return plans
 
@@ -137,7 +295,7 @@ def compileStep(graph: Graph, partition: Partition, batch: int = 1, device_scala
     schedule = []
     for p in plans:
         # handles own workspaces, so kernels with a workspace are not shared between nodes
-        shareable = p.group[0].op not in ("gemm", "fa2_attn", "argmax")
+        shareable = len(p.group) == 1 and p.group[0].op not in ("gemm", "fa2_attn", "argmax") and not p.spec.startswith("gemv_fused")
         if shareable and p.spec in cache:
             k = cache[p.spec]
         else:
@@ -214,6 +372,7 @@ class DecodeEnv:
         self.graph = graph
         self.inplace = inplace_state
         self.ptr: dict[str, int] = {}
+        self.aux: dict[str, int] = {}
         self.state_bufs: dict[str, list] = {}
         self.state_cur: dict[str, int] = {}
         self.non_rotating: set = set()
@@ -259,7 +418,20 @@ class DecodeEnv:
         """Device pointers of the weights, to share them with another DecodeEnv (device_weights=...)."""
         return {n: p for n, p in self.ptr.items() if self.graph.tensors[n].role == "weight"}
 
+    def add_aux(self, name: str, nbytes: int) -> int:
+        """A buffer that only fused kernels of one compiled step see (not a tensor of the graph)."""
+        if name not in self.aux:
+            self.aux[name] = self._own(rt.cuAlloc(nbytes))
+        return self.aux[name]
+
+    def bind(self, compiled: "CompiledStep") -> None:
+        for plan, _ in compiled.schedule:
+            for name, nbytes in plan.aux.items():
+                self.add_aux(name, nbytes)
+
     def resolve(self, name: str) -> int:
+        if name in self.aux:
+            return self.aux[name]
         t = self.graph.t(name)
         if t.role == "scalar":
             raise KeyError(f"resolve: scalar '{name}' is passed by the runner")
@@ -299,6 +471,7 @@ class DeviceLoop:
             raise ValueError("DeviceLoop needs DecodeEnv(inplace_state=True)")
         self.graph, self.env, self.batch, self.max_steps = graph, env, batch, max_steps
         self.compiled = compileStep(graph, partition or choosePartition(graph), batch, device_scalars=True)
+        env.bind(self.compiled)
         ids = np.asarray(start_tokens, np.int32).reshape(batch)
         pos = np.broadcast_to(np.asarray(start_pos, np.int32), (batch,)).copy()
         self.d_ids = rt.to_device(ids)

@@ -107,3 +107,72 @@ def test_gemv_fused_swiglu(orc, dev, K, N, batch):
     for b in range(batch):
         ref = orc.swiglu(orc.gemv_q4k_q8_1(Wg, xq_rows[b], N, K), orc.gemv_q4k_q8_1(Wu, xq_rows[b], N, K))
         assert np.array_equal(got[b], ref), b
+
+
+@pytest.mark.parametrize("Hg,B", [(16, 1), (3, 2)])
+def test_gdn_conv_is_conv1d_then_delta_rule(orc, dev, Hg, B):
+    """gdn_conv = conv1d_decode + gdn_delta_rule: output, S and the shifted conv state, to the bit."""
+    print(f"gdn_conv Hg={Hg} B={B}", flush=True)
+    g = synth.rng(700 + Hg + B)
+    C = 3 * Hg * 128
+    qkv = bf(g.standard_normal((B, C)).astype(np.float32))
+    st = bf(g.standard_normal((B, 3, C)).astype(np.float32))
+    cw = bf((g.standard_normal((C, 4)) * 0.5).astype(np.float32))
+    z = bf(g.standard_normal((B, Hg * 128)).astype(np.float32))
+    A_log = g.uniform(-2, 1, Hg).astype(np.float32)
+    dt_bias = bf(g.standard_normal(Hg).astype(np.float32))
+    a_p = g.standard_normal((B, Hg)).astype(np.float32); b_p = g.standard_normal((B, Hg)).astype(np.float32)
+    norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    S = (g.standard_normal((B, Hg, 128, 128)) * 0.02).astype(np.float32)
+    dout, dS, dst = dev.empty(B * Hg * 128 * 2), dev.empty(S.nbytes), dev.up(st)
+    launch(f"gdn_conv LVH={Hg} LKD=128 LVD=128 batch={B}",
+           [dev.up(qkv), dst, dev.up(cw), dev.up(z), dev.up(A_log), dev.up(dt_bias), dev.up(a_p), dev.up(b_p), dev.up(norm_w),
+            dev.up(S), dout, dst, dS])        # conv state updated in place
+    out = rt.from_device(dout, (B, Hg * 128), np.uint16); Sn = rt.from_device(dS, S.shape, np.float32)
+    stn = rt.from_device(dst, (B, 3, C), np.uint16)
+    for b in range(B):
+        conv, rs = orc.conv1d_decode(qkv[b], st[b], cw)
+        ro, rS = orc.gdn_step(conv, z[b], A_log, dt_bias, a_p[b], b_p[b], norm_w, S[b], Hg, rows_per_chain=16)
+        assert np.array_equal(stn[b], rs)
+        assert np.array_equal(Sn[b].view(np.uint32), rS.view(np.uint32))
+        assert np.array_equal(out[b], ro)
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_fa2_fused_is_norm_rope_append_attend(orc, dev, batch):
+    """fa2_fused = qnorm, rope, knorm, ropek, cache append (all to the bit: the caches are compared) + attention
+    (2e-2 max-abs against the checker fed with the same normalised, rotated q)."""
+    print(f"fa2_fused batch={batch}", flush=True)
+    g = synth.rng(720 + batch)
+    NH, NKV, HD, HALF, MAXL = 16, 2, 256, 32, 512
+    ppseq = MAXL // 16
+    pos = [300, 15, 16][:batch]
+    cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+    kc = bf(g.standard_normal((batch * ppseq, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((batch * ppseq, NKV, 16, HD)).astype(np.float32))
+    qgate = bf(g.standard_normal((batch, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((batch, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((batch, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    dkc, dvc = dev.up(kc), dev.up(rt.v_pages_to_device_layout(vc))
+    dout = dev.empty(batch * NH * HD * 2)
+    spec = f"fa2_fused HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF}"
+    common = [dev.up(qgate), dev.up(k), dev.up(v), dev.up(qw), dev.up(kw), dev.up(cos_t), dev.up(sin_t)]
+    if batch == 1:
+        launch(spec, common + [pos[0], dkc, dvc, dout])
+    else:
+        launch(spec + f" batch={batch} pos_dev=1", common + [dev.up(np.array(pos, np.int32)), dkc, dvc, dout])
+    out = rt.from_device(dout, (batch, NH, HD), np.uint16)
+    bt = np.arange(batch * ppseq, dtype=np.int32).reshape(batch, ppseq)
+    qn = np.empty((batch, NH, HD), np.uint16)
+    for b in range(batch):
+        qb = orc.headnorm(qgate[b].ravel(), qw, NH, HD, 2 * HD)
+        qn[b] = orc.rope(qb, cos_t, sin_t, pos[b], NH, HD, HALF).reshape(NH, HD)
+        kb = orc.rope(orc.headnorm(k[b].ravel(), kw, NKV, HD, HD), cos_t, sin_t, pos[b], NKV, HD, HALF)
+        orc.kv_append(kb.reshape(NKV, HD), v[b], kc, vc, bt[b], pos[b], NKV, HD, 16)
+    kc_d = rt.from_device(dkc, kc.shape, np.uint16)
+    vc_d = rt.from_device(dvc, (batch * ppseq, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
+    assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
+    ctx = np.array(pos, np.int32) + 1
+    ro, _ = orc.attn_decode_paged(qn, kc, vc, bt, ctx, batch, NH, NKV, HD, 16, gate=qgate.ravel()[HD:],
+                                  gate_bstride=NH * 2 * HD, gate_hstride=2 * HD)
+    assert np.abs(f32(out).astype(np.float64) - f32(ro)).max() <= 2e-2

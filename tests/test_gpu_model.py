@@ -28,7 +28,7 @@ def _fa_layers(D):
     return [l for l in range(D.NL) if D.is_full_attention(l)]
 
 
-def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None):
+def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=False):
     """GPU DeviceLoop one token at a time against the checker continued from the GPU's attention outputs.
 
     check: the sequences of the batch the checker recomputes (all by default; sequences are independent)."""
@@ -37,7 +37,8 @@ def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None):
     check = list(range(B)) if check is None else list(check)
     g = model.buildModelGraph(D, B)
     env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
-    loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=use_graph)
+    loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=use_graph,
+                             partition=runner.fusedPartition(g) if fused else None)
     fa_nodes = [n for n in g.nodes if n.op == "fa2_attn"]
     logits_name = next(n for n in g.nodes if n.op == "argmax").inputs[0].tensorName
     ref = RefModel(D, W, {k: np.asarray(v)[check] for k, v in S.items()}, batch=len(check))
@@ -110,23 +111,25 @@ def test_tiny_model_reference_loop(orc):
     env.close()
 
 
-@pytest.mark.parametrize("use_graph", [False, True])
-def test_tiny_model_device_loop_batch3(orc, use_graph):
+@pytest.mark.parametrize("use_graph,fused", [(False, False), (True, False), (False, True), (True, True)])
+def test_tiny_model_device_loop_batch3(orc, use_graph, fused):
     D = TINY
     W = synth_model.synth_weights(D, seed=11)
     S = synth_model.synth_state(D, batch=3, seed=13)
-    toks, vals = _strict_decode(D, W, S, [77, 5, 900], 40, 6, use_graph)
+    toks, vals = _strict_decode(D, W, S, [77, 5, 900], 40, 6, use_graph, fused=fused)
     _free_running(D, W, S, [77, 5, 900], 40, 6, toks, vals)
 
 
-def test_synthetic_qwen35_decode_step_bs1(orc):
-    """BASELINE configs[4], batch 1: 24 layers (3 GDN : 1 FA), hidden 2048, FFN 6144, vocab 151936, KV at 4096."""
+@pytest.mark.parametrize("fused", [False, True])
+def test_synthetic_qwen35_decode_step_bs1(orc, fused):
+    """BASELINE configs[4], batch 1: 24 layers (3 GDN : 1 FA), hidden 2048, FFN 6144, vocab 151936, KV at 4096.
+    fused: the partition with the fused kernels (138 launches per token instead of 425); same bits."""
     D = SYNTH
     print("generating weights", flush=True)
     W = synth_model.synth_weights(D, seed=2026)
     S = synth_model.synth_state(D, batch=1, seed=7)
     steps, pos0, tok0 = 6, 4096, 9419          # start token of the reference's benches (bench_graph_decode.ts:77)
-    toks, vals = _strict_decode(D, W, S, [tok0], pos0, steps, use_graph=True)
+    toks, vals = _strict_decode(D, W, S, [tok0], pos0, steps, use_graph=True, fused=fused)
     _free_running(D, W, S, [tok0], pos0, steps, toks, vals)
 
 
@@ -137,6 +140,8 @@ def test_tiny_model_batch32_mfma_path(orc):
     S = synth_model.synth_state(D, batch=32, seed=14)
     starts = [(37 * i + 5) % D.VOCAB for i in range(32)]
     toks, vals = _strict_decode(D, W, S, starts, 40, 4, use_graph=True)
+    tf, vf = _strict_decode(D, W, S, starts, 40, 4, use_graph=True, fused=True)
+    assert np.array_equal(tf, toks) and np.array_equal(vf.view(np.uint32), vals.view(np.uint32))
     # a sequence decodes to the same tokens alone (GEMV path) as inside the batch (MFMA path)
     S1 = {k: np.asarray(v)[7:8] for k, v in S.items()}
     t1, v1 = _strict_decode(D, W, S1, [starts[7]], 40, 4, use_graph=False)
@@ -150,4 +155,4 @@ def test_synthetic_qwen35_decode_step_bs32(orc):
     W = synth_model.synth_weights(D, seed=2026)
     S = synth_model.synth_state(D, batch=32, seed=8, share_kv_across_batch=True)
     starts = [(9419 + 4099 * i) % D.VOCAB for i in range(32)]
-    _strict_decode(D, W, S, starts, 4096, 2, use_graph=True, check=[0, 13, 31])
+    _strict_decode(D, W, S, starts, 4096, 2, use_graph=True, check=[0, 13, 31], fused=True)

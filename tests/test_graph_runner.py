@@ -93,3 +93,43 @@ def test_reference_model_runs_on_cpu(orc):
     k0 = "model.layers.3.kv_k"
     assert not np.array_equal(m.S[k0][0, 40 // 16, :, 40 % 16], S[k0][0, 40 // 16, :, 40 % 16])
     assert np.array_equal(m.S[k0][0, 0], S[k0][0, 0])
+
+
+def test_fused_partition_groups_and_specs():
+    """Every node lands in exactly one group; the groups are the five fusions; a scrambled fused partition
+    still orders by dependencies; the fused specs carry shapes and epilogues."""
+    import collections
+    g = model.buildModelGraph(SYNTH)
+    part = runner.fusedPartition(g)
+    ids = [n.id for grp in part for n in grp]
+    assert sorted(ids) == [n.id for n in g.nodes]
+    kinds = collections.Counter(tuple(n.op for n in grp) for grp in part)
+    assert kinds[("rmsnorm", "gemm", "gemm", "gemm", "gemm")] == 18          # qkv, z, a, b
+    assert kinds[("rmsnorm", "gemm", "gemm", "gemm")] == 6                   # q, k, v
+    assert kinds[("rmsnorm", "gemm", "gemm", "swiglu")] == 24
+    assert kinds[("gemm", "cast", "add")] == 48                             # out/o_proj and down with their residual adds
+    assert kinds[("conv1d_decode", "gdn_delta_rule")] == 18
+    assert kinds[("qnorm", "rope", "knorm", "ropek", "fa2_attn")] == 6
+    assert kinds[("rmsnorm",)] == 1 and kinds[("gemm",)] == 1               # final norm and lm_head stay apart
+    assert len(part) == 124
+    ordered = runner.topoOrder(g, part[::-1])
+    done = set()
+    for grp in ordered:
+        inside = {n.id for n in grp}
+        for n in grp:
+            for d in g.deps()[n.id]:
+                assert d in done or d in inside
+        done |= inside
+    plans = runner.compilePartition(g, runner.topoOrder(g, part), 1, True)
+    specs = [p.spec for p in plans]
+    assert "gemv_fused K=2048 pro=2 G=4 N0=6144 epi0=1 N1=2048 epi1=1 N2=16 epi2=0 N3=16 epi3=0" in specs
+    assert "gemv_fused K=2048 pro=2 G=2 swiglu=1 N0=6144 N1=6144" in specs
+    assert "gemv_fused K=6144 pro=1 G=1 N0=2048 epi0=2" in specs
+    assert "fa2_fused HD=256 NH=16 NKV=2 MAX_LEN=4352 ROT_HALF=32 pos_dev=1" in specs
+    # lm_head reads the Q8_1 row the stand-alone final norm leaves in an auxiliary buffer
+    norm = next(p for p in plans if p.spec.startswith("rmsnorm_q8_1"))
+    head = next(p for p in plans if "N0=151936" in p.spec)
+    assert list(norm.aux) == [head.args[0]] and "pro=0" in head.spec
+    # residual of the fused matmul + cast + add is the add's other input
+    down = next(p for p in plans if p.spec.startswith("gemv_fused K=6144"))
+    assert g.t(down.args[2]).producer.op == "add" and g.t(down.args[3]).producer.op == "add"
