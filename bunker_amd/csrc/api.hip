@@ -82,6 +82,21 @@ static int matmul_q8_1(const void* W, const void* xq, void* y, int N, int K, int
   }
   return BK_OK;
 }
+// several matrices over the same activation rows, 32 rows of the batch per launch
+static int matmul_group_mfma(const void* xq, int K, int batch, int G, const void* const* W, void* const* out, const void* const* res,
+                             const int* N, const int* epi) {
+  for (int b0 = 0; b0 < batch; b0 += 32) {
+    const int nbat = batch - b0 < 32 ? batch - b0 : 32;
+    void* o[4]; const void* r[4];
+    for (int i = 0; i < G; i++) {
+      o[i] = (uint8_t*)out[i] + (size_t)b0 * N[i] * (epi[i] == 0 ? 4 : 2);
+      r[i] = res[i] ? (const uint8_t*)res[i] + (size_t)b0 * N[i] * 2 : nullptr;
+    }
+    int rc = launch_gemm_group_mfma((const uint8_t*)xq + (size_t)b0 * (K / 32) * 36, K, nbat, G, W, o, r, N, epi);
+    if (rc) return rc;
+  }
+  return BK_OK;
+}
 static int run_gemm(Kernel& k, const uint64_t* s) {
   const int N = (int)k.get("N", 0), K = (int)k.get("K", 0), batch = (int)k.get("batch", 1);
   int rc = launch_quantize_q8_1(P<void>(s[0]), DT_BF16, k.scratch, K, batch);
@@ -120,10 +135,16 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   if (swiglu) {
     float* g = (float*)((uint8_t*)k.scratch + (size_t)batch * (K / 32) * 36);
     float* u = g + (size_t)batch * N[0];
-    if ((rc = matmul_q8_1(W[0], xq, g, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
-    if ((rc = matmul_q8_1(W[1], xq, u, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
+    if (batch >= GEMM_MFMA_MIN_BATCH) {
+      void* gu[2] = {g, u}; const void* nores[2] = {nullptr, nullptr}; const int n2[2] = {N[0], N[0]}, e2[2] = {0, 0};
+      if ((rc = matmul_group_mfma(xq, K, batch, 2, W, gu, nores, n2, e2))) return rc;
+    } else {
+      if ((rc = matmul_q8_1(W[0], xq, g, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
+      if ((rc = matmul_q8_1(W[1], xq, u, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
+    }
     return launch_elementwise(EW_SWIGLU_OP, g, u, out[0], (int64_t)batch * N[0]);
   }
+  if (batch >= GEMM_MFMA_MIN_BATCH) return matmul_group_mfma(xq, K, batch, G, W, out, res, N, epi);
   for (int i = 0; i < G; i++)
     if ((rc = matmul_q8_1(W[i], xq, out[i], N[i], K, batch, epi[i] == 0 ? DT_F32 : DT_BF16, res[i], -1))) return rc;
   return BK_OK;

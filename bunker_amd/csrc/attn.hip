@@ -26,6 +26,8 @@ namespace bk {
 constexpr int ATT_HD = 256;
 constexpr int ATT_PAGE = 16;
 constexpr int ATT_WAVES = 4;
+constexpr int ATT_MAX_PPS = 1024;     // pages per split (the split's page table is staged in LDS)
+constexpr int ATT_MAX_SPLITS = 256;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
@@ -51,9 +53,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
 }
 
+// PF = pages a wave requests ahead of the one it computes on (0 or 2).  Loads are issued
+// unconditionally (past its last page a wave re-requests that page), so the number of loads in
+// flight at every wait is known when the kernel is compiled and a wait covers only the page needed.
+template <int PF>
 __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A) {
-  __shared__ float lds_o[ATT_HD][16];           // merged O^T, 16 KiB
+  __shared__ float lds_o2[2][ATT_HD][16];       // exchange buffers for the merge of the four waves, 2 x 16 KiB
   __shared__ float lds_m[ATT_WAVES][16], lds_l[ATT_WAVES][16];
+  __shared__ int lds_bt[ATT_MAX_PPS];           // physical page of every page of this split
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -78,20 +85,24 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   float m_run = -INFINITY;     // running max of head n (same in the 4 lanes that share n)
   float l_run = 0.0f;          // this lane's share of the running sum (tokens 4*kg .. 4*kg+3 of every page)
 
-  for (int pg = p_begin + wave; pg < p_end; pg += ATT_WAVES) {
-    const int phys = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + pg] : b * A.bt_stride + pg;
+  // The page table of the split is read once, into LDS: a table lookup in front of every page would
+  // put a dependent global load (and a wait for everything in flight) between the page requests.
+  for (int i = threadIdx.x; i < p_end - p_begin; i += ATT_WAVES * 64)
+    lds_bt[i] = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + p_begin + i] : b * A.bt_stride + p_begin + i;
+  __syncthreads();
+  auto load_page = [&](int pg, uint4 (&kr)[8], uint2 (&vr)[16]) {
+    const int phys = lds_bt[pg - p_begin];
     const int64_t base = ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
     // K page as the A operand: lane (token n, group kg) holds dims 32*s + 8*kg .. +8
     const uint16_t* kp = A.kc + base + n * ATT_HD + 8 * kg;
-    uint4 kreg[8];
 #pragma unroll
-    for (int s = 0; s < 8; s++) kreg[s] = *(const uint4*)(kp + 32 * s);
+    for (int s = 0; s < 8; s++) kr[s] = *(const uint4*)(kp + 32 * s);
     // V page as the A operand: lane (dim 16*t + n, group kg) holds tokens 4*kg .. +4
     const uint16_t* vp = A.vc + base + n * ATT_PAGE + 4 * kg;
-    uint2 vreg[16];
 #pragma unroll
-    for (int t = 0; t < 16; t++) vreg[t] = *(const uint2*)(vp + t * 16 * ATT_PAGE);
-
+    for (int t = 0; t < 16; t++) vr[t] = *(const uint2*)(vp + t * 16 * ATT_PAGE);
+  };
+  auto compute_page = [&](const uint4 (&kreg)[8], const uint2 (&vreg)[16], int pg) {
     f32x4_t s4 = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 8; s++)
@@ -134,9 +145,31 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
       oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pl),
                                                           oacc[t], 0, 0, 0);
     }
+  };
+
+  {
+    int pg = p_begin + wave;
+    if (PF == 0) {
+      for (; pg < p_end; pg += ATT_WAVES) {
+        uint4 kr[8]; uint2 vr[16];
+        load_page(pg, kr, vr);
+        compute_page(kr, vr, pg);
+      }
+    } else if (pg < p_end) {
+      const int last = pg + ((p_end - 1 - pg) / ATT_WAVES) * ATT_WAVES;      // this wave's last page
+      uint4 k0[8], k1[8], k2[8];
+      uint2 v0[16], v1[16], v2[16];
+      load_page(pg, k0, v0);
+      load_page(min(pg + ATT_WAVES, last), k1, v1);
+      while (true) {
+        load_page(min(pg + 2 * ATT_WAVES, last), k2, v2); compute_page(k0, v0, pg); pg += ATT_WAVES; if (pg > last) break;
+        load_page(min(pg + 2 * ATT_WAVES, last), k0, v0); compute_page(k1, v1, pg); pg += ATT_WAVES; if (pg > last) break;
+        load_page(min(pg + 2 * ATT_WAVES, last), k1, v1); compute_page(k2, v2, pg); pg += ATT_WAVES; if (pg > last) break;
+      }
+    }
   }
 
-  // ---- merge the four waves (fixed order 0,1,2,3)
+  // ---- merge the four waves as (0 + 1) + (2 + 3): two exchange rounds through LDS, a third for the transposed write
   float l_tot = l_run + __shfl_xor(l_run, 16);
   l_tot += __shfl_xor(l_tot, 32);
   if (kg == 0) { lds_m[wave][n] = m_run; lds_l[wave][n] = l_tot; }
@@ -151,19 +184,28 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
     const float mw = lds_m[w][n];
     L += (mw == -INFINITY) ? 0.0f : lds_l[w][n] * __expf(mw - M);
   }
-  for (int w = 0; w < ATT_WAVES; w++) {
-    if (wave == w) {
 #pragma unroll
-      for (int t = 0; t < 16; t++)
+  for (int t = 0; t < 16; t++) { oacc[t][0] *= wscale; oacc[t][1] *= wscale; oacc[t][2] *= wscale; oacc[t][3] *= wscale; }
+  auto put = [&](int buf) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          float* dst = &lds_o[16 * t + 4 * kg + r][n];
-          const float v = oacc[t][r] * wscale;
-          *dst = (w == 0) ? v : (*dst + v);
-        }
-    }
-    __syncthreads();
-  }
+    for (int t = 0; t < 16; t++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) lds_o2[buf][16 * t + 4 * kg + r][n] = oacc[t][r];
+  };
+  auto add = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < 16; t++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) oacc[t][r] += lds_o2[buf][16 * t + 4 * kg + r][n];
+  };
+  if (wave & 1) put(wave >> 1);           // waves 1 and 3 hand over
+  __syncthreads();
+  if (!(wave & 1)) add(wave >> 1);        // 0 += 1 (buffer 0), 2 += 3 (buffer 1)
+  if (wave == 2) put(1);                  // buffer 1 was read by wave 2 alone, so it can take the sum straight away
+  __syncthreads();
+  if (wave == 0) { add(1); put(0); }      // (0 + 1) + (2 + 3), then out for the transposed write (buffer 0: wave 0 was its only reader)
+  __syncthreads();
+  const float (*lds_o)[16] = lds_o2[0];
 
   // ---- write: thread = dim, loop over the G heads of the group
   const int d = threadIdx.x;   // 0..255
@@ -197,22 +239,39 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   }
 }
 
-// Merge of the split partials: one workgroup per (head, batch), thread = dim.
+// Merge of the split partials: one workgroup per (head, batch), thread = dim.  The weights
+// exp(m_s - M) of all splits are computed side by side first (thread = split) and kept in LDS, so the
+// loop over the partial outputs has nothing but independent loads in it.
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
+  __shared__ float wsh[ATT_MAX_SPLITS];
+  __shared__ float redm[4], redl[4];
   const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const int kvh = head / A.G, h = head % A.G;
   const int64_t p0 = ((int64_t)b * A.NKV + kvh) * A.splits;
-  float M = -INFINITY;
-  for (int s = 0; s < A.splits; s++) M = fmaxf(M, A.part_ml[((p0 + s) * 16 + h) * 2]);
-  float L = 0.0f, o = 0.0f;
-  for (int s = 0; s < A.splits; s++) {
-    const float ms = A.part_ml[((p0 + s) * 16 + h) * 2];
-    if (ms == -INFINITY) continue;
-    const float w = __expf(ms - M);
-    L += A.part_ml[((p0 + s) * 16 + h) * 2 + 1] * w;
-    o += A.part_o[((p0 + s) * 16 + h) * ATT_HD + d] * w;
+  const bool has = d < A.splits;
+  const float ms = has ? A.part_ml[((p0 + d) * 16 + h) * 2] : -INFINITY;
+  const float ls = has ? A.part_ml[((p0 + d) * 16 + h) * 2 + 1] : 0.0f;
+  float M = wave_max(ms);
+  if ((d & 63) == 0) redm[d >> 6] = M;
+  __syncthreads();
+  M = fmaxf(fmaxf(redm[0], redm[1]), fmaxf(redm[2], redm[3]));
+  const float w = (ms == -INFINITY) ? 0.0f : __expf(ms - M);
+  wsh[d] = w;
+  float L = wave_sum(ls * w);
+  if ((d & 63) == 0) redl[d >> 6] = L;
+  __syncthreads();
+  L = (redl[0] + redl[1]) + (redl[2] + redl[3]);
+  const float* po = A.part_o + (p0 * 16 + h) * ATT_HD + d;
+  float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+  int s = 0;
+  for (; s + 4 <= A.splits; s += 4) {
+    o0 = fmaf(po[(int64_t)(s + 0) * 16 * ATT_HD], wsh[s + 0], o0);
+    o1 = fmaf(po[(int64_t)(s + 1) * 16 * ATT_HD], wsh[s + 1], o1);
+    o2 = fmaf(po[(int64_t)(s + 2) * 16 * ATT_HD], wsh[s + 2], o2);
+    o3 = fmaf(po[(int64_t)(s + 3) * 16 * ATT_HD], wsh[s + 3], o3);
   }
-  o = o / L;
+  for (; s < A.splits; s++) o0 = fmaf(po[(int64_t)s * 16 * ATT_HD], wsh[s], o0);
+  float o = ((o0 + o1) + (o2 + o3)) / L;
   if (A.gate) {
     const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
     o = __fmul_rn(o, sigmoid_f64(gv));
@@ -227,11 +286,11 @@ size_t attn_workspace_bytes(int batch, int NKV, int max_splits) {
 
 int attn_choose_splits(int batch, int NKV, int max_ctx) {
   const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
-  // aim at ~4 workgroups per CU, but keep at least 8 pages (2 per wave) in a split
+  // aim at ~4 workgroups per CU, but keep at least one page per wave in a split
   int want = (4 * num_cus() + batch * NKV - 1) / (batch * NKV);
-  int cap = (pages + 7) / 8;
+  int cap = (pages + ATT_WAVES - 1) / ATT_WAVES;
   int s = want < cap ? want : cap;
-  return s < 1 ? 1 : (s > 256 ? 256 : s);
+  return s < 1 ? 1 : (s > ATT_MAX_SPLITS ? ATT_MAX_SPLITS : s);
 }
 
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
@@ -249,6 +308,8 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   if (splits <= 0) splits = attn_choose_splits(batch, NKV, max_ctx);
   const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
   if (splits > pages) splits = pages;
+  BK_REQUIRE(splits <= ATT_MAX_SPLITS, "attn_decode: at most %d splits", ATT_MAX_SPLITS);
+  BK_REQUIRE((pages + splits - 1) / splits <= ATT_MAX_PPS, "attn_decode: %d pages in %d splits exceed %d pages per split", pages, splits, ATT_MAX_PPS);
   AttnArgs A{};
   A.q = (const uint16_t*)q; A.kc = (const uint16_t*)kc; A.vc = (const uint16_t*)vc;
   A.block_table = block_table; A.ctx_len = ctx_len; A.gate = (const uint16_t*)gate;
@@ -263,7 +324,11 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
     A.part_o = (float*)workspace;
     A.part_ml = A.part_o + (size_t)batch * NKV * splits * 16 * ATT_HD;
   }
-  hipLaunchKernelGGL(attn_decode_kernel, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
+  // waves with three pages or more keep two pages in flight ahead of the one they work on
+  if (A.pages_per_split >= 3 * ATT_WAVES)
+    hipLaunchKernelGGL(attn_decode_kernel<2>, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
+  else
+    hipLaunchKernelGGL(attn_decode_kernel<0>, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
   if (splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, batch), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;

@@ -26,16 +26,38 @@ enum : int { GEPI_F32 = 0, GEPI_BF16 = 1, GEPI_BF16_ADD = 2 };
 // rows of the 32x32 accumulator held by a lane: r = 0..15 -> 8*(r/4) + 4*(lane/32) + r%4
 __device__ __forceinline__ int mfma32_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
 
-template <int EPI, int NW>
-__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq,
-                                                                     void* __restrict__ out, const uint16_t* __restrict__ res,
-                                                                     int N, int nb, int B) {
+// Up to four matrices that share the activation rows run as one launch: their 32-row tiles are laid end to end.
+struct MfmaGroup {
+  const uint8_t* W;
+  void* out;
+  const uint16_t* res;
+  int N, epi;
+};
+struct MfmaArgs {
+  MfmaGroup g[4];
+  int tile_first[5];      // first tile of each matrix; tile_first[i >= ngroups] = number of tiles
+  const uint8_t* xq;
+  int nb, B;
+};
+
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
   __shared__ double lds_d8[NW][8][32], lds_s8[NW][8][32];
   __shared__ double lds_acc[NW > 1 ? 16 * 64 : 1];
 
+  const int tile = blockIdx.x;
+  const bool s1 = tile >= A.tile_first[1], s2 = tile >= A.tile_first[2], s3 = tile >= A.tile_first[3];
+  const uint8_t* __restrict__ W = s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
+  void* __restrict__ out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
+  const uint16_t* __restrict__ res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
+  const int N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
+  const int EPI = s3 ? A.g[3].epi : s2 ? A.g[2].epi : s1 ? A.g[1].epi : A.g[0].epi;
+  const uint8_t* __restrict__ xq = A.xq;
+  const int nb = A.nb, B = A.B;
+
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const int n0 = blockIdx.x * 32;
+  const int n0 = (tile - (s3 ? A.tile_first[3] : s2 ? A.tile_first[2] : s1 ? A.tile_first[1] : 0)) * 32;
   const int n = min(n0 + col, N - 1);                 // rows past N recompute row N-1 and are not stored
   const uint8_t* wrow = W + (int64_t)n * nb * 144;
   const int64_t xrow_bytes = (int64_t)nb * 8 * 36;
@@ -146,40 +168,47 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(const uint8
 
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
 
-template <int NW>
-static void launch_gemm_nw(int epi, dim3 grid, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int nb, int batch) {
-  const dim3 block(64 * NW);
-  if (epi == GEPI_F32) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_F32, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
-  else if (epi == GEPI_BF16) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<GEPI_BF16_ADD, NW>), grid, block, 0, stream(), w, x, y, r, N, nb, batch);
+int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
+                           const void* const* res, const int* N, const int* epi) {
+  BK_REQUIRE(xq && ngroups >= 1 && ngroups <= 4, "gemm_q4k_q8_1_mfma: bad arguments");
+  BK_REQUIRE(K > 0 && K % 256 == 0, "gemm_q4k_q8_1_mfma: K=%d must be a positive multiple of 256", K);
+  BK_REQUIRE(batch >= 1 && batch <= 32, "gemm_q4k_q8_1_mfma: batch=%d must be 1..32", batch);
+  BK_REQUIRE(((uintptr_t)xq & 3) == 0, "gemm_q4k_q8_1_mfma: xq must be 4-byte aligned");
+  MfmaArgs A{};
+  A.xq = (const uint8_t*)xq; A.nb = K / 256; A.B = batch;
+  int tiles = 0;
+  for (int i = 0; i < ngroups; i++) {
+    BK_REQUIRE(W[i] && out[i] && N[i] > 0 && ((uintptr_t)W[i] & 15) == 0, "gemm_q4k_q8_1_mfma: matrix %d: null, misaligned or N <= 0", i);
+    BK_REQUIRE(epi[i] == GEPI_F32 || epi[i] == GEPI_BF16 || epi[i] == GEPI_BF16_ADD, "gemm_q4k_q8_1_mfma: bad epilogue %d", epi[i]);
+    BK_REQUIRE(epi[i] != GEPI_BF16_ADD || res[i], "gemm_q4k_q8_1_mfma: the add epilogue needs a residual");
+    A.g[i].W = (const uint8_t*)W[i]; A.g[i].out = out[i]; A.g[i].res = (const uint16_t*)res[i]; A.g[i].N = N[i]; A.g[i].epi = epi[i];
+    A.tile_first[i] = tiles;
+    tiles += (N[i] + 31) / 32;
+  }
+  for (int i = ngroups; i < 5; i++) A.tile_first[i] = tiles;
+  // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
+  // and two ways when the tiles alone fill the chip many times over (lm_head)
+  int nw = g_tune_gemm_nw;
+  if (nw <= 0) {
+    nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
+    if (tiles >= 8 * num_cus() && nw > 2) nw = 2;
+  }
+  const dim3 grid(tiles);
+  if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8>), grid, dim3(512), 0, stream(), A);
+  else if (nw >= 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4>), grid, dim3(256), 0, stream(), A);
+  else if (nw >= 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2>), grid, dim3(128), 0, stream(), A);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1>), grid, dim3(64), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
 }
 
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
                               const void* residual) {
   BK_REQUIRE(W && xq && y, "gemm_q4k_q8_1_mfma: null pointer");
-  BK_REQUIRE(N > 0 && K > 0 && K % 256 == 0, "gemm_q4k_q8_1_mfma: K=%d must be a positive multiple of 256 (N=%d)", K, N);
-  BK_REQUIRE(batch >= 1 && batch <= 32, "gemm_q4k_q8_1_mfma: batch=%d must be 1..32", batch);
   BK_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gemm_q4k_q8_1_mfma: out_dtype must be 0 (f32) or 1 (bf16)");
   BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemm_q4k_q8_1_mfma: a residual needs bf16 output");
-  BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "gemm_q4k_q8_1_mfma: W must be 16-byte and xq 4-byte aligned");
-  const dim3 grid((N + 31) / 32);
-  const uint8_t* w = (const uint8_t*)W; const uint8_t* x = (const uint8_t*)xq; const uint16_t* r = (const uint16_t*)residual;
-  const int nb = K / 256;
   const int epi = out_dtype == DT_F32 ? GEPI_F32 : (residual ? GEPI_BF16_ADD : GEPI_BF16);
-  // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
-  // and two ways when the tiles alone fill the chip many times over (lm_head)
-  int nw = g_tune_gemm_nw;
-  if (nw <= 0) {
-    const int tiles = (N + 31) / 32;
-    nw = nb >= 16 ? 8 : (nb >= 4 ? 4 : (nb >= 2 ? 2 : 1));
-    if (tiles >= 8 * num_cus() && nw > 2) nw = 2;
-  }
-  if (nw >= 8) launch_gemm_nw<8>(epi, grid, w, x, y, r, N, nb, batch);
-  else if (nw >= 4) launch_gemm_nw<4>(epi, grid, w, x, y, r, N, nb, batch);
-  else if (nw >= 2) launch_gemm_nw<2>(epi, grid, w, x, y, r, N, nb, batch);
-  else launch_gemm_nw<1>(epi, grid, w, x, y, r, N, nb, batch);
-  BK_LAUNCH_CHECK();
-  return BK_OK;
+  return launch_gemm_group_mfma(xq, K, batch, 1, &W, &y, &residual, &N, &epi);
 }
 
 }  // namespace bk

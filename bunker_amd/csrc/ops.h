@@ -42,6 +42,8 @@ int launch_gemv_swiglu_q8(const void* Wg, const void* Wu, const void* xq, void* 
 
 // gemm_mfma.hip
 extern int g_tune_gemm_nw;
+int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
+                           const void* const* res, const int* N, const int* epi);
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
                               const void* residual);
 
