@@ -152,10 +152,26 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
   return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 
+// Q8_1 rounding of one value: q = floor(fl64(f / d) + 0.5) with d = fl64(amax / 127) (bench/bench.ts:53-72,
+// ECMAScript Math.round).  The quotient is first formed in f32 (t = f * (127 / amax), off by at most 3e-5 from
+// the double quotient); only when t + 0.5 lies within 1e-3 of an integer — where the two could round
+// differently — is the double division carried out.  Both paths return the reference's integer.
+__device__ __forceinline__ int q8_1_round(float f, float inv, double div) {
+  const float u = f * inv + 0.5f;
+  const float fl = floorf(u);
+  const float nr = rintf(u);
+  if (fabsf(u - nr) < 1e-3f) {               // rare: decided by the double quotient
+    const double qd = (double)f / div;
+    double r = floor(qd);
+    if (qd - r >= 0.5) r += 1.0;
+    return (int)r;
+  }
+  return (int)fl;
+}
+
 // Q8_1 of one 32-element block held by four consecutive lanes (8 values each, already rounded to
-// the activation's storage type).  bench/bench.ts:53-72: d = amax/127 and the quotient in double,
-// round half toward +infinity, s = trunc16(float(sum(q) * d)) with the unrounded d.  Returns the
-// lane's 8 int8 in pk[0..1] and the packed (d, s) halves, the same in all four lanes.
+// the activation's storage type).  d = amax/127 in double, s = trunc16(float(sum(q) * d)) with the
+// unrounded d.  Returns the lane's 8 int8 in pk[0..1] and the packed (d, s) halves, the same in all four lanes.
 __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk)[2]) {
   float amax = 0.0f;
 #pragma unroll
@@ -163,14 +179,12 @@ __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk
   amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
   amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
   const double d = (double)amax / 127.0, div = d != 0.0 ? d : 1.0;
+  const float inv = amax != 0.0f ? 127.0f / amax : 0.0f;      // amax = 0: every value is 0 and so is every q
   int sum = 0;
   pk[0] = 0; pk[1] = 0;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
-    const double qd = (double)f[j] / div;
-    double r = floor(qd);
-    if (qd - r >= 0.5) r += 1.0;
-    int q = (int)r;
+    int q = q8_1_round(f[j], inv, div);
     sum += q;
     q = q < -128 ? -128 : (q > 127 ? 127 : q);
     pk[j >> 2] |= (uint32_t)(q & 0xff) << (8 * (j & 3));

@@ -89,12 +89,14 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_q4k_q8_1_lds_kernel(
   int row0 = wave * RPI;
   uint4* tile = tiles[wv];
 
-  StageRegs<NR, RPI> g;
-  if (row0 < N) stage_load<NR, RPI>(g, W, (int64_t)row0 * row_bytes, last_piece_off, lane);
-
+  // the activation slice first, the weight rows right behind it: loads return in issue order, and the slice
+  // (cache-resident) must not queue up behind rows that come from HBM
   XQ x[NR];
 #pragma unroll
   for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, true);
+
+  StageRegs<NR, RPI> g;
+  stage_load<NR, RPI>(g, W, (int64_t)min(row0, N - 1) * row_bytes, last_piece_off, lane);
 
   while (row0 < N) {
     stage_park<NR, RPI>(g, tile, lane);

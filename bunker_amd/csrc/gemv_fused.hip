@@ -6,7 +6,8 @@
 // pass, the sum of squares in double through the same block reduction as the stand-alone
 // RMSNorm kernel, the Q8_1 blocks by groups of four lanes.  The quantized row lives in LDS in
 // the Q8_1 byte layout; each lane then takes its slice into registers as the plain GEMV does.
-// The first weight loads are requested before the prologue, so its latency hides behind them.
+// The activation loads go out first and the first weight rows right behind them, so the prologue
+// runs while the weight rows are on their way.
 //
 // Rows.  As in the LDS-staged GEMV: a wave step fetches RPI contiguous rows with coalesced
 // 16-byte loads, parks them in the wave's LDS tile and reads them back in the (block, chunk)
@@ -57,16 +58,34 @@ __device__ __forceinline__ StepSel select_step(const FusedArgs& A, int s) {
   return r;
 }
 
-// ---- prologue: activation row -> Q8_1 in LDS (36-byte blocks)
-template <int PRO>
-__device__ __forceinline__ void stage_activation(const uint16_t* __restrict__ xr, const uint16_t* __restrict__ w, int K,
-                                                 uint8_t* lds_xq, double* lds_red) {
+// ---- prologue: activation row -> Q8_1 in LDS (36-byte blocks).  K = 2048 * NR: NR passes of 256 threads x 8 elements.
+// Everything the prologue reads from memory (the row and, for RMSNorm, the norm weight) is requested up front.
+// Loads return to a wave in the order they were issued, so these go out BEFORE the weight rows: the prologue then
+// waits for a few small, cache-resident loads only and runs while the weight rows are still on their way.
+template <int NR>
+struct ActRegs {
+  uint4 xv[NR], wv[NR];
+};
+template <int PRO, int NR>
+__device__ __forceinline__ void act_load(ActRegs<NR>& r, const uint16_t* __restrict__ xr, const uint16_t* __restrict__ w) {
+#pragma unroll
+  for (int p = 0; p < NR; p++) {
+    const int i = threadIdx.x * 8 + p * 2048;
+    r.xv[p] = *(const uint4*)(xr + i);
+    if (PRO == PRO_RMSNORM) r.wv[p] = *(const uint4*)(w + i);
+  }
+}
+template <int PRO, int NR>
+__device__ __forceinline__ void stage_activation(const ActRegs<NR>& regs, uint8_t* lds_xq, double* lds_red) {
+  constexpr int K = NR * 2048;
+  const uint4 (&xv)[NR] = regs.xv;
+  const uint4 (&wv)[NR] = regs.wv;
   float rstd = 0.0f;
   if (PRO == PRO_RMSNORM) {
     double ss = 0.0;
-    for (int i = threadIdx.x * 8; i < K; i += 256 * 8) {
-      const uint4 v = *(const uint4*)(xr + i);
-      const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int p = 0; p < NR; p++) {
+      const uint32_t u[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
@@ -76,13 +95,13 @@ __device__ __forceinline__ void stage_activation(const uint16_t* __restrict__ xr
     ss = block_sum_f64<4>(ss, lds_red);
     rstd = rsqrt_f64(ss / (double)K + 1e-6);
   }
-  for (int i = threadIdx.x * 8; i < K; i += 256 * 8) {
-    const uint4 v = *(const uint4*)(xr + i);
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int p = 0; p < NR; p++) {
+    const int i = threadIdx.x * 8 + p * 2048;
+    const uint32_t u[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w};
     float f[8];
     if (PRO == PRO_RMSNORM) {
-      const uint4 wv = *(const uint4*)(w + i);
-      const uint32_t uw[4] = {wv.x, wv.y, wv.z, wv.w};
+      const uint32_t uw[4] = {wv[p].x, wv[p].y, wv[p].z, wv[p].w};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
@@ -118,13 +137,13 @@ __device__ __forceinline__ void fused_stage_load(StageRegs<NR, RPI>& g, const ui
   const int64_t base = (int64_t)row0 * row_bytes;
 #pragma unroll
   for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
-    const int piece = lane + 64 * u;
-    if (piece < PIECES) {
-      const bool second = SWIGLU && piece >= PIECES / 2;
-      const int64_t off = base + (int64_t)(second ? piece - PIECES / 2 : piece) * 16;
-      const uint8_t* W = second ? W1 : W0;
-      g.v[u] = load_w16(W + (off < last ? off : last));     // past the matrix: re-read its last piece
-    }
+    // every lane loads in every round (lanes past the tile re-request its last piece): the number of loads in
+    // flight is then known at compile time and waits can be counted instead of draining the queue
+    const int piece = min(lane + 64 * u, PIECES - 1);
+    const bool second = SWIGLU && piece >= PIECES / 2;
+    const int64_t off = base + (int64_t)(second ? piece - PIECES / 2 : piece) * 16;
+    const uint8_t* W = second ? W1 : W0;
+    g.v[u] = load_w16(W + (off < last ? off : last));       // past the matrix: re-read its last piece
   }
 }
 
@@ -147,10 +166,15 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
   const int total = A.step_first[4];
   uint4* tile = tiles[wv];
 
+  ActRegs<NR> act;
+  if (PRO != PRO_Q8) act_load<PRO, NR>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
+
   int s = blockIdx.x * GEMV_WAVES + wv;
   StepSel cur = select_step<ROWS_PER_STEP>(A, s < total ? s : 0);
   StageRegs<NR, RPI> g;
-  if (s < total) fused_stage_load<NR, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
+  // unconditional (a wave without a step of its own requests step 0): with a branch around these loads the
+  // prologue's first wait could not be counted and would drain the weight rows as well
+  fused_stage_load<NR, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
 
   XQ x[NR];
   if (PRO == PRO_Q8) {
@@ -158,7 +182,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
 #pragma unroll
     for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, true);
   } else {
-    stage_activation<PRO>((const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w, K, lds_xq, lds_red);
+    stage_activation<PRO, NR>(act, lds_xq, lds_red);
 #pragma unroll
     for (int r = 0; r < NR; r++) load_xq(x[r], lds_xq, r * 8 + b, c, true);
   }

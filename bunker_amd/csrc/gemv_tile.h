@@ -227,11 +227,11 @@ __device__ __forceinline__ void stage_load(StageRegs<NR, RPI>& g, const uint8_t*
                                            int64_t last_piece_off, int lane) {
 #pragma unroll
   for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
-    const int piece = lane + 64 * u;
-    if (piece < StageRegs<NR, RPI>::PIECES) {
-      const int64_t off = tile_off + (int64_t)piece * 16;
-      g.v[u] = load_w16(W + (off < last_piece_off ? off : last_piece_off));   // past the matrix: re-read its last piece
-    }
+    // every lane loads in every round (lanes past the tile re-request its last piece), so that the number of
+    // loads in flight is known at compile time
+    const int piece = min(lane + 64 * u, StageRegs<NR, RPI>::PIECES - 1);
+    const int64_t off = tile_off + (int64_t)piece * 16;
+    g.v[u] = load_w16(W + (off < last_piece_off ? off : last_piece_off));   // past the matrix: re-read its last piece
   }
 }
 
