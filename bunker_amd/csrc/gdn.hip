@@ -45,19 +45,28 @@ struct GdnArgs {
   int C;
 };
 
-// One channel of conv1d_decode: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); returns bf16(r * sigmoid(r)) and
-// writes the state rows (s1, s2, x).  The thread that reads a channel's rows is the one that rewrites them.
-__device__ __forceinline__ uint16_t conv_channel(const GdnArgs& A, int b, int ch, uint16_t xbits) {
+// One channel of conv1d_decode: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); out = bf16(r * sigmoid(r)), new state rows
+// (s1, s2, x).  Loading and computing are separate so that a kernel can request everything it needs first.
+struct ConvIn {
+  uint16_t x, s0, s1, s2;
+  uint2 w;
+};
+__device__ __forceinline__ ConvIn conv_load(const GdnArgs& A, int b, int ch, const uint16_t* xrow) {
   const uint16_t* sb = A.conv_st + (int64_t)b * 3 * A.C;
-  const uint16_t s0 = sb[ch], s1 = sb[A.C + ch], s2 = sb[2 * A.C + ch];
-  const uint2 wv = *(const uint2*)(A.conv_w + 4 * (int64_t)ch);
-  const float w0 = __uint_as_float(wv.x << 16), w1 = __uint_as_float(wv.x & 0xffff0000u);
-  const float w2 = __uint_as_float(wv.y << 16), w3 = __uint_as_float(wv.y & 0xffff0000u);
+  ConvIn c;
+  c.x = xrow[ch]; c.s0 = sb[ch]; c.s1 = sb[A.C + ch]; c.s2 = sb[2 * A.C + ch];
+  c.w = *(const uint2*)(A.conv_w + 4 * (int64_t)ch);
+  return c;
+}
+// The thread that read a channel's rows is the one that rewrites them, so the state may be updated in place.
+__device__ __forceinline__ uint16_t conv_apply(const GdnArgs& A, int b, int ch, const ConvIn& c) {
+  const float w0 = __uint_as_float(c.w.x << 16), w1 = __uint_as_float(c.w.x & 0xffff0000u);
+  const float w2 = __uint_as_float(c.w.y << 16), w3 = __uint_as_float(c.w.y & 0xffff0000u);
   // products of two bf16 values are exact in f32
-  const float r = __fadd_rn(__fadd_rn(w0 * bf16_to_f32(s0), w1 * bf16_to_f32(s1)),
-                            __fadd_rn(w2 * bf16_to_f32(s2), w3 * bf16_to_f32(xbits)));
+  const float r = __fadd_rn(__fadd_rn(w0 * bf16_to_f32(c.s0), w1 * bf16_to_f32(c.s1)),
+                            __fadd_rn(w2 * bf16_to_f32(c.s2), w3 * bf16_to_f32(c.x)));
   uint16_t* nb = A.conv_st_new + (int64_t)b * 3 * A.C;
-  nb[ch] = s1; nb[A.C + ch] = s2; nb[2 * A.C + ch] = xbits;
+  nb[ch] = c.s1; nb[A.C + ch] = c.s2; nb[2 * A.C + ch] = c.x;
   return f32_to_bf16(__fmul_rn(r, sigmoid_f64(r)));
 }
 
@@ -80,26 +89,48 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   const int col0 = slab * COLS + vq * 4;    // first of the thread's 4 columns (within the head)
   const int64_t bh = (int64_t)b * A.Hg + h;
 
-  // S rows go out first: the loads are in flight while q, k and the gates are prepared
+  const uint16_t* qp = A.q + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* kp = A.k + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* vp = A.v + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* xrow = A.q + (int64_t)b * A.qkv_bstride;
+  const bool isk = tid >= 128;              // fused mode: threads 0..127 hold q, 128..255 hold k
+  const int i = tid & 127;
+
+  // Loads come back in the order they were issued.  The small operands (q, k, v, the conv taps and state, the gate
+  // inputs) are requested first and the 64 KiB of S right behind them: the norms and gates are then computed while
+  // S is still on its way from HBM.
+  ConvIn cqk{}, cv{};
+  uint16_t xbits = 0;
+  uint2 vv_g = make_uint2(0, 0);
+  float zin = 0.0f, nw = 0.0f, ap = 0.0f, bp = 0.0f, alog = 0.0f, dtb = 0.0f;
+  const int ch_qk = (int)((isk ? kp : qp) - xrow) + i, ch_v = (int)(vp - xrow) + i;
+  if (FUSED) {
+    if (CONV) {
+      cqk = conv_load(A, b, ch_qk, xrow);
+      cv = conv_load(A, b, ch_v, xrow);      // every thread loads (no branch around loads: waits stay countable); q threads use it
+    } else {
+      xbits = (isk ? kp : qp)[i];
+    }
+    ap = A.a_p[bh]; bp = A.b_p[bh]; alog = A.A_log[h]; dtb = bf16_to_f32(A.dt_bias[h]);
+    zin = bf16_to_f32(A.z[bh * GDN_D + i]); nw = A.norm_w[i];
+  } else {
+    xbits = tid < 128 ? qp[tid] : kp[tid - 128];
+  }
+  if (!CONV) vv_g = *(const uint2*)(vp + col0);
+
   const float* Sp = A.S_in + bh * GDN_D * GDN_D;
   float4 S[ROWS];
 #pragma unroll
   for (int r = 0; r < ROWS; r++) S[r] = *(const float4*)(Sp + (int64_t)(kg * ROWS + r) * GDN_D + col0);
 
-  const uint16_t* qp = A.q + (int64_t)b * A.qkv_bstride + h * GDN_D;
-  const uint16_t* kp = A.k + (int64_t)b * A.qkv_bstride + h * GDN_D;
-  const uint16_t* vp = A.v + (int64_t)b * A.qkv_bstride + h * GDN_D;
   float decay, beta;
   if (FUSED) {
-    // threads 0..127 hold q, 128..255 hold k
-    const bool isk = tid >= 128;
-    const int i = tid & 127;
     float x;
     if (CONV) {
-      x = bf16_to_f32(conv_channel(A, b, (int)((isk ? kp : qp) - (A.q + (int64_t)b * A.qkv_bstride)) + i, (isk ? kp : qp)[i]));
-      if (!isk) vsh[i] = conv_channel(A, b, (int)(vp - (A.q + (int64_t)b * A.qkv_bstride)) + i, vp[i]);
+      x = bf16_to_f32(conv_apply(A, b, ch_qk, cqk));
+      if (!isk) vsh[i] = conv_apply(A, b, ch_v, cv);
     } else {
-      x = bf16_to_f32((isk ? kp : qp)[i]);
+      x = bf16_to_f32(xbits);
     }
     const double ss = wave_sum_f64((double)(x * x));       // square of a bf16 value: exact in f32
     if ((tid & 63) == 0) red[tid >> 6] = ss;
@@ -108,13 +139,13 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     const float rs = rsqrt_f64(tot + 1e-6);
     if (isk) kn[i] = x * rs;
     else qn[i] = x * (rs * 0.08838834764831845f);     // 1/sqrt(128)
-    const float sp_in = A.a_p[bh] + bf16_to_f32(A.dt_bias[h]);
+    const float sp_in = ap + dtb;
     const float softplus = (float)log1p(exp((double)sp_in));
-    decay = (float)exp(-(double)((float)exp((double)A.A_log[h]) * softplus));
-    beta = sigmoid_f64(A.b_p[bh]);
+    decay = (float)exp(-(double)((float)exp((double)alog) * softplus));
+    beta = sigmoid_f64(bp);
   } else {
-    if (tid < 128) qn[tid] = bf16_to_f32(qp[tid]);
-    else kn[tid - 128] = bf16_to_f32(kp[tid - 128]);
+    if (tid < 128) qn[tid] = bf16_to_f32(xbits);
+    else kn[tid - 128] = bf16_to_f32(xbits);
     decay = (float)exp((double)A.g[bh]);
     beta = A.beta[bh];
   }
@@ -141,7 +172,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     kS.x += p.x; kS.y += p.y; kS.z += p.z; kS.w += p.w;
   }
   __syncthreads();   // part is reused for o below
-  const uint2 vv = CONV ? *(const uint2*)(vsh + col0) : *(const uint2*)(vp + col0);
+  const uint2 vv = CONV ? *(const uint2*)(vsh + col0) : vv_g;
   float4 d;
   d.x = (__uint_as_float(vv.x << 16) - kS.x) * beta;
   d.y = (__uint_as_float(vv.x & 0xffff0000u) - kS.y) * beta;
@@ -178,9 +209,8 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   __syncthreads();
   if (tid < GDN_D) {
     const float orstd = rsqrt_f64((red[0] + red[1]) / (double)GDN_D + 1e-6);
-    const float zv = bf16_to_f32(A.z[bh * GDN_D + tid]);
-    const float zs = zv * sigmoid_f64(zv);
-    outp[tid] = f32_to_bf16(((o * orstd) * A.norm_w[tid]) * zs);
+    const float zs = zin * sigmoid_f64(zin);
+    outp[tid] = f32_to_bf16(((o * orstd) * nw) * zs);
   }
 }
 
