@@ -33,6 +33,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant GEMV kernel (average over its three shapes), from two rocprofv3 --pmc runs of
+# `bench.py --sections gemv,calib` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter
+# reads for memcopy_kernel of 175030272 bytes (FETCH_SIZE reads 0.50006 of the bytes: factor 1.99979; WRITE_SIZE factor 1.0).
+# The summary with the per-shape counters is profiles/gemv_q4k_q8_1_decode_shapes.md.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65724716
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
 ROTATION = 4            # weight sets; one set is 203 MB, so the rotation spans 813 MB
 
@@ -296,7 +301,7 @@ def main():
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": "gemv_q4k_q8_1_lds_kernel<1,0,4>", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": None}
+                "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH}
 
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak); synthetic Qwen3.5 decode tok/s at bs=1/32",

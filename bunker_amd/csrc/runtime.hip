@@ -115,7 +115,9 @@ int bk_device_info(char* buf, int cap) {
   BK_REQUIRE(buf && cap > 0, "bk_device_info: bad buffer");
   hipDeviceProp_t prop;
   BK_HIP(hipGetDeviceProperties(&prop, g_device));
-  snprintf(buf, cap, "%s|%s|%d|%zu", prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.totalGlobalMem);
+  // some driver stacks leave the marketing name empty: fall back to the architecture name
+  snprintf(buf, cap, "%s|%s|%d|%zu", prop.name[0] ? prop.name : prop.gcnArchName, prop.gcnArchName, prop.multiProcessorCount,
+           prop.totalGlobalMem);
   return BK_OK;
 }
 
