@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # `bench.py --sections gemv,calib` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter
 # reads for memcopy_kernel of 175030272 bytes (FETCH_SIZE reads 0.50006 of the bytes: factor 1.99979; WRITE_SIZE factor 1.0).
 # The summary with the per-shape counters is profiles/gemv_q4k_q8_1_decode_shapes.md.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65724716
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65721624
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
 ROTATION = 4            # weight sets; one set is 203 MB, so the rotation spans 813 MB
 
