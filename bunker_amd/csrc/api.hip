@@ -367,13 +367,13 @@ using namespace bk;
 
 extern "C" {
 
-// Tuning hook for experiments: "gemv_rpi" (1, 2, 4, 8), "gemv_cap" (workgroups per CU).
+// Tuning hooks for measurements: "gemv_impl" (0 direct loads, 2 rows through LDS), "gemv_rpi" (rows per wave step),
+// "gemv_cap" (workgroups per CU), "gemm_nw" (waves per MFMA tile), "memread_*" (calibration read kernel).
 int bk_tune_set(const char* key, int value) {
   BK_REQUIRE(key, "bk_tune_set: null key");
   if (!strcmp(key, "gemv_rpi")) bk::g_tune_rpi = value;
   else if (!strcmp(key, "gemv_cap")) bk::g_tune_cap = value;
   else if (!strcmp(key, "gemv_impl")) bk::g_tune_gemv_impl = value;
-  else if (!strcmp(key, "gemv_ks_rows")) bk::g_tune_ks_rows = value;
   else if (!strcmp(key, "gemm_nw")) bk::g_tune_gemm_nw = value;
   else if (!strcmp(key, "memread_unroll")) bk::g_tune_mr_unroll = value;
   else if (!strcmp(key, "memread_cap")) bk::g_tune_mr_cap = value;

@@ -185,8 +185,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
   }
 }
 
-int g_tune_gemv_impl = 2;               // 2: rows staged through LDS when K is a multiple of 2048 (else as 0), 1: eight-rows-per-wave
-                                        // layout (gemv8.hip), 0: direct loads in the (block, chunk) mapping
+int g_tune_gemv_impl = 2;               // 2: rows staged through LDS when K is a multiple of 2048 (else as 0),
+                                        // 0: direct loads in the (block, chunk) mapping
 int g_tune_rpi = 4, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows per wave step, workgroups per CU
 
 static int gemv_grid(int N, int rows_per_wg) {
@@ -239,11 +239,6 @@ int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, i
   BK_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gemv_q4k_q8_1: out_dtype must be 0 (f32) or 1 (bf16)");
   BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemv_q4k_q8_1: a residual needs bf16 output");
   BK_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)xq & 3) == 0, "gemv_q4k_q8_1: W must be 16-byte and xq 4-byte aligned");
-  if (g_tune_gemv_impl == 1) {
-    const int epi = out_dtype == DT_F32 ? 0 : (residual ? 2 : 1);
-    const void* Ws[1] = {W}; void* outs[1] = {y}; const void* rs[1] = {residual};
-    return launch_gemv_group(xq, K, batch, 1, Ws, outs, rs, &N, &epi);
-  }
   const int nb = K / 256;
   if (out_dtype == DT_F32) launch_q8_1_variant<EPI_F32>(W, xq, y, nullptr, N, nb, batch);
   else if (!residual) launch_q8_1_variant<EPI_BF16>(W, xq, y, nullptr, N, nb, batch);

@@ -24,7 +24,7 @@ int launch_memread(const void* src, int64_t bytes, void* sink);
 int launch_memcopy(const void* src, void* dst, int64_t bytes);
 
 // gemv.hip
-extern int g_tune_rpi, g_tune_cap, g_tune_mr_unroll, g_tune_mr_cap, g_tune_mr_nt, g_tune_gemv_impl, g_tune_ks_rows;
+extern int g_tune_rpi, g_tune_cap, g_tune_mr_unroll, g_tune_mr_cap, g_tune_mr_nt, g_tune_gemv_impl;
 int launch_gemv_q4k_f32(const void* W, const float* x, float* y, int N, int K);
 int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, int batch,
                          int out_dtype, const void* residual);
@@ -34,11 +34,6 @@ int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, in
 bool gemv_fused_fast_path(int K, int batch, bool swiglu);
 int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
                       void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
-
-// gemv8.hip
-int launch_gemv_group(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
-                      const void* const* res, const int* N, const int* epi);
-int launch_gemv_swiglu_q8(const void* Wg, const void* Wu, const void* xq, void* act, void* act_q8, int N, int K, int batch);
 
 // gemm_mfma.hip
 extern int g_tune_gemm_nw;

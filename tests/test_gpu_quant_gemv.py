@@ -147,6 +147,27 @@ def test_gemv_q4k_q8_1_decode_shapes(orc, dev, name):
     assert np.array_equal(rt.from_device(dy, (N,), np.float32).view(np.uint32), y.view(np.uint32))
 
 
+@pytest.mark.parametrize("N,K", [(1001, 2048), (515, 4096), (258, 6144)])
+def test_gemv_variants_return_the_same_bits(orc, dev, N, K):
+    """Every kernel variant behind bk_gemv_q4k_q8_1 (rows through LDS; direct loads with 1, 2 or 4 rows per wave step;
+    few or many workgroups per CU) returns the checker's bits: the arithmetic does not depend on the launch shape."""
+    print(f"gemv variants N={N} K={K}", flush=True)
+    g = synth.rng(350 + N)
+    W = synth.q4k_random(g, N, K)
+    xq = orc.pack_q8_1(g.standard_normal(K).astype(np.float32))
+    ref = orc.gemv_q4k_q8_1(W, xq, N, K)
+    dW, dxq, dy = dev.up(W), dev.up(xq), dev.empty(N * 4)
+    try:
+        for impl, rpi, cap in [(2, 4, 16), (2, 2, 1), (0, 1, 16), (0, 2, 2), (0, 4, 1), (0, 4, 64)]:
+            rt.tune_set("gemv_impl", impl); rt.tune_set("gemv_rpi", rpi); rt.tune_set("gemv_cap", cap)
+            rt.cuMemset(dy, 0xCD, N * 4)
+            rt.gemv_q4k_q8_1(dW, dxq, dy, N, K)
+            y = rt.from_device(dy, (N,), np.float32)
+            assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (impl, rpi, cap, int((y != ref).sum()))
+    finally:
+        rt.tune_set("gemv_impl", 2); rt.tune_set("gemv_rpi", 4); rt.tune_set("gemv_cap", 16)
+
+
 @pytest.mark.parametrize("N,K", [(64, 256), (33, 768), (100, 1792), (128, 4096), (77, 8192), (5, 2048)])
 def test_gemv_q4k_q8_1_ragged_shapes(orc, dev, N, K):
     print(f"gemv ragged N={N} K={K}", flush=True)
