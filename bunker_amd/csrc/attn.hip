@@ -286,9 +286,9 @@ size_t attn_workspace_bytes(int batch, int NKV, int max_splits) {
 
 int attn_choose_splits(int batch, int NKV, int max_ctx) {
   const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
-  // aim at ~2 workgroups per CU (a CU cannot keep more page requests in flight than that; longer splits amortise
-  // the merge), but keep at least one page per wave in a split
-  int want = (2 * num_cus() + batch * NKV - 1) / (batch * NKV);
+  // aim at one workgroup per CU (measured best at every size: a CU cannot keep more page requests in flight than one
+  // workgroup issues, and longer splits amortise start-up and merge), but keep at least one page per wave in a split
+  int want = (num_cus() + batch * NKV - 1) / (batch * NKV);
   int cap = (pages + ATT_WAVES - 1) / ATT_WAVES;
   int s = want < cap ? want : cap;
   return s < 1 ? 1 : (s > ATT_MAX_SPLITS ? ATT_MAX_SPLITS : s);
