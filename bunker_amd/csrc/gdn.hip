@@ -214,6 +214,8 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   }
 }
 
+int g_tune_gdn_cs = 0;    // column slabs per head for the core entry point (0 = from the shape)
+
 static int check_common(const GdnArgs& A, int batch) {
   BK_REQUIRE(A.q && A.k && A.v && A.S_in && A.S_out && A.out, "gdn_step: null pointer");
   BK_REQUIRE(A.Hg > 0 && A.Hg <= 65535 && batch > 0 && batch <= 65535, "gdn_step: bad Hg=%d batch=%d", A.Hg, batch);
@@ -266,9 +268,13 @@ int launch_gdn_core(const void* q, const void* k, const void* v, const float* g,
   BK_REQUIRE(g && beta, "gdn_core: null pointer");
   int rc = check_common(A, batch);
   if (rc) return rc;
-  // few (batch, head) pairs: cut every head into 4 column slabs so that more CUs stream S
-  if ((int64_t)Hg * batch < 2 * num_cus())
+  // up to a few (batch, head) pairs per CU: cut every head into two column slabs (measured best at 32 .. 512 pairs)
+  const int64_t pairs = (int64_t)Hg * batch;
+  const int cs = g_tune_gdn_cs > 0 ? g_tune_gdn_cs : (pairs <= 4 * num_cus() ? 2 : 1);
+  if (cs == 4)
     hipLaunchKernelGGL((gdn_step_kernel<4, false>), dim3(Hg, 4, batch), dim3(GDN_THREADS), 0, stream(), A);
+  else if (cs == 2)
+    hipLaunchKernelGGL((gdn_step_kernel<2, false>), dim3(Hg, 2, batch), dim3(GDN_THREADS), 0, stream(), A);
   else
     hipLaunchKernelGGL((gdn_step_kernel<1, false>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
   BK_LAUNCH_CHECK();

@@ -60,6 +60,7 @@ int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* 
                    int max_steps);
 
 // gdn.hip
+extern int g_tune_gdn_cs;
 int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
                      const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch);
 int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv_w, const void* z, const float* A_log,
