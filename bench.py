@@ -4,12 +4,13 @@
 Headline workload (BASELINE.json configs[1]): the Q4_K x Q8_1 GEMV at the four decode
 shapes, batch 1 — qkv 2048->6144, gate+up 2048->12288, down 6144->2048, lm_head
 2048->151936.  One "step" is one launch of each shape.  Weights are resident in HBM before
-timing and every launch reads a different copy out of a > 512 MiB rotation, so neither L2
-nor the 256 MiB Infinity Cache serves re-reads.  `value` is algorithmic GB/s over the whole
-timed region (formula: N*K*144/256 + (K/32)*36 + N*4 bytes per launch).
+timing and every launch of a shape reads a different copy out of a >= 600 MB rotation of that
+shape, so neither L2 nor the 256 MiB Infinity Cache serves re-reads.  `value` is algorithmic
+GB/s over the whole timed region (formula: N*K*144/256 + (K/32)*36 + N*4 bytes per launch).
 
-The timed region holds exactly K steps; launches are grouped by shape with a HIP event
-between groups (recorded on the library's stream), which gives each kernel's average
+The timed region holds exactly K steps, grouped by shape: W warm-up launches of the shape, a
+HIP event, its K launches (replayed from one HIP graph, or queued from the host with
+--mode stream), a HIP event (both on the library's stream).  That gives each kernel's average
 launch duration from the same region that `value` is taken from.
 
 Further sections, reported under "decode" and "kernels" of the same line: greedy decode of the
@@ -17,7 +18,7 @@ synthetic Qwen3.5-style model (BASELINE configs[4]) at batch 1 and 32 in tok/s a
 byte floor of one step, and the gated-DeltaNet step (configs[2]) and the paged decode attention
 (configs[3]) in algorithmic GB/s.  `--sections gemv` runs the headline part alone.
 
-Prints ONE JSON line.  `python bench.py --gpus 1 --steps 200 --warmup 20`.
+Prints ONE JSON line.  `python bench.py --gpus 1 --steps 2000 --warmup 500`.
 """
 from __future__ import annotations
 
@@ -37,9 +38,9 @@ HBM_PEAK_GBS = 8000.0
 # `bench.py --sections gemv,calib` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter
 # reads for memcopy_kernel of 175030272 bytes (FETCH_SIZE reads 0.50006 of the bytes: factor 1.99979; WRITE_SIZE factor 1.0).
 # The summary with the per-shape counters is profiles/gemv_q4k_q8_1_decode_shapes.md.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65721624
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65721604
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
-ROTATION = 4            # weight sets; one set is 203 MB, so the rotation spans 813 MB
+ROTATION_BYTES = 600e6  # every shape rotates through copies of its matrix that add up to at least this much
 
 
 def gemv_bytes(N, K, batch=1):
@@ -73,7 +74,7 @@ def cpu_baseline(seconds_target=12.0):
                       f"{dt:.1f} s on {threads} OpenMP threads of the host CPU"}
 
 
-def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16, fused=True):
+def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=True):
     """tok/s of the full synthetic decode step at batch 1 and 32 (device-resident loop, HIP graph replay)."""
     from bunker_amd import model, runner, synth_model
 
@@ -90,7 +91,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=48, steps_bs32=16, fused=T
         envs.append(env)
         dev_w = dev_w or env.weight_ptrs()
         starts = [(9419 + 4099 * i) % D.VOCAB for i in range(B)]
-        warm = 3
+        warm = 8 if B == 1 else 4          # warm + steps stays inside the KV capacity (4096 + 256 tokens)
         loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph,
                                  partition=runner.fusedPartition(g) if fused else None)
         loop.step(warm)
@@ -198,14 +199,16 @@ def bench_kernels(rt, synth, use_graph=True, iters=50):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # 2000 timed steps after 500 warm-up steps: the clocks of an idle GPU take a few thousand launches to settle
+    # (the same kernels measure 8 % slower in a 200-step run); the whole GEMV section still lasts 0.2 s
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sections", default="gemv,decode,kernels",
                     help="comma list of gemv (headline, always on), decode, kernels")
-    ap.add_argument("--mode", choices=["graph", "stream"], default="stream",
-                    help="GEMV section. stream: K individual launches per shape, queued back to back; "
-                         "graph: the K launches replayed from one HIP graph")
+    ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
+                    help="GEMV section. graph: the K launches of a shape replayed from one HIP graph (the device's own launch "
+                         "rate); stream: K individual launches per shape queued from the host (used under rocprofv3)")
     ap.add_argument("--unfused", action="store_true", help="decode section: one kernel per graph node (the reference's partition)")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode and kernels sections launch eagerly instead of replaying HIP graphs "
@@ -213,9 +216,10 @@ def main():
     args = ap.parse_args()
     # under rocprofv3 the decode and kernels sections launch eagerly: its tracer faults inside hipGraphLaunch on this ROCm
     profiled = "rocprof" in os.environ.get("LD_PRELOAD", "") or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
-    if profiled and not args.no_graph:
+    if profiled:
         args.no_graph = True
-        print("bench.py: profiler attached, decode/kernels sections launch eagerly", file=sys.stderr)
+        args.mode = "stream"
+        print("bench.py: profiler attached, every section launches from the host instead of replaying HIP graphs", file=sys.stderr)
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives, no sharding).", file=sys.stderr)
         sys.exit(2)
@@ -227,21 +231,19 @@ def main():
     info = rt.device_info()
     g = synth.rng(2026)
 
-    # one weight set on the host, ROTATION copies on the device
-    sets = []          # sets[r][shape] = device pointer
-    host = {}
+    # per shape: as many device copies of the matrix as it takes to span ROTATION_BYTES (launches are grouped by shape,
+    # so each shape needs its own > 256 MiB working set: 85 copies of qkv and down, 43 of gate_up, 4 of lm_head)
+    copies = {}        # copies[shape] = [device pointers]
     for name, N, K in SHAPES:
-        host[name] = synth.q4k_random(g, N, K)
-    for r in range(ROTATION):
-        ptrs = {}
-        for name, N, K in SHAPES:
-            if r == 0:
-                ptrs[name] = rt.to_device(host[name])
-            else:
-                ptrs[name] = rt.cuAlloc(host[name].nbytes)
-                rt.cuDtoD(ptrs[name], sets[0][name], host[name].nbytes)
-        sets.append(ptrs)
-    del host
+        h = synth.q4k_random(g, N, K)
+        n = max(2, int(-(-ROTATION_BYTES // h.nbytes)))
+        first = rt.to_device(h)
+        copies[name] = [first]
+        for _ in range(n - 1):
+            p = rt.cuAlloc(h.nbytes)
+            rt.cuDtoD(p, first, h.nbytes)
+            copies[name].append(p)
+        del h
     xq, y = {}, {}
     for name, N, K in SHAPES:
         x = g.standard_normal(K).astype(np.float32)
@@ -252,40 +254,65 @@ def main():
     rt.cuSync()
 
     def launch(name, N, K, i):
-        rt.gemv_q4k_q8_1(sets[i % ROTATION][name], xq[name], y[name], N, K)
+        rt.gemv_q4k_q8_1(copies[name][i % len(copies[name])], xq[name], y[name], N, K)
 
-    for w in range(args.warmup):
-        for name, N, K in SHAPES:
-            launch(name, N, K, w)
-    rt.cuSync()
-
-    graphs = []
+    # each shape: one HIP graph of K launches (graph mode), W warm-up launches of that shape directly before its timed
+    # K launches, an event on either side.  The timed region of the workload is the sum of the four: exactly K steps.
+    graphs = {}
     if args.mode == "graph":
         for name, N, K in SHAPES:
             with rt.Graph() as gr:
                 for i in range(args.steps):
                     launch(name, N, K, i)
-            graphs.append(gr)
+            graphs[name] = gr
         rt.cuSync()
 
-    ev = [rt.Event() for _ in range(len(SHAPES) + 1)]
-    rt.cuSync()
-    t0 = time.perf_counter()
-    ev[0].record()
-    for si, (name, N, K) in enumerate(SHAPES):
-        if graphs:
-            graphs[si].launch()
+    def run_region(name, N, K, n):
+        e0, e1 = rt.Event(), rt.Event()
+        for w in range(args.warmup):
+            launch(name, N, K, w)
+        e0.record()
+        if args.mode == "graph":
+            graphs[name].launch()
         else:
-            for i in range(args.steps):
+            for i in range(n):
                 launch(name, N, K, i)
-        ev[si + 1].record()
+        e1.record()
+        rt.cuSync()
+        return e0.elapsed_ms(e1)
+
+    # duration of the shortest possible launch in the same mode (16-byte read by one workgroup): the floor under every
+    # kernel here, and the reason the three small shapes cannot come near the HBM roofline
+    sink = rt.cuAlloc(256)
+    n_floor = min(args.steps, 500)
+    for _ in range(20):
+        rt.memread(sink, 16, sink + 128)
     rt.cuSync()
+    if args.mode == "graph":
+        with rt.Graph() as gfl:
+            for _ in range(n_floor):
+                rt.memread(sink, 16, sink + 128)
+        rt.cuSync()
+    f0, f1 = rt.Event(), rt.Event()
+    f0.record()
+    if args.mode == "graph":
+        gfl.launch()
+    else:
+        for _ in range(n_floor):
+            rt.memread(sink, 16, sink + 128)
+    f1.record()
+    rt.cuSync()
+    launch_floor_us = f0.elapsed_ms(f1) * 1e3 / n_floor
+    rt.cuFree(sink)
+
+    t0 = time.perf_counter()
+    region_ms = {name: run_region(name, N, K, args.steps) for name, N, K in SHAPES}
     wall = time.perf_counter() - t0
 
     per_shape = {}
-    total_ms = ev[0].elapsed_ms(ev[-1])
+    total_ms = sum(region_ms.values())
     for si, (name, N, K) in enumerate(SHAPES):
-        ms = ev[si].elapsed_ms(ev[si + 1]) / args.steps
+        ms = region_ms[name] / args.steps
         b = gemv_bytes(N, K)
         per_shape[name] = {"N": N, "K": K, "us_per_launch": round(ms * 1e3, 3), "bytes": b,
                            "GBps": round(b / (ms * 1e-3) / 1e9, 1),
@@ -310,15 +337,17 @@ def main():
         "vs_baseline": None, "dtype": "u4 x int8 -> int32 dots, f64 fold, f32 out", "data": "synthetic",
         "config": {"workload": "Q4_K x Q8_1 GEMV, batch 1, decode shapes qkv/gate_up/down/lm_head "
                                "(BASELINE configs[1]); one step = one launch of each shape",
-                   "weight_rotation_MB": round(ROTATION * sum(N * K * 144 // 256 for _, N, K in SHAPES) / 1e6),
+                   "weight_rotation_MB_per_shape": {n: round(len(c) * NN * KK * 144 // 256 / 1e6) for (n, NN, KK), c in
+                                                    zip(SHAPES, copies.values())},
                    "launch_mode": args.mode, "device": info["name"], "cus": info["cus"]},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
+        "launch_floor_us": round(launch_floor_us, 3),
+        "wall_ms_per_step_incl_warmup": round(wall * 1e3 / args.steps, 5),
         "per_shape": per_shape,
         "roofline": roofline,
     }
-    for r in sets:
-        for p in r.values():
+    for c in copies.values():
+        for p in c:
             rt.cuFree(p)
     sections = set(args.sections.split(","))
     if "calib" in sections:
