@@ -16,7 +16,8 @@ launch duration from the same region that `value` is taken from.
 Further sections, reported under "decode" and "kernels" of the same line: greedy decode of the
 synthetic Qwen3.5-style model (BASELINE configs[4]) at batch 1 and 32 in tok/s against the
 byte floor of one step, and the gated-DeltaNet step (configs[2]) and the paged decode attention
-(configs[3]) in algorithmic GB/s.  `--sections gemv` runs the headline part alone.
+(configs[3]) in algorithmic GB/s, and under "gemm_bs32" the batch-32 int8-MFMA matmul at the
+decode shapes (weight GB/s and int8 TOP/s).  `--sections gemv` runs the headline part alone.
 
 Prints ONE JSON line.  `python bench.py --gpus 1 --steps 2000 --warmup 500`.
 """
@@ -135,6 +136,37 @@ def _time_launches(rt, enqueue, use_graph):
     return e0.elapsed_ms(e1) * 1e3
 
 
+MFMA_INT8_PEAK_TOPS = 5000.0      # MI355X dense int8
+
+
+def bench_gemm(rt, synth, use_graph=True, iters=60, batch=32):
+    """The batched decode matmul (int8 MFMA, batch 32) at the decode shapes: weight GB/s and int8 TOP/s."""
+    g = synth.rng(9)
+    res = {}
+    for name, N, K in SHAPES:
+        h = synth.q4k_random(g, N, K)
+        n = max(2, int(-(-ROTATION_BYTES // h.nbytes)))
+        first = rt.to_device(h)
+        ws = [first]
+        for _ in range(n - 1):
+            p = rt.cuAlloc(h.nbytes); rt.cuDtoD(p, first, h.nbytes); ws.append(p)
+        dx = rt.to_device(g.standard_normal((batch, K)).astype(np.float32))
+        xq = rt.cuAlloc(batch * (K // 32) * 36)
+        rt.quantize_q8_1(dx, xq, K, batch, rt.F32)
+        y = rt.cuAlloc(batch * N * 4)
+        for i in range(10):
+            rt.gemm_q4k_q8_1(ws[i % n], xq, y, N, K, batch)
+        us = _time_launches(rt, lambda: [rt.gemm_q4k_q8_1(ws[i % n], xq, y, N, K, batch) for i in range(iters)], use_graph) / iters
+        nbytes = gemv_bytes(N, K, batch)
+        tops = 2.0 * N * K * batch / us / 1e6
+        res[name] = {"N": N, "K": K, "batch": batch, "us": round(us, 3), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "int8_TOPs": round(tops, 1),
+                     "frac_mfma_int8_peak": round(tops / MFMA_INT8_PEAK_TOPS, 5)}
+        for p in ws + [dx, xq, y]:
+            rt.cuFree(p)
+    return res
+
+
 def bench_kernels(rt, synth, use_graph=True, iters=50):
     """Gated-DeltaNet step (configs[2]) and paged decode attention (configs[3]) in algorithmic GB/s."""
     g = synth.rng(5)
@@ -204,8 +236,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sections", default="gemv,decode,kernels",
-                    help="comma list of gemv (headline, always on), decode, kernels")
+    ap.add_argument("--sections", default="gemv,decode,kernels,gemm",
+                    help="comma list of gemv (headline, always on), decode, kernels, gemm, calib")
     ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
                     help="GEMV section. graph: the K launches of a shape replayed from one HIP graph (the device's own launch "
                          "rate); stream: K individual launches per shape queued from the host (used under rocprofv3)")
@@ -364,6 +396,8 @@ def main():
         out["decode"] = bench_decode(rt, synth, use_graph=not args.no_graph, fused=not args.unfused)
     if "kernels" in sections:
         out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
+    if "gemm" in sections:
+        out["gemm_bs32"] = bench_gemm(rt, synth, use_graph=not args.no_graph)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
