@@ -42,7 +42,7 @@ struct MfmaArgs {
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
-  __shared__ double lds_d8[NW][8][32], lds_s8[NW][8][32];
+  __shared__ double2 lds_ds[NW][8][32];          // (d8, s8) of activation block (j, b) of the wave's current super-block, as doubles
   __shared__ double lds_acc[NW > 1 ? 16 * 64 : 1];
 
   const int tile = blockIdx.x;
@@ -88,8 +88,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
       const int t = lane + 64 * i;
       const int b = t >> 3, j = t & 7;
       const uint32_t ds = *(const uint32_t*)(xq + (int64_t)min(b, B - 1) * xrow_bytes + (int64_t)(blk * 8 + j) * 36 + 32);
-      lds_d8[wave][j][b] = (double)half_to_f32((uint16_t)(ds & 0xffffu));
-      lds_s8[wave][j][b] = (double)half_to_f32((uint16_t)(ds >> 16));
+      lds_ds[wave][j][b] = make_double2((double)half_to_f32((uint16_t)(ds & 0xffffu)), (double)half_to_f32((uint16_t)(ds >> 16)));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -124,12 +123,21 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
       c = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb, c, 0, 0, 0);
       const int sc = (int)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xffu);
       const double mj = (double)(((j < 4 ? m_lo : m_hi) >> (8 * (j & 3))) & 0xffu);
+      // the scales of eight outputs are requested together and consumed as they arrive (LDS returns in order);
+      // without the scheduling fences the compiler pairs every read with its use and exposes the LDS latency 16 times
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int b = mfma32_row(r, half);
-        const int p = __mul24(sc, c[r]);                            // 6-bit x 17-bit: exact
-        sblk[r] = fma(lds_d8[wave][j][b], (double)p, sblk[r]);
-        mblk[r] = fma(mj, lds_s8[wave][j][b], mblk[r]);
+      for (int r0 = 0; r0 < 16; r0 += 8) {
+        double2 ds8[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) ds8[r] = lds_ds[wave][j][mfma32_row(r0 + r, half)];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+          const int p = __mul24(sc, c[r0 + r]);                     // 6-bit x 17-bit: exact
+          sblk[r0 + r] = fma(ds8[r].x, (double)p, sblk[r0 + r]);
+          mblk[r0 + r] = fma(mj, ds8[r].y, mblk[r0 + r]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     const double dd = (double)d, dm = (double)dmin;
@@ -191,6 +199,7 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   int nw = g_tune_gemm_nw;
   if (nw <= 0) {
     nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
+    if (tiles <= num_cus() / 2 && A.nb >= 8) nw = 8;          // few tiles: one super-block per wave
     if (tiles >= 8 * num_cus() && nw > 2) nw = 2;
   }
   const dim3 grid(tiles);
