@@ -165,12 +165,15 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   }
   *(float4*)&part[kg][vq * 4] = acc;
   __syncthreads();
+  // all partials are requested before the first is added (the fence keeps the compiler from pairing every LDS read
+  // with its use, which would expose the LDS latency KG times); the sum keeps its order
+  float4 pk[KG];
+#pragma unroll
+  for (int j = 0; j < KG; j++) pk[j] = *(const float4*)&part[j][vq * 4];
+  __builtin_amdgcn_sched_barrier(0);
   float4 kS = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-  for (int j = 0; j < KG; j++) {
-    const float4 p = *(const float4*)&part[j][vq * 4];
-    kS.x += p.x; kS.y += p.y; kS.z += p.z; kS.w += p.w;
-  }
+  for (int j = 0; j < KG; j++) { kS.x += pk[j].x; kS.y += pk[j].y; kS.z += pk[j].z; kS.w += pk[j].w; }
   __syncthreads();   // part is reused for o below
   const uint2 vv = CONV ? *(const uint2*)(vsh + col0) : vv_g;
   float4 d;
