@@ -444,6 +444,10 @@ int bk_quantize_q8_1(uint64_t x, int x_dtype, uint64_t out, int K, int batch) {
   BK_NEED_INIT();
   return launch_quantize_q8_1(P<void>(x), x_dtype, P<void>(out), K, batch);
 }
+int bk_quantize_q4k(uint64_t w, int w_dtype, uint64_t out, int64_t rows, int K) {
+  BK_NEED_INIT();
+  return launch_quantize_q4k(P<void>(w), w_dtype, P<void>(out), rows, K);
+}
 int bk_gemv_q4k_f32(uint64_t W, uint64_t x, uint64_t y, int N, int K) {
   BK_NEED_INIT();
   return launch_gemv_q4k_f32(P<void>(W), P<float>(x), P<float>(y), N, K);

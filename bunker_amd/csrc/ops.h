@@ -20,6 +20,9 @@ int launch_dequant_legacy_i8(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_nibbles(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_dequant_f32(const void* blocks, void* out, int64_t nblocks);
 
+// quant_q4k.hip
+int launch_quantize_q4k(const void* w, int w_dtype, void* out, int64_t rows, int K);
+
 int launch_memread(const void* src, int64_t bytes, void* sink);
 int launch_memcopy(const void* src, void* dst, int64_t bytes);
 

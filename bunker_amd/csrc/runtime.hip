@@ -162,6 +162,42 @@ int bk_dtod(uint64_t dst, uint64_t src, uint64_t bytes) {
   BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToDevice, g_stream));
   return BK_OK;
 }
+// Pinned staging memory and copies that return before the data has moved (cuMemAllocHost /
+// cuMemcpyHtoDAsync of the reference's loaders); the caller orders them with bk_sync or events.
+int bk_host_alloc(uint64_t bytes, uint64_t* out) {
+  BK_NEED_INIT();
+  BK_REQUIRE(out && bytes, "bk_host_alloc: null pointer or zero size");
+  void* p = nullptr;
+  BK_HIP(hipHostMalloc(&p, bytes, hipHostMallocDefault));
+  *out = (uint64_t)(uintptr_t)p;
+  return BK_OK;
+}
+int bk_host_free(uint64_t ptr) {
+  BK_NEED_INIT();
+  if (!ptr) return BK_OK;
+  BK_HIP(hipHostFree((void*)(uintptr_t)ptr));
+  return BK_OK;
+}
+int bk_htod_async(uint64_t dst, const void* src, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst && src, "bk_htod_async: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+  return BK_OK;
+}
+int bk_dtoh_async(void* dst, uint64_t src, uint64_t bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(dst && src, "bk_dtoh_async: null pointer");
+  if (!bytes) return BK_OK;
+  BK_HIP(hipMemcpyAsync(dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToHost, g_stream));
+  return BK_OK;
+}
+int bk_event_sync(uint64_t ev) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ev, "bk_event_sync: null event");
+  BK_HIP(hipEventSynchronize((hipEvent_t)(uintptr_t)ev));
+  return BK_OK;
+}
 int bk_memset(uint64_t dst, int value, uint64_t bytes) {
   BK_NEED_INIT();
   BK_REQUIRE(dst, "bk_memset: null pointer");

@@ -38,6 +38,8 @@ _SIGS = {
     "bk_alloc": [u64, C.POINTER(u64)], "bk_free": [u64],
     "bk_htod": [u64, vp, u64], "bk_dtoh": [vp, u64, u64], "bk_dtod": [u64, u64, u64],
     "bk_memset": [u64, i32, u64], "bk_sync": [],
+    "bk_host_alloc": [u64, C.POINTER(u64)], "bk_host_free": [u64],
+    "bk_htod_async": [u64, vp, u64], "bk_dtoh_async": [vp, u64, u64], "bk_event_sync": [u64],
     "bk_event_create": [C.POINTER(u64)], "bk_event_record": [u64],
     "bk_event_elapsed_ms": [u64, u64, C.POINTER(C.c_float)], "bk_event_destroy": [u64],
     "bk_prof_enable": [i32], "bk_prof_reset": [], "bk_prof_report": [C.c_char_p, i32],
@@ -48,6 +50,7 @@ _SIGS = {
     "bk_kernel_describe": [i32, C.c_char_p, i32],
     "bk_memread": [u64, i64, u64], "bk_memcopy": [u64, u64, i64],
     "bk_quantize_q8_1": [u64, i32, u64, i32, i32],
+    "bk_quantize_q4k": [u64, i32, u64, i64, i32],
     "bk_gemv_q4k_f32": [u64, u64, u64, i32, i32],
     "bk_gemv_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
     "bk_gemm_q4k_q8_1": [u64, u64, u64, i32, i32, i32, i32, u64],
@@ -156,6 +159,39 @@ def cuDtoD(dst: int, src: int, nbytes: int) -> None:
     _check(cu().bk_dtod(dst, src, nbytes), "cuDtoD")
 
 
+def cuHtoDAsync(dev: int, host, nbytes: int | None = None) -> None:
+    """Enqueue the copy and return (src/ttir.ts:305-308); ``host`` must be pinned (``cuAllocHost``) and left
+    untouched until ``cuSync`` or an event recorded after the copy has been waited for."""
+    addr, n = _host_view(host)
+    _check(cu().bk_htod_async(dev, addr, int(nbytes if nbytes is not None else n)), "cuHtoDAsync")
+
+
+def cuDtoHAsync(host, dev: int, nbytes: int | None = None) -> None:
+    addr, n = _host_view(host)
+    _check(cu().bk_dtoh_async(addr, dev, int(nbytes if nbytes is not None else n)), "cuDtoHAsync")
+
+
+class PinnedBuffer:
+    """Page-locked host staging memory, viewed as a numpy uint8 array (``.array``)."""
+
+    def __init__(self, nbytes: int):
+        out = u64(0)
+        _check(cu().bk_host_alloc(int(nbytes), C.byref(out)), f"cuAllocHost({nbytes})")
+        self.ptr = int(out.value)
+        self.nbytes = int(nbytes)
+        self.array = np.ctypeslib.as_array((C.c_uint8 * self.nbytes).from_address(self.ptr))
+
+    def free(self) -> None:
+        if self.ptr:
+            self.array = None
+            _check(cu().bk_host_free(self.ptr), "cuFreeHost")
+            self.ptr = 0
+
+
+def cuAllocHost(nbytes: int) -> PinnedBuffer:
+    return PinnedBuffer(nbytes)
+
+
 def to_device(arr: np.ndarray) -> int:
     """Allocate and upload a numpy array; returns the device pointer."""
     arr = np.ascontiguousarray(arr)
@@ -245,10 +281,17 @@ class Event:
         _check(cu().bk_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "bk_event_elapsed_ms")
         return float(ms.value)
 
+    def sync(self):
+        _check(cu().bk_event_sync(self.h), "bk_event_sync")
+
     def destroy(self):
         if self.h:
             cu().bk_event_destroy(self.h)
             self.h = 0
+
+
+def eventSync(ev: "Event") -> None:
+    ev.sync()
 
 
 class Graph:
@@ -296,6 +339,11 @@ def memcopy(src: int, dst: int, nbytes: int) -> None:
 
 def quantize_q8_1(x: int, out: int, K: int, batch: int = 1, x_dtype: int = F32) -> None:
     _check(cu().bk_quantize_q8_1(x, x_dtype, out, K, batch), "bk_quantize_q8_1")
+
+
+def quantize_q4k(w: int, out: int, rows: int, K: int, w_dtype: int = BF16) -> None:
+    """[rows, K] f32 / bf16 weights on the device -> rows * K/256 Q4_K super-blocks (144 bytes each)."""
+    _check(cu().bk_quantize_q4k(w, w_dtype, out, rows, K), "bk_quantize_q4k")
 
 
 def gemv_q4k_f32(W: int, x: int, y: int, N: int, K: int) -> None:

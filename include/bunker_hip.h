@@ -43,11 +43,19 @@ BK_API int bk_dtoh(void* dst, uint64_t src, uint64_t bytes);         /* cuDtoH, 
 BK_API int bk_dtod(uint64_t dst, uint64_t src, uint64_t bytes);
 BK_API int bk_memset(uint64_t dst, int value, uint64_t bytes);
 BK_API int bk_sync(void);                            /* cuSync, src/ttir.ts:285 */
+/* Pinned host staging and copies that do not wait (cuHtoDAsync / cuDtoHAsync, src/ttir.ts:305-317):
+ * enqueued on the library's stream; the host buffer must stay untouched until bk_sync or an event
+ * recorded after the copy has been waited for (bk_event_sync). */
+BK_API int bk_host_alloc(uint64_t bytes, uint64_t* out);
+BK_API int bk_host_free(uint64_t ptr);
+BK_API int bk_htod_async(uint64_t dst, const void* src, uint64_t bytes);
+BK_API int bk_dtoh_async(void* dst, uint64_t src, uint64_t bytes);
 
 /* ---- timing: replaces the cuEvent* calls of src/ttir.ts:352-417 */
 BK_API int bk_event_create(uint64_t* out);
 BK_API int bk_event_record(uint64_t ev);             /* on the library's stream */
 BK_API int bk_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms);  /* waits for stop */
+BK_API int bk_event_sync(uint64_t ev);                /* host waits until the event has happened */
 BK_API int bk_event_destroy(uint64_t ev);
 BK_API int bk_prof_enable(int on);                   /* BUNKER_GPU_PROF=1: an event pair around every bk_launch */
 BK_API int bk_prof_reset(void);                      /* profGpuReset, src/ttir.ts:385-388 */
@@ -90,6 +98,15 @@ BK_API int bk_memcopy(uint64_t src, uint64_t dst, int64_t bytes);
  * reference).  x is [batch, K] f32 (x_dtype 0) or bf16 (1); out is
  * [batch, K/32] blocks of 36 bytes: int8 q[32] @0, fp16 d @32, fp16 s @34. */
 BK_API int bk_quantize_q8_1(uint64_t x, int x_dtype, uint64_t out, int K, int batch);
+
+/* Weight quantizer, run once at model load: w is [rows, K] f32 (w_dtype 0) or bf16 (1),
+ * K a multiple of 256; out is rows * K/256 super-blocks of 144 bytes, row-major.  The
+ * reference quantizes weights only into its legacy 20-byte block (packQ4_K_col,
+ * bench/bench.ts:74-96) from the bf16 checkpoint tensors its loaders place on the device
+ * (prototypes/safetensors_loader.ts:13-78, prototypes/decode.ts:64-75); for the super-block this
+ * is the published ggml fit (quantize_row_q4_K_ref / make_qkx2_quants), evaluated per sub-block
+ * in the host loop's own operation order so the bytes equal a host run's. */
+BK_API int bk_quantize_q4k(uint64_t w, int w_dtype, uint64_t out, int64_t rows, int K);
 
 /* Q4_K dequantize + f32 GEMV on 144-byte super-blocks: y[N] = W[N,K] . x[K],
  * x f32.  The dequant-then-dot the reference's CPU path computes (packers and

@@ -32,6 +32,11 @@
  *                                   the published ggml layout, a hand-built
  *                                   block, pack/unpack round trips and the
  *                                   integer-dot special case
+ *   orc_quantize_q4k                PARITY UNPINNED against ggml (absent); invariants:
+ *                                   constant blocks, representable grids, fitted error
+ *                                   <= min/max grid error, reconstruction error bound
+ *   orc_f32_to_half_rne             exhaustive round trip of all 65536 halves, midpoints,
+ *                                   numpy float16 on random values
  *   orc_gdn_step                    closed-form invariants (beta=0, S=0) and a
  *                                   numpy float64 restatement of refGDN
  *   orc_attn_decode_paged           numpy float64 softmax, len=1, page permutation
@@ -278,6 +283,166 @@ ORC_API void orc_q4k_dequant(const uint8_t* blocks, int64_t nblocks, float* out)
         out[b * 256 + 64 * g + l] = d0 * (float)(qs[32 * g + l] & 15) - m0;
         out[b * 256 + 64 * g + 32 + l] = d1 * (float)(qs[32 * g + l] >> 4) - m1;
       }
+  }
+}
+
+/* ---- f32 weights -> Q4_K super-blocks ------------------------------- */
+/* The reference quantizes weights only into its legacy 20-byte block
+ * (packQ4_K_col, bench/bench.ts:74-96: per-32 min/max affine).  For the
+ * 144-byte super-block the published algorithm is ggml's
+ * quantize_row_q4_K_ref with make_qkx2_quants (ggml-quants.c; ggml is not a
+ * dependency of the reference, so no version is pinned): per 32-element
+ * sub-block a weighted least-squares fit of (scale, min) over 21 candidate
+ * grids, weights av_x + |x|; then the 8 scales and 8 mins of a super-block are
+ * quantized to 6 bits against their maxima, d and dmin stored as
+ * round-to-nearest-even fp16, and the nibbles re-derived from the stored
+ * (fp16, 6-bit) values.  All arithmetic is f32, one IEEE operation per written
+ * operation, sums in ascending element order.
+ * PARITY UNPINNED against ggml itself (absent here); pinned by invariants:
+ * constant sub-blocks, exactly representable grids, fitted error <= min/max
+ * grid error, and the reconstruction error bound. */
+
+/* round to nearest, ties to even, of |v| <= 2^22 (ggml nearest_int) */
+static inline int nearest_int_(float v) {
+  float t = v + 12582912.f;
+  int32_t i; memcpy(&i, &t, 4);
+  return (i & 0x007fffff) - 0x00400000;
+}
+
+/* IEEE f32 -> fp16, round to nearest even, subnormals kept */
+ORC_API uint16_t orc_f32_to_half_rne(float f) {
+  uint32_t u = f2u(f), sign = (u >> 16) & 0x8000u;
+  u &= 0x7fffffffu;
+  if (u > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+  if (u == 0x7f800000u) return (uint16_t)(sign | 0x7c00u);
+  int e = (int)(u >> 23) - 127 + 15;
+  if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (e <= 0) {                                   /* |f| < 2^-14: multiples of 2^-24 */
+    float scaled = u2f(u) * 16777216.0f;          /* exact scaling (or a flush of f32 denormals toward 0) */
+    return (uint16_t)(sign | (uint32_t)lrintf(scaled));   /* default rounding mode = nearest even; 1024 = smallest normal */
+  }
+  uint32_t mant = u & 0x7fffffu, h = ((uint32_t)e << 10) | (mant >> 13), rem = mant & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;    /* a carry runs into the exponent, up to Inf */
+  return (uint16_t)(sign | h);
+}
+
+/* make_qkx2_quants(n=32, nmax=15, rmin=-1, rdelta=0.1, nstep=20, use_mad=false) */
+static float qkx2_fit32_(const float* x, const float* weights, uint8_t* L, float* the_min) {
+  const int n = 32, nmax = 15, nstep = 20;
+  const float rmin = -1.f, rdelta = 0.1f;
+  uint8_t Laux[32];
+  float min = x[0], max = x[0];
+  float sum_w = weights[0];
+  float sum_x = sum_w * x[0];
+  for (int i = 1; i < n; i++) {
+    if (x[i] < min) min = x[i];
+    if (x[i] > max) max = x[i];
+    float w = weights[i];
+    sum_w += w;
+    sum_x += w * x[i];
+  }
+  if (min > 0) min = 0;
+  if (max == min) {
+    for (int i = 0; i < n; i++) L[i] = 0;
+    *the_min = -min;
+    return 0.f;
+  }
+  float iscale = (float)nmax / (max - min);
+  float scale = 1 / iscale;
+  float best = 0;
+  for (int i = 0; i < n; i++) {
+    int l = nearest_int_(iscale * (x[i] - min));
+    l = l < 0 ? 0 : (l > nmax ? nmax : l);
+    L[i] = (uint8_t)l;
+    float diff = scale * (float)L[i] + min - x[i];
+    diff = diff * diff;
+    best += weights[i] * diff;
+  }
+  for (int is = 0; is <= nstep; is++) {
+    iscale = (rmin + rdelta * (float)is + (float)nmax) / (max - min);
+    float sum_l = 0, sum_l2 = 0, sum_xl = 0;
+    for (int i = 0; i < n; i++) {
+      int l = nearest_int_(iscale * (x[i] - min));
+      l = l < 0 ? 0 : (l > nmax ? nmax : l);
+      Laux[i] = (uint8_t)l;
+      float w = weights[i];
+      sum_l += w * (float)l;
+      sum_l2 += w * (float)l * (float)l;
+      sum_xl += w * (float)l * x[i];
+    }
+    float D = sum_w * sum_l2 - sum_l * sum_l;
+    if (D > 0) {
+      float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
+      float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+      if (this_min > 0) {
+        this_min = 0;
+        this_scale = sum_xl / sum_l2;
+      }
+      float err = 0;
+      for (int i = 0; i < n; i++) {
+        float diff = this_scale * (float)Laux[i] + this_min - x[i];
+        diff = diff * diff;
+        err += weights[i] * diff;
+      }
+      if (err < best) {
+        for (int i = 0; i < n; i++) L[i] = Laux[i];
+        best = err;
+        scale = this_scale;
+        min = this_min;
+      }
+    }
+  }
+  *the_min = -min;
+  return scale;
+}
+
+/* the fit alone, for the invariants that hold before the 6-bit step */
+ORC_API float orc_qkx2_fit32(const float* x, const float* weights, uint8_t* L, float* the_min) {
+  return qkx2_fit32_(x, weights, L, the_min);
+}
+
+/* x: n f32 values, n a multiple of 256; out: n/256 blocks of 144 bytes */
+ORC_API void orc_quantize_q4k(const float* x, int64_t n, uint8_t* out) {
+  int64_t nb = n / 256;
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < nb; b++) {
+    const float* xb = x + b * 256;
+    uint8_t* blk = out + b * 144;
+    uint8_t L[256];
+    float weights[32], mins[8], scales[8];
+    float max_scale = 0, max_min = 0;
+    for (int j = 0; j < 8; j++) {
+      float sum_x2 = 0;
+      for (int l = 0; l < 32; l++) sum_x2 += xb[32 * j + l] * xb[32 * j + l];
+      float av_x = sqrtf(sum_x2 / 32);
+      for (int l = 0; l < 32; l++) weights[l] = av_x + fabsf(xb[32 * j + l]);
+      scales[j] = qkx2_fit32_(xb + 32 * j, weights, L + 32 * j, &mins[j]);
+      if (scales[j] > max_scale) max_scale = scales[j];
+      if (mins[j] > max_min) max_min = mins[j];
+    }
+    float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+    float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
+    uint8_t sc[8], m[8];
+    for (int j = 0; j < 8; j++) {
+      uint8_t ls = (uint8_t)nearest_int_(inv_scale * scales[j]);
+      uint8_t lm = (uint8_t)nearest_int_(inv_min * mins[j]);
+      sc[j] = ls > 63 ? 63 : ls;
+      m[j] = lm > 63 ? 63 : lm;
+    }
+    orc_q4k_pack_scales(sc, m, blk + 4);
+    uint16_t hd = orc_f32_to_half_rne(max_scale / 63.f), hm = orc_f32_to_half_rne(max_min / 63.f);
+    memcpy(blk, &hd, 2); memcpy(blk + 2, &hm, 2);
+    for (int j = 0; j < 8; j++) {
+      const float d = orc_half_to_float(hd) * (float)sc[j];
+      if (!d) continue;
+      const float dm = orc_half_to_float(hm) * (float)m[j];
+      for (int i = 0; i < 32; i++) {
+        int l = nearest_int_((xb[32 * j + i] + dm) / d);
+        L[32 * j + i] = (uint8_t)(l < 0 ? 0 : (l > 15 ? 15 : l));
+      }
+    }
+    for (int g = 0; g < 4; g++)
+      for (int l = 0; l < 32; l++) blk[16 + 32 * g + l] = (uint8_t)(L[64 * g + l] | (L[64 * g + 32 + l] << 4));
   }
 }
 

@@ -44,6 +44,8 @@ def lib():
         _lib.orc_half_to_float_ftz.argtypes = [C.c_uint16]
         _lib.orc_f32_to_bf16.restype = C.c_uint16
         _lib.orc_f32_to_bf16.argtypes = [C.c_float]
+        _lib.orc_f32_to_half_rne.restype = C.c_uint16
+        _lib.orc_f32_to_half_rne.argtypes = [C.c_float]
     return _lib
 
 
@@ -165,6 +167,30 @@ def q4k_dequant(blocks) -> np.ndarray:
     nb = blocks.size // 144
     out = np.empty(nb * 256, np.float32)
     lib().orc_q4k_dequant(_p(blocks), C.c_int64(nb), _p(out))
+    return out
+
+
+def f32_to_half_rne(v: float) -> int:
+    return int(lib().orc_f32_to_half_rne(float(v)))
+
+
+def qkx2_fit32(x, weights):
+    """(scale, the_min, L[32]) of one 32-element sub-block."""
+    x = _c(x, np.float32); weights = _c(weights, np.float32)
+    assert x.size == 32 and weights.size == 32
+    L = np.zeros(32, np.uint8); the_min = C.c_float(0)
+    f = lib().orc_qkx2_fit32
+    f.restype = C.c_float
+    scale = f(_p(x), _p(weights), _p(L), C.byref(the_min))
+    return float(scale), float(the_min.value), L
+
+
+def quantize_q4k(x) -> np.ndarray:
+    """f32 values (a multiple of 256 of them, row-major weights) -> 144-byte super-blocks."""
+    x = _c(x, np.float32).ravel()
+    assert x.size % 256 == 0
+    out = np.zeros(x.size // 256 * 144, np.uint8)
+    lib().orc_quantize_q4k(_p(x), C.c_int64(x.size), _p(out))
     return out
 
 

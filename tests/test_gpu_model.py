@@ -28,7 +28,7 @@ def _fa_layers(D):
     return [l for l in range(D.NL) if D.is_full_attention(l)]
 
 
-def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=False):
+def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=False, device_weights=None):
     """GPU DeviceLoop one token at a time against the checker continued from the GPU's attention outputs.
 
     check: the sequences of the batch the checker recomputes (all by default; sequences are independent)."""
@@ -36,7 +36,7 @@ def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=Fa
     B = len(starts)
     check = list(range(B)) if check is None else list(check)
     g = model.buildModelGraph(D, B)
-    env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+    env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True, device_weights=device_weights)
     loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=use_graph,
                              partition=runner.fusedPartition(g) if fused else None)
     fa_nodes = [n for n in g.nodes if n.op == "fa2_attn"]
