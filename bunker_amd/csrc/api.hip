@@ -276,6 +276,38 @@ static int run_fa2_fused(Kernel& k, const uint64_t* s) {
                             (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - (size_t)batch * NH * HD * 2,
                             batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
 }
+// ---- prefill ops: T consecutive tokens of ONE sequence per launch (rows of the activation buffers = tokens)
+// conv1d_prefill   slots: qkv [T, QKVD], conv_state_in [3, QKVD], weight, out [T, QKVD], conv_state_new    params: QKVD, T
+static int run_conv1d_prefill(Kernel& k, const uint64_t* s) {
+  return launch_conv1d_prefill(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), (int)k.get("QKVD", 0),
+                               (int)k.get("T", 0));
+}
+// gdn_prefill      slots as gdn_delta_rule with T rows in conv_out, z, a_p, b_p, out and one state     params: LVH, T
+static int run_gdn_prefill(Kernel& k, const uint64_t* s) {
+  return launch_gdn_prefill(P<void>(s[0]), P<void>(s[1]), P<float>(s[2]), P<void>(s[3]), P<float>(s[4]), P<float>(s[5]),
+                            P<float>(s[6]), P<float>(s[7]), P<void>(s[8]), P<float>(s[9]), k.scratch, k.scratch_bytes,
+                            (int)k.get("LVH", 0), (int)k.get("T", 0));
+}
+// fa2_prefill      the norm + rotation + cache append of fa2_fused for T tokens at positions pos[t], then causal attention:
+//                  token t attends to cache positions 0 .. pos[t] of the sequence whose pages block_table lists.
+// slots: qgate [T, NH, 2*HD], k [T, NKV, HD], v, q_norm.weight, k_norm.weight, rope_cos, rope_sin, pos (int32 [T], device),
+//        block_table (int32 [MAX_LEN/16], device), kv_k, kv_v, out [T, NH*HD]          params: HD, NH, NKV, MAX_LEN, ROT_HALF, T
+static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
+  const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0), NKV = (int)k.get("NKV", 0), T = (int)k.get("T", 0);
+  const int max_len = (int)k.get("MAX_LEN", 0), half = (int)k.get("ROT_HALF", 0);
+  const int32_t* pos = P<int32_t>(s[7]);
+  const int32_t* table = P<int32_t>(s[8]);
+  BK_REQUIRE(pos && table, "fa2_prefill: null position or block table pointer");
+  void* qn = k.scratch;
+  void* ws = (uint8_t*)k.scratch + (size_t)T * NH * HD * 2;
+  int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
+                            pos, 0, half, max_len, qn, P<void>(s[9]), P<void>(s[10]), table, 0, T, NH, NKV, HD, 16);
+  if (rc) return rc;
+  return launch_attn_decode(qn, P<void>(s[9]), P<void>(s[10]), table, 0, pos, 0, 1, max_len, P<uint16_t>(s[0]) + HD,
+                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - (size_t)T * NH * HD * 2,
+                            T, NH, NKV, HD, 16, (int)k.get("splits", 0));
+}
+
 // ---- op: argmax (src/model.ts:198-201)   slots: logits, val, idx     params: VOCAB, batch=1
 static int run_argmax(Kernel& k, const uint64_t* s) {
   return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
@@ -331,6 +363,30 @@ static int build_kernel(Kernel& k) {
     const size_t qbytes = (size_t)batch * k.get("NH", 0) * k.get("HD", 0) * 2;
     if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(batch, NKV, splits) : 0)))) return rc;
     k.run = run_fa2_fused; k.nslots = 11;
+    return BK_OK;
+  }
+  if (k.op == "conv1d_prefill") {
+    if ((rc = need(k, "QKVD")) || (rc = need(k, "T"))) return rc;
+    k.run = run_conv1d_prefill; k.nslots = 5;
+    return BK_OK;
+  }
+  if (k.op == "gdn_prefill") {
+    if ((rc = need(k, "LVH")) || (rc = need(k, "T"))) return rc;
+    BK_REQUIRE(k.get("LVH", 0) >= 1 && k.get("T", 0) >= 1 && k.get("T", 0) <= 65535, "gdn_prefill: bad LVH/T");
+    if ((rc = alloc_scratch(k, gdn_prefill_workspace_bytes((int)k.get("LVH", 0), (int)k.get("T", 0))))) return rc;
+    k.run = run_gdn_prefill; k.nslots = 10;
+    return BK_OK;
+  }
+  if (k.op == "fa2_prefill") {
+    for (const char* p : {"HD", "NH", "NKV", "MAX_LEN", "ROT_HALF", "T"})
+      if ((rc = need(k, p))) return rc;
+    const int T = (int)k.get("T", 0), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
+    BK_REQUIRE(T >= 1 && T <= 65535 && NKV >= 1 && max_len >= 1, "fa2_prefill: bad T/NKV/MAX_LEN");
+    int splits = (int)k.get("splits", 0);
+    if (splits <= 0) { splits = attn_choose_splits(T, NKV, max_len); k.p["splits"] = splits; }
+    const size_t qbytes = (size_t)T * k.get("NH", 0) * k.get("HD", 0) * 2;
+    if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(T, NKV, splits) : 0)))) return rc;
+    k.run = run_fa2_prefill; k.nslots = 12;
     return BK_OK;
   }
   if (k.op == "argmax") {

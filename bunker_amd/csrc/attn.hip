@@ -291,6 +291,8 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
   int want = (num_cus() + batch * NKV - 1) / (batch * NKV);
   int cap = (pages + ATT_WAVES - 1) / ATT_WAVES;
   int s = want < cap ? want : cap;
+  const int need = (pages + ATT_MAX_PPS - 1) / ATT_MAX_PPS;     // a split's page table must fit its LDS copy
+  if (s < need) s = need;
   return s < 1 ? 1 : (s > ATT_MAX_SPLITS ? ATT_MAX_SPLITS : s);
 }
 
@@ -304,7 +306,9 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   BK_REQUIRE(batch > 0 && batch <= 65535 && NKV <= 65535, "attn_decode: bad batch=%d", batch);
   BK_REQUIRE(ctx_len || ctx_scalar + ctx_add >= 1, "attn_decode: context length must be >= 1");
   BK_REQUIRE(max_ctx >= 1 && (ctx_len || ctx_scalar + ctx_add <= max_ctx), "attn_decode: context %d exceeds max_ctx=%d", ctx_scalar + ctx_add, max_ctx);
-  BK_REQUIRE(bt_stride >= (max_ctx + ATT_PAGE - 1) / ATT_PAGE, "attn_decode: block table rows hold %d pages, context needs %d", bt_stride, (max_ctx + ATT_PAGE - 1) / ATT_PAGE);
+  // bt_stride 0 with a table: every row of the batch reads the same sequence's pages (the tokens of one prompt)
+  BK_REQUIRE(bt_stride >= (max_ctx + ATT_PAGE - 1) / ATT_PAGE || (block_table && bt_stride == 0),
+             "attn_decode: block table rows hold %d pages, context needs %d", bt_stride, (max_ctx + ATT_PAGE - 1) / ATT_PAGE);
   BK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kc & 15) == 0 && ((uintptr_t)vc & 15) == 0, "attn_decode: q, K and V must be 16-byte aligned");
   if (splits <= 0) splits = attn_choose_splits(batch, NKV, max_ctx);
   const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;

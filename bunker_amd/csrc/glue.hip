@@ -182,6 +182,66 @@ int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out
   return BK_OK;
 }
 
+// ---------------------------------------------------------------- conv1d over a run of T tokens
+// The same 4-tap causal convolution + SiLU for T consecutive tokens of ONE sequence (prefill form,
+// prototypes/conv1d.ts:53-61, with the three rows of carried state in place of zero padding): token t reads
+// rows t-3 .. t of the virtual sequence [state row 0, 1, 2, x_0 .. x_{T-1}].  Same expression per channel as
+// conv1d_decode, so T single-token steps give the same bits.  The new state (the last three rows of the
+// virtual sequence) is written by a second kernel after every token has read the old one, so it may be
+// updated in place.
+__global__ __launch_bounds__(256) void conv1d_prefill_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ st,
+                                                             const uint16_t* __restrict__ w, uint16_t* __restrict__ out, int C) {
+  const int t = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 2;
+  if (c >= C) return;
+  uint32_t rows[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int r = t - 3 + j;
+    rows[j] = *(const uint32_t*)((r >= 0 ? x + (int64_t)r * C : st + (int64_t)(3 + r) * C) + c);
+  }
+  const uint4 wv = *(const uint4*)(w + 4 * c);
+  uint32_t o = 0;
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const uint32_t wl = k ? wv.z : wv.x, wh = k ? wv.w : wv.y;
+    const float w0 = __uint_as_float(wl << 16), w1 = __uint_as_float(wl & 0xffff0000u);
+    const float w2 = __uint_as_float(wh << 16), w3 = __uint_as_float(wh & 0xffff0000u);
+    float f[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) f[j] = k ? __uint_as_float(rows[j] & 0xffff0000u) : __uint_as_float(rows[j] << 16);
+    const float r = __fadd_rn(__fadd_rn(w0 * f[0], w1 * f[1]), __fadd_rn(w2 * f[2], w3 * f[3]));
+    o |= (uint32_t)f32_to_bf16(__fmul_rn(r, sigmoid_f64(r))) << (16 * k);
+  }
+  *(uint32_t*)(out + (int64_t)t * C + c) = o;
+}
+__global__ __launch_bounds__(256) void conv1d_prefill_state_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ st,
+                                                                   uint16_t* __restrict__ stn, int C, int T) {
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 2;
+  if (c >= C) return;
+  uint32_t rows[3];
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    const int r = T - 3 + j;
+    rows[j] = *(const uint32_t*)((r >= 0 ? x + (int64_t)r * C : st + (int64_t)(3 + r) * C) + c);
+  }
+#pragma unroll
+  for (int j = 0; j < 3; j++) *(uint32_t*)(stn + (int64_t)j * C + c) = rows[j];
+}
+
+int launch_conv1d_prefill(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int T) {
+  BK_REQUIRE(x && st && w && out && st_new, "conv1d_prefill: null pointer");
+  BK_REQUIRE(C > 0 && C % 2 == 0 && T > 0 && T <= 65535, "conv1d_prefill: bad C=%d T=%d", C, T);
+  BK_REQUIRE(out != x, "conv1d_prefill: the output must not overwrite the input rows");
+  const int wgs = (C / 2 + 255) / 256;
+  hipLaunchKernelGGL(conv1d_prefill_kernel, dim3(wgs, T), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)st,
+                     (const uint16_t*)w, (uint16_t*)out, C);
+  hipLaunchKernelGGL(conv1d_prefill_state_kernel, dim3(wgs), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)st,
+                     (uint16_t*)st_new, C, T);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
 // ---------------------------------------------------------------- per-head norm (+ RoPE)
 // src/emitters.ts:123-147 emitQNorm / emitKNorm: bf16((x * rsqrt(mean(x^2) + 1e-6)) * (1 + w))
 // per head of HD values; the input rows are `in_stride` apart (2*HD for the interleaved

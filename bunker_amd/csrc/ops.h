@@ -20,6 +20,12 @@ int launch_dequant_legacy_i8(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_nibbles(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_dequant_f32(const void* blocks, void* out, int64_t nblocks);
 
+// gdn_prefill.hip
+size_t gdn_prefill_workspace_bytes(int Hg, int T);
+int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
+                       const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, void* workspace,
+                       size_t workspace_bytes, int Hg, int T);
+
 // quant_q4k.hip
 int launch_quantize_q4k(const void* w, int w_dtype, void* out, int64_t rows, int K);
 
@@ -51,6 +57,7 @@ int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void*
 int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows);
 int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t n);
 int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch);
+int launch_conv1d_prefill(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int T);
 int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD, int in_stride, int64_t in_bstride,
                     int batch, const float* cos_t, const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half,
                     int max_len);

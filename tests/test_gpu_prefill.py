@@ -1,0 +1,170 @@
+"""Prompt processing on the GPU against token-by-token runs of the CPU checker.
+
+conv1d_prefill and gdn_prefill must give the bits of T single-token steps; fa2_prefill must leave the same cache
+bytes and attention outputs within 2e-2; the whole prefill must leave the state and the last token's logits of a
+token-by-token run (the checker continues from the GPU's attention outputs, as in the decode tests), and decoding
+must continue from that state as if every prompt token had been decoded."""
+import numpy as np
+import pytest
+
+from bunker_amd import model, prefill, runner, synth, synth_model
+from bunker_amd import runtime as rt
+from bunker_amd.model import TINY
+
+pytestmark = pytest.mark.gpu
+
+bf = synth.f32_to_bf16
+f32 = synth.bf16_to_f32
+
+
+def _launch(spec, args):
+    k = rt.compileAndLoad(spec)
+    rc = rt.cuLaunch(k, [1, 1, 1], [128, 1, 1], args)
+    assert rc == 0, rt.last_error()
+    rt.cuSync()
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 7, 40])
+def test_conv1d_prefill_is_T_decode_steps(orc, T):
+    print(f"conv1d_prefill T={T}", flush=True)
+    g = synth.rng(800 + T)
+    C = 768
+    x = bf(g.standard_normal((T, C)).astype(np.float32))
+    st = bf(g.standard_normal((3, C)).astype(np.float32))
+    w = bf((g.standard_normal((C, 4)) * 0.5).astype(np.float32))
+    dx, dst, dw = rt.to_device(x), rt.to_device(st), rt.to_device(w)
+    dout = rt.cuAlloc(T * C * 2)
+    _launch(f"conv1d_prefill QKVD={C} T={T}", [dx, dst, dw, dout, dst])        # state updated in place
+    got = rt.from_device(dout, (T, C), np.uint16); gst = rt.from_device(dst, (3, C), np.uint16)
+    s = st
+    for t in range(T):
+        ref, s = orc.conv1d_decode(x[t], s, w)
+        assert np.array_equal(got[t], ref), t
+    assert np.array_equal(gst, s)
+    for p in (dx, dst, dw, dout):
+        rt.cuFree(p)
+
+
+@pytest.mark.parametrize("Hg,T", [(2, 1), (3, 5), (16, 33)])
+def test_gdn_prefill_is_T_decode_steps(orc, Hg, T):
+    print(f"gdn_prefill Hg={Hg} T={T}", flush=True)
+    g = synth.rng(820 + Hg + T)
+    C = 3 * Hg * 128
+    conv = bf(g.standard_normal((T, C)).astype(np.float32))
+    z = bf(g.standard_normal((T, Hg * 128)).astype(np.float32))
+    A_log = g.uniform(-2, 1, Hg).astype(np.float32)
+    dt_bias = bf(g.standard_normal(Hg).astype(np.float32))
+    a_p = g.standard_normal((T, Hg)).astype(np.float32); b_p = g.standard_normal((T, Hg)).astype(np.float32)
+    norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    S = (g.standard_normal((Hg, 128, 128)) * 0.02).astype(np.float32)
+    ptrs = [rt.to_device(a) for a in (conv, z, A_log, dt_bias, a_p, b_p, norm_w, S)]
+    dout = rt.cuAlloc(T * Hg * 128 * 2)
+    _launch(f"gdn_prefill LVH={Hg} T={T}", ptrs + [dout, ptrs[7]])                # S updated in place
+    got = rt.from_device(dout, (T, Hg * 128), np.uint16); gS = rt.from_device(ptrs[7], S.shape, np.float32)
+    s = S
+    for t in range(T):
+        ro, s = orc.gdn_step(conv[t], z[t], A_log, dt_bias, a_p[t], b_p[t], norm_w, s, Hg, rows_per_chain=16)
+        assert np.array_equal(got[t], ro), t
+    assert np.array_equal(gS.view(np.uint32), s.view(np.uint32))
+    for p in ptrs + [dout]:
+        rt.cuFree(p)
+
+
+@pytest.mark.parametrize("T,pos0", [(1, 0), (5, 0), (37, 12)])
+def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0):
+    print(f"fa2_prefill T={T} pos0={pos0}", flush=True)
+    g = synth.rng(840 + T)
+    NH, NKV, HD, HALF, MAXL = 16, 2, 256, 32, 128
+    pages = MAXL // 16
+    seq = 1                                       # the second sequence of a two-sequence cache
+    cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+    kc = bf(g.standard_normal((2 * pages, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((2 * pages, NKV, 16, HD)).astype(np.float32))
+    qgate = bf(g.standard_normal((T, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((T, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((T, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    table = (seq * pages + np.arange(pages)).astype(np.int32)
+    pos = (pos0 + np.arange(T)).astype(np.int32)
+    dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
+    dout = rt.cuAlloc(T * NH * HD * 2)
+    ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
+    _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T}", ptrs + [dkc, dvc, dout])
+    out = rt.from_device(dout, (T, NH, HD), np.uint16)
+    worst = 0.0
+    for t in range(T):
+        qn = orc.rope(orc.headnorm(qgate[t].ravel(), qw, NH, HD, 2 * HD), cos_t, sin_t, pos[t], NH, HD, HALF).reshape(1, NH, HD)
+        kn = orc.rope(orc.headnorm(k[t].ravel(), kw, NKV, HD, HD), cos_t, sin_t, pos[t], NKV, HD, HALF)
+        orc.kv_append(kn.reshape(NKV, HD), v[t], kc, vc, table, pos[t], NKV, HD, 16)
+        ro, _ = orc.attn_decode_paged(qn, kc, vc, table[None], np.array([pos[t] + 1], np.int32), 1, NH, NKV, HD, 16,
+                                      gate=qgate[t].ravel()[HD:], gate_bstride=0, gate_hstride=2 * HD)
+        worst = max(worst, float(np.abs(f32(out[t]).astype(np.float64) - f32(ro[0])).max()))
+    assert worst <= 2e-2, worst
+    kc_d = rt.from_device(dkc, kc.shape, np.uint16)
+    vc_d = rt.from_device(dvc, (2 * pages, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
+    assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
+    for p in ptrs + [dkc, dvc, dout]:
+        rt.cuFree(p)
+
+
+@pytest.mark.parametrize("n_prompt,chunk", [(23, 8), (9, 16)])
+def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
+    """TINY model, two sequences in the cache; the prompt goes to sequence 1 in chunks (with a shorter last chunk),
+    then both the checker and the GPU decode 3 more tokens from the state the prompt left."""
+    print(f"prefill n={n_prompt} chunk={chunk}", flush=True)
+    from oracle.model_ref import RefModel
+    D = TINY
+    B, seq = 2, 1
+    W = synth_model.synth_weights(D, seed=31)
+    S = synth_model.synth_state(D, B, seed=32)
+    for key in S:                                 # a fresh sequence: no conv history, S = 0
+        if key.endswith("conv_state") or key.endswith("s_state"):
+            S[key][seq] = 0
+    g = model.buildModelGraph(D, B)
+    env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+    prompt = synth.rng(33).integers(0, D.VOCAB, n_prompt).astype(np.int32)
+    captured = {}
+    pf = prefill.Prefill(D, env, chunk=chunk,
+                         on_attention=lambda layer, first, rows: captured.setdefault(layer, {}).update({first + i: r for i, r in enumerate(rows)}))
+    tok, val = pf.run(prompt, seq=seq, pos0=0)
+    glogits = rt.from_device(pf.d_logits, (D.VOCAB,), np.float32)
+
+    ref = RefModel(D, W, {k: np.asarray(v)[[seq]] for k, v in S.items()}, batch=1)
+    for t in range(n_prompt):
+        inj = {l: captured[l][t][None] for l in captured}
+        idx, rv, rlogits = ref.step([prompt[t]], [t], attn_override=inj)
+    assert max(ref.attn_err) <= 2e-2, max(ref.attn_err)
+    assert np.array_equal(glogits.view(np.uint32), rlogits[0].view(np.uint32)), \
+        f"{int((glogits != rlogits[0]).sum())} logits differ, worst {np.abs(glogits - rlogits[0]).max():.3e}"
+    assert tok == int(idx[0]) and np.float32(val).view(np.uint32) == rv[0].view(np.uint32)
+    for l in range(D.NL):
+        p = f"model.layers.{l}"
+        if not D.is_full_attention(l):
+            Sg = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32)
+            assert np.array_equal(Sg[seq].view(np.uint32), ref.S[f"{p}.s_state"][0].view(np.uint32)), p
+            assert np.array_equal(Sg[0], S[f"{p}.s_state"][0]), "the other sequence's state was touched"
+            cg = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)
+            assert np.array_equal(cg[seq], ref.S[f"{p}.conv_state"][0]), p
+        else:
+            kg = env.read_state(f"{p}.kv_k", (B,) + ref.S[f"{p}.kv_k"].shape[1:], np.uint16)
+            assert np.array_equal(kg[seq], ref.S[f"{p}.kv_k"][0]) and np.array_equal(kg[0], np.asarray(S[f"{p}.kv_k"])[0]), p
+            vg = env.read_state(f"{p}.kv_v", (B, D.MAX_LEN // 16, D.NKV, D.HD, 16), np.uint16).swapaxes(-1, -2)
+            assert np.array_equal(vg[seq], ref.S[f"{p}.kv_v"][0]), p
+    pf.close()
+
+    # decode continues from the prompt's state: sequence 1 from its first generated token at pos n_prompt
+    steps = 3
+    loop = runner.DeviceLoop(g, env, B, [7, tok], [40, n_prompt], max_steps=steps, partition=runner.fusedPartition(g))
+    fa_nodes = [n for n in g.nodes if n.op == "fa2_attn"]
+    fa_layers = [l for l in range(D.NL) if D.is_full_attention(l)]
+    toks, pos = np.array([tok], np.int32), np.array([n_prompt], np.int32)
+    for step in range(steps):
+        loop.step(1)
+        rt.cuSync()
+        inj = {l: rt.from_device(env.resolve(n.outputs[0].tensorName), (B, D.NH * D.HD), np.uint16)[[seq]]
+               for l, n in zip(fa_layers, fa_nodes)}
+        idx, rv, _ = ref.step(toks, pos, attn_override=inj)
+        gt, gv = loop.tokens()
+        assert gt[step][seq] == idx[0] and gv[step][seq].view(np.uint32) == rv[0].view(np.uint32), (step, gt[step], idx)
+        toks, pos = idx, pos + 1
+    assert max(ref.attn_err) <= 2e-2
+    env.close()
