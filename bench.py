@@ -116,8 +116,56 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
                          "launch": "hip graph replay" if use_graph else "eager", "launches_per_step": len(loop.launches), "partition": "fused" if fused else "node per kernel", "step_bytes": weight_bytes + state_bytes,
                          "hbm_floor_us": round(floor_us, 1), "frac_of_floor": round(floor_us / (ms * 1e3), 4),
                          "first_tokens": toks[:4, 0].tolist()}
+    # prompt processing on the same model (sequence 0 of the batch-1 environment, from an empty state)
+    from bunker_amd import prefill
+    n_prompt, chunk = 2048, 1024
+    pf = prefill.Prefill(D, envs[0], chunk=chunk)
+    prompt = ((9419 + 7919 * np.arange(n_prompt, dtype=np.int64)) % D.VOCAB).astype(np.int32)
+    pf.run(prompt[:chunk], 0, 0)           # loads the kernels
+    rt.cuSync()
+    t0 = time.perf_counter()
+    tok, _ = pf.run(prompt, 0, 0)
+    wall = time.perf_counter() - t0
+    pf.close()
+    out["prefill"] = {"prompt_tokens": n_prompt, "chunk": chunk, "tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
+                      "first_generated_token": tok}
     for env in envs:
         env.close()
+    return out
+
+
+def bench_load(rt, synth):
+    """Weights path: the Q4_K quantizer alone, and a bf16 safetensors file -> resident buffer (file read + PCIe)."""
+    import os
+    import tempfile
+    from bunker_amd import loader
+
+    rows, K = 32768, 2048
+    g = synth.rng(99)
+    w = synth.f32_to_bf16(g.standard_normal((rows, K), dtype=np.float32) * np.float32(0.02))
+    d = rt.to_device(w)
+    q = rt.cuAlloc(rows * (K // 256) * 144)
+    rt.quantize_q4k(d, q, rows, K, rt.BF16)
+    rt.cuSync()
+    e0, e1 = rt.Event().record(), rt.Event()
+    for _ in range(5):
+        rt.quantize_q4k(d, q, rows, K, rt.BF16)
+    e1.record(); rt.cuSync()
+    ms = e0.elapsed_ms(e1) / 5
+    rt.cuFree(d); rt.cuFree(q)
+    out = {"quantize_q4k": {"rows": rows, "K": K, "ms": round(ms, 3), "gelem_per_s": round(rows * K / ms / 1e6, 2)}}
+    tmp = tempfile.mkdtemp(prefix="bunker_bench_")
+    path = os.path.join(tmp, "w.safetensors")
+    loader.writeSafeTensors(path, {f"t{i}": ("BF16", w) for i in range(2)})
+    size = os.path.getsize(path)
+    loader.loadSafeTensors(path).free()
+    t0 = time.perf_counter()
+    f = loader.loadSafeTensors(path)
+    dt = time.perf_counter() - t0
+    f.free()
+    os.remove(path); os.rmdir(tmp)
+    out["load_safetensors"] = {"bytes": size, "ms": round(dt * 1e3, 1), "gb_per_s": round(size / dt / 1e9, 2),
+                               "note": "page-cache-warm file -> pinned staging -> device, PCIe included"}
     return out
 
 
@@ -237,7 +285,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sections", default="gemv,decode,kernels,gemm",
-                    help="comma list of gemv (headline, always on), decode, kernels, gemm, calib")
+                    help="comma list of gemv (headline, always on), decode (with prefill), kernels, gemm, calib, load (weights path)")
     ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
                     help="GEMV section. graph: the K launches of a shape replayed from one HIP graph (the device's own launch "
                          "rate); stream: K individual launches per shape queued from the host (used under rocprofv3)")
@@ -398,6 +446,8 @@ def main():
         out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
     if "gemm" in sections:
         out["gemm_bs32"] = bench_gemm(rt, synth, use_graph=not args.no_graph)
+    if "load" in sections:
+        out["weights_path"] = bench_load(rt, synth)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -73,29 +73,12 @@ constexpr int GEMM_MFMA_MIN_BATCH = 8;
 static int matmul_q8_1(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype, const void* res, int force) {
   const bool mfma = force >= 0 ? force != 0 : batch >= GEMM_MFMA_MIN_BATCH;
   if (!mfma) return launch_gemv_q4k_q8_1(W, xq, y, N, K, batch, out_dtype, res);
-  for (int b0 = 0; b0 < batch; b0 += 32) {
-    const int nb = batch - b0 < 32 ? batch - b0 : 32;
-    const size_t osz = out_dtype == DT_BF16 ? 2 : 4;
-    int rc = launch_gemm_q4k_q8_1_mfma(W, (const uint8_t*)xq + (size_t)b0 * (K / 32) * 36, (uint8_t*)y + (size_t)b0 * N * osz, N, K, nb,
-                                       out_dtype, res ? (const uint8_t*)res + (size_t)b0 * N * 2 : nullptr);
-    if (rc) return rc;
-  }
-  return BK_OK;
+  return launch_gemm_q4k_q8_1_mfma(W, xq, y, N, K, batch, out_dtype, res);
 }
-// several matrices over the same activation rows, 32 rows of the batch per launch
+// several matrices over the same activation rows (the kernel cuts the batch into 32-row tiles)
 static int matmul_group_mfma(const void* xq, int K, int batch, int G, const void* const* W, void* const* out, const void* const* res,
                              const int* N, const int* epi) {
-  for (int b0 = 0; b0 < batch; b0 += 32) {
-    const int nbat = batch - b0 < 32 ? batch - b0 : 32;
-    void* o[4]; const void* r[4];
-    for (int i = 0; i < G; i++) {
-      o[i] = (uint8_t*)out[i] + (size_t)b0 * N[i] * (epi[i] == 0 ? 4 : 2);
-      r[i] = res[i] ? (const uint8_t*)res[i] + (size_t)b0 * N[i] * 2 : nullptr;
-    }
-    int rc = launch_gemm_group_mfma((const uint8_t*)xq + (size_t)b0 * (K / 32) * 36, K, nbat, G, W, o, r, N, epi);
-    if (rc) return rc;
-  }
-  return BK_OK;
+  return launch_gemm_group_mfma(xq, K, batch, G, W, out, res, N, epi);
 }
 static int run_gemm(Kernel& k, const uint64_t* s) {
   const int N = (int)k.get("N", 0), K = (int)k.get("K", 0), batch = (int)k.get("batch", 1);

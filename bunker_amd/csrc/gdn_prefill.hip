@@ -6,7 +6,7 @@
 // Three kernels:
 //   prep     per (token, head): q^ = q * rsqrt(sum q^2 + 1e-6) / sqrt(128), k^ = k * rsqrt(sum k^2 + 1e-6),
 //            decay = exp(-exp(A_log) * softplus(a + dt_bias)), beta = sigmoid(b); all tokens in parallel
-//   scan     per (head, slab of 32 v columns): thread (row group kg, column c) owns rows 16*kg .. 16*kg+15 of
+//   scan     per (head, slab of 32 v columns): lane (row group kg, column c) owns rows 16*kg .. 16*kg+15 of
 //            one column; per token: decay, kS by an fmaf chain over the 16 rows and the sum of the 8 group
 //            results in order, delta, update, o the same way.  The order of every sum is the one the
 //            single-token kernel uses, so the results are equal to the bit.
@@ -61,73 +61,151 @@ __global__ __launch_bounds__(256) void gdn_prefill_prep_kernel(GdnPrefillArgs A)
   }
 }
 
-struct ScanIn {
+// The scan.  A workgroup owns 32 v columns of one head; its four wavefronts are independent: wavefront w owns columns
+// 8w .. 8w+7, lane (column c = lane / 8, row group kg = lane % 8) holds rows 16*kg .. 16*kg+15 of its column for the
+// whole run.  The eight row-group results of a column sit in eight neighbouring lanes, so they meet through lane
+// permutes (no LDS round trip, no barrier) and every lane adds them in group order.  The per-token operands (q^, k^,
+// v, decay, beta) are staged in LDS a block of GP_TB tokens at a time, the next block's global loads in flight while
+// the current block is computed; the workgroup synchronises once per block, for that hand-over only.
+constexpr int GP_TB = 16;
+
+struct TokenIn {
   float4 k[4], q[4];
   float v, decay, beta;
 };
-__device__ __forceinline__ void scan_load(ScanIn& in, const GdnPrefillArgs& A, int t, int h, int kg, int col) {
-  const int64_t th = (int64_t)t * A.Hg + h;
-  const float4* qp = (const float4*)(A.qk + th * 2 * GP_D + kg * GP_ROWS);
-  const float4* kp = (const float4*)(A.qk + (th * 2 + 1) * GP_D + kg * GP_ROWS);
+
+// Sum over the eight row groups of a column in group order, ((p0 + p1) + ... + p7): the lanes of the lower quad
+// hold p0..p3 themselves (quad broadcasts) and fetch p4..p7 from the upper quad (mirror within the eight lanes).
+// Lanes of the upper quad end up with another order of additions; they take the lower quad's result when `all`.
+template <bool ALL>
+__device__ __forceinline__ float group_sum8(float x, bool upper) {
+  const float a0 = dpp_f32<0x00>(x), a1 = dpp_f32<0x55>(x), a2 = dpp_f32<0xAA>(x), a3 = dpp_f32<0xFF>(x);   // own quad's four
+  const float b0 = dpp_f32<DPP_ROW_HALF_MIRROR>(a0), b1 = dpp_f32<DPP_ROW_HALF_MIRROR>(a1);                  // the other quad's
+  const float b2 = dpp_f32<DPP_ROW_HALF_MIRROR>(a2), b3 = dpp_f32<DPP_ROW_HALF_MIRROR>(a3);
+  const float s = ((((((a0 + a1) + a2) + a3) + b0) + b1) + b2) + b3;
+  if (!ALL) return s;                                         // valid in the lower quad only
+  const float lower = dpp_f32<DPP_ROW_HALF_MIRROR>(s);
+  return upper ? lower : s;
+}
+
+struct ScanState {
+  float S[GP_ROWS];
+};
+// one token of the recurrence for this lane's 16 rows of one column; returns the column's output (lower quad)
+__device__ __forceinline__ float scan_token(ScanState& st, const TokenIn& in, bool upper) {
+  const float kr[GP_ROWS] = {in.k[0].x, in.k[0].y, in.k[0].z, in.k[0].w, in.k[1].x, in.k[1].y, in.k[1].z, in.k[1].w,
+                             in.k[2].x, in.k[2].y, in.k[2].z, in.k[2].w, in.k[3].x, in.k[3].y, in.k[3].z, in.k[3].w};
+  const float qr[GP_ROWS] = {in.q[0].x, in.q[0].y, in.q[0].z, in.q[0].w, in.q[1].x, in.q[1].y, in.q[1].z, in.q[1].w,
+                             in.q[2].x, in.q[2].y, in.q[2].z, in.q[2].w, in.q[3].x, in.q[3].y, in.q[3].z, in.q[3].w};
+  float acc = 0.f;
 #pragma unroll
-  for (int r = 0; r < 4; r++) { in.q[r] = qp[r]; in.k[r] = kp[r]; }
-  in.v = bf16_to_f32(A.conv_out[(int64_t)t * 3 * A.Hg * GP_D + 2 * A.Hg * GP_D + h * GP_D + col]);
-  in.decay = A.gates[th * 2];
-  in.beta = A.gates[th * 2 + 1];
+  for (int r = 0; r < GP_ROWS; r++) {
+    st.S[r] *= in.decay;
+    acc = fmaf(kr[r], st.S[r], acc);
+  }
+  const float kS = group_sum8<true>(acc, upper);
+  const float d = (in.v - kS) * in.beta;
+  acc = 0.f;
+#pragma unroll
+  for (int r = 0; r < GP_ROWS; r++) {
+    st.S[r] = fmaf(kr[r], d, st.S[r]);
+    acc = fmaf(qr[r], st.S[r], acc);
+  }
+  return group_sum8<false>(acc, upper);
 }
 
 __global__ __launch_bounds__(256) void gdn_prefill_scan_kernel(GdnPrefillArgs A) {
-  __shared__ float part_k[GP_KG][GP_COLS], part_o[GP_KG][GP_COLS];
+  __shared__ __align__(16) float s_qk[2][GP_TB][2 * GP_D];     // q^ | k^ of each staged token
+  __shared__ float s_v[2][GP_TB][GP_COLS];
+  __shared__ float s_g[2][GP_TB][2];
   const int h = blockIdx.x, slab = blockIdx.y, tid = threadIdx.x;
-  const int kg = tid / GP_COLS, c = tid % GP_COLS;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int kg = lane & 7, c = wave * 8 + (lane >> 3);        // column within the slab
+  const bool upper = (lane & 4) != 0;
   const int col = slab * GP_COLS + c;
+  const int64_t KEYDIM = (int64_t)A.Hg * GP_D;
   const float* Sp = A.S_in + (int64_t)h * GP_D * GP_D + (int64_t)(kg * GP_ROWS) * GP_D + col;
-  float S[GP_ROWS];
+  ScanState st;
 #pragma unroll
-  for (int r = 0; r < GP_ROWS; r++) S[r] = Sp[(int64_t)r * GP_D];
+  for (int r = 0; r < GP_ROWS; r++) st.S[r] = Sp[(int64_t)r * GP_D];
 
-  ScanIn cur, nxt;
-  scan_load(cur, A, 0, h, kg, col);
-  for (int t = 0; t < A.T; t++) {
-    // the next token's operands are requested before this token's arithmetic (clamped: the last request is a repeat)
-    scan_load(nxt, A, t + 1 < A.T ? t + 1 : t, h, kg, col);
-    const float kr[GP_ROWS] = {cur.k[0].x, cur.k[0].y, cur.k[0].z, cur.k[0].w, cur.k[1].x, cur.k[1].y, cur.k[1].z, cur.k[1].w,
-                               cur.k[2].x, cur.k[2].y, cur.k[2].z, cur.k[2].w, cur.k[3].x, cur.k[3].y, cur.k[3].z, cur.k[3].w};
-    const float qr[GP_ROWS] = {cur.q[0].x, cur.q[0].y, cur.q[0].z, cur.q[0].w, cur.q[1].x, cur.q[1].y, cur.q[1].z, cur.q[1].w,
-                               cur.q[2].x, cur.q[2].y, cur.q[2].z, cur.q[2].w, cur.q[3].x, cur.q[3].y, cur.q[3].z, cur.q[3].w};
-    float acc = 0.f;
-#pragma unroll
-    for (int r = 0; r < GP_ROWS; r++) {
-      S[r] *= cur.decay;
-      acc = fmaf(kr[r], S[r], acc);
-    }
-    part_k[kg][c] = acc;
-    __syncthreads();
-    float kS = 0.f;
-#pragma unroll
-    for (int j = 0; j < GP_KG; j++) kS += part_k[j][c];
-    const float d = (cur.v - kS) * cur.beta;
-    acc = 0.f;
-#pragma unroll
-    for (int r = 0; r < GP_ROWS; r++) {
-      S[r] = fmaf(kr[r], d, S[r]);
-      acc = fmaf(qr[r], S[r], acc);
-    }
-    part_o[kg][c] = acc;
-    __syncthreads();
-    // part_k is rewritten only after the next token's first barrier has been passed by every thread, part_o only
-    // after its second: two buffers, two barriers per token
-    if (tid < GP_COLS) {
-      float o = 0.f;
-#pragma unroll
-      for (int j = 0; j < GP_KG; j++) o += part_o[j][tid];
-      A.o_raw[((int64_t)t * A.Hg + h) * GP_D + slab * GP_COLS + tid] = o;
-    }
-    cur = nxt;
+  // staging: thread tid moves float4 pieces tid, tid+256, tid+512, tid+768 of the block's 16 x 256 floats of q^/k^,
+  // two v values and one gate value; token indices past the end repeat the last token (never consumed)
+  float4 gq0, gq1, gq2, gq3;
+  uint32_t gv;
+  float gg;
+#define GP_STAGE_LOAD(T0)                                                                                              \
+  {                                                                                                                    \
+    const float* qk_h = A.qk + (int64_t)h * 2 * GP_D + (tid % 64) * 4;                                                 \
+    const int64_t tstride = (int64_t)A.Hg * 2 * GP_D;                                                                  \
+    gq0 = *(const float4*)(qk_h + min((T0) + tid / 64, A.T - 1) * tstride);                                            \
+    gq1 = *(const float4*)(qk_h + min((T0) + 4 + tid / 64, A.T - 1) * tstride);                                        \
+    gq2 = *(const float4*)(qk_h + min((T0) + 8 + tid / 64, A.T - 1) * tstride);                                        \
+    gq3 = *(const float4*)(qk_h + min((T0) + 12 + tid / 64, A.T - 1) * tstride);                                       \
+    gv = *(const uint32_t*)(A.conv_out + (int64_t)min((T0) + tid / 16, A.T - 1) * 3 * KEYDIM + 2 * KEYDIM + h * GP_D + \
+                            slab * GP_COLS + (tid % 16) * 2);                                                          \
+    gg = A.gates[((int64_t)min((T0) + (tid & 31) / 2, A.T - 1) * A.Hg + h) * 2 + (tid & 1)];                           \
   }
+#define GP_STAGE_STORE(BUF)                                                              \
+  {                                                                                      \
+    *(float4*)&s_qk[BUF][tid / 64][(tid % 64) * 4] = gq0;                                \
+    *(float4*)&s_qk[BUF][4 + tid / 64][(tid % 64) * 4] = gq1;                            \
+    *(float4*)&s_qk[BUF][8 + tid / 64][(tid % 64) * 4] = gq2;                            \
+    *(float4*)&s_qk[BUF][12 + tid / 64][(tid % 64) * 4] = gq3;                           \
+    s_v[BUF][tid / 16][(tid % 16) * 2] = __uint_as_float(gv << 16);                      \
+    s_v[BUF][tid / 16][(tid % 16) * 2 + 1] = __uint_as_float(gv & 0xffff0000u);          \
+    if (tid < 32) s_g[BUF][tid / 2][tid & 1] = gg;                                       \
+  }
+  auto token_read = [&](TokenIn& in, int buf, int t) {
+    const float4* qp = (const float4*)&s_qk[buf][t][kg * GP_ROWS];
+    const float4* kp = (const float4*)&s_qk[buf][t][GP_D + kg * GP_ROWS];
+#pragma unroll
+    for (int r = 0; r < 4; r++) { in.q[r] = qp[r]; in.k[r] = kp[r]; }
+    in.v = s_v[buf][t][c];
+    in.decay = s_g[buf][t][0];
+    in.beta = s_g[buf][t][1];
+  };
+
+  GP_STAGE_LOAD(0)
+  GP_STAGE_STORE(0)
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = 0; t0 < A.T; t0 += GP_TB) {
+    const int nt = min(GP_TB, A.T - t0);
+    GP_STAGE_LOAD(t0 + GP_TB)                                  // next block (clamped), in flight during this block
+    float* orow = A.o_raw + ((int64_t)t0 * A.Hg + h) * GP_D + col;
+    const int64_t ostride = (int64_t)A.Hg * GP_D;
+    if (nt == GP_TB) {
+      // a full block, unrolled: two operand sets alternate, the next token's LDS reads are issued ahead of the
+      // arithmetic of the current one, and the output chain of one token overlaps the kS chain of the next
+      TokenIn in0, in1;
+      token_read(in0, buf, 0);
+#pragma unroll
+      for (int tt = 0; tt < GP_TB; tt += 2) {
+        token_read(in1, buf, tt + 1);
+        const float o0 = scan_token(st, in0, upper);
+        if (kg == 0) orow[(int64_t)tt * ostride] = o0;
+        if (tt + 2 < GP_TB) token_read(in0, buf, tt + 2);
+        const float o1 = scan_token(st, in1, upper);
+        if (kg == 0) orow[(int64_t)(tt + 1) * ostride] = o1;
+      }
+    } else {
+      for (int tt = 0; tt < nt; tt++) {
+        TokenIn in;
+        token_read(in, buf, tt);
+        const float o = scan_token(st, in, upper);
+        if (kg == 0) orow[(int64_t)tt * ostride] = o;
+      }
+    }
+    GP_STAGE_STORE(buf ^ 1)    // nobody reads buf ^ 1 in this block; the barrier below publishes it and retires buf
+    __syncthreads();
+    buf ^= 1;
+  }
+#undef GP_STAGE_LOAD
+#undef GP_STAGE_STORE
   float* So = A.S_out + (int64_t)h * GP_D * GP_D + (int64_t)(kg * GP_ROWS) * GP_D + col;
 #pragma unroll
-  for (int r = 0; r < GP_ROWS; r++) So[(int64_t)r * GP_D] = S[r];
+  for (int r = 0; r < GP_ROWS; r++) So[(int64_t)r * GP_D] = st.S[r];
 }
 
 __global__ __launch_bounds__(128) void gdn_prefill_outnorm_kernel(GdnPrefillArgs A) {

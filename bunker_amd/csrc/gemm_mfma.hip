@@ -10,6 +10,7 @@
 // (every term exact, ~1e-16 accumulation error, one rounding to f32), so the batched
 // path returns the same bits as the batch-1 path:
 //   y[b, n] = sum_blk ( d * sum_j d8_j[b] * (sc_j * I_j) - dmin * sum_j m_j * s8_j[b] )
+// Batches of more than 32 rows are cut into 32-row tiles along blockIdx.y (one launch, every tile its own workgroup).
 // A workgroup owns one 32 x 32 output tile; its NW wavefronts split K by super-block (wave w takes
 // blocks w, w + NW, ...) and add their double partials in wave order through LDS at the end.  The
 // int8 activation operand is read straight from the Q8_1 rows (16-byte pieces, L2-resident); only
@@ -52,8 +53,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
   const uint16_t* __restrict__ res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
   const int N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
   const int EPI = s3 ? A.g[3].epi : s2 ? A.g[2].epi : s1 ? A.g[1].epi : A.g[0].epi;
-  const uint8_t* __restrict__ xq = A.xq;
-  const int nb = A.nb, B = A.B;
+  const int nb = A.nb;
+  const int b0 = blockIdx.y * 32;                     // first batch row of this tile
+  const int B = min(32, A.B - b0);
+  const uint8_t* __restrict__ xq = A.xq + (int64_t)b0 * nb * 8 * 36;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -165,7 +168,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
     for (int r = 0; r < 16; r++) {
       const int b = mfma32_row(r, half);
       if (b >= B) continue;
-      const int64_t o = (int64_t)b * N + n0 + col;
+      const int64_t o = (int64_t)(b0 + b) * N + n0 + col;
       const float v = (float)acc[r];
       if (EPI == GEPI_F32) ((float*)out)[o] = v;
       else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
@@ -180,7 +183,7 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
                            const void* const* res, const int* N, const int* epi) {
   BK_REQUIRE(xq && ngroups >= 1 && ngroups <= 4, "gemm_q4k_q8_1_mfma: bad arguments");
   BK_REQUIRE(K > 0 && K % 256 == 0, "gemm_q4k_q8_1_mfma: K=%d must be a positive multiple of 256", K);
-  BK_REQUIRE(batch >= 1 && batch <= 32, "gemm_q4k_q8_1_mfma: batch=%d must be 1..32", batch);
+  BK_REQUIRE(batch >= 1 && batch <= 32 * 65535, "gemm_q4k_q8_1_mfma: bad batch=%d", batch);
   BK_REQUIRE(((uintptr_t)xq & 3) == 0, "gemm_q4k_q8_1_mfma: xq must be 4-byte aligned");
   MfmaArgs A{};
   A.xq = (const uint8_t*)xq; A.nb = K / 256; A.B = batch;
@@ -196,13 +199,15 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   for (int i = ngroups; i < 5; i++) A.tile_first[i] = tiles;
   // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
   // and two ways when the tiles alone fill the chip many times over (lm_head)
+  const int btiles = (batch + 31) / 32;
+  const int64_t wgs = (int64_t)tiles * btiles;
   int nw = g_tune_gemm_nw;
   if (nw <= 0) {
     nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
-    if (tiles <= num_cus() / 2 && A.nb >= 8) nw = 8;          // few tiles: one super-block per wave
-    if (tiles >= 8 * num_cus() && nw > 2) nw = 2;
+    if (wgs <= num_cus() / 2 && A.nb >= 8) nw = 8;          // few tiles: one super-block per wave
+    if (wgs >= 8 * num_cus() && nw > 2) nw = 2;
   }
-  const dim3 grid(tiles);
+  const dim3 grid(tiles, btiles);
   if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8>), grid, dim3(512), 0, stream(), A);
   else if (nw >= 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4>), grid, dim3(256), 0, stream(), A);
   else if (nw >= 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2>), grid, dim3(128), 0, stream(), A);

@@ -45,7 +45,7 @@ def test_conv1d_prefill_is_T_decode_steps(orc, T):
         rt.cuFree(p)
 
 
-@pytest.mark.parametrize("Hg,T", [(2, 1), (3, 5), (16, 33)])
+@pytest.mark.parametrize("Hg,T", [(2, 1), (3, 5), (4, 32), (16, 33)])
 def test_gdn_prefill_is_T_decode_steps(orc, Hg, T):
     print(f"gdn_prefill Hg={Hg} T={T}", flush=True)
     g = synth.rng(820 + Hg + T)

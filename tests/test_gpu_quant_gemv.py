@@ -272,7 +272,7 @@ def test_gemm_op_launch_surface(orc, dev):
 
 
 @pytest.mark.parametrize("N,K,B", [(6144, 2048, 32), (2048, 6144, 32), (16, 2048, 32), (100, 768, 7), (2048, 4096, 17),
-                                   (4096, 2048, 40)])
+                                   (4096, 2048, 40), (520, 512, 100)])
 def test_gemm_mfma_equals_gemv_and_oracle(orc, dev, N, K, B):
     """Batched int8-MFMA matmul: same bits as the GEMV path and as the host loop in double, for every batch row."""
     print(f"gemm mfma N={N} K={K} B={B}", flush=True)
