@@ -41,10 +41,13 @@ struct MfmaArgs {
   int nb, B;
 };
 
-template <int NW>
+template <int NW, bool PF>
 __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
-  __shared__ double2 lds_ds[NW][8][32];          // (d8, s8) of activation block (j, b) of the wave's current super-block, as doubles
-  __shared__ double lds_acc[NW > 1 ? 16 * 64 : 1];
+  // one buffer, two uses: during the K loop (d8, s8) of activation block (j, b) of each wave's current super-block, as
+  // doubles [NW][8][32]; afterwards the waves' partial sums [NW][16][64]
+  constexpr int LDS_DS_BYTES = NW * 8 * 32 * 16, LDS_PART_BYTES = NW > 1 ? NW * 16 * 64 * 8 : 0;
+  __shared__ __align__(16) unsigned char lds_raw[LDS_DS_BYTES > LDS_PART_BYTES ? LDS_DS_BYTES : LDS_PART_BYTES];
+  double2 (*lds_ds)[8][32] = (double2 (*)[8][32])lds_raw;
 
   const int tile = blockIdx.x;
   const bool s1 = tile >= A.tile_first[1], s2 = tile >= A.tile_first[2], s3 = tile >= A.tile_first[3];
@@ -71,12 +74,17 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0;
 
-  for (int blk = wave; blk < nb; blk += NW) {
-    // weights of this lane's row: header + its half of every 32-byte nibble group
-    const uint4 hdr = *(const uint4*)(wrow + blk * 144);
-    uint4 qs[4];
+  // weights of this lane's row: header + its half of every 32-byte nibble group.  A wave with several super-blocks
+  // requests the next one's weights (the HBM round trip) behind the current one's activation loads, so that only the
+  // first super-block waits for memory; the requests are unconditional (clamped) to keep the waits countable.
+  uint4 hdr_n, qs_n[4];
+  {
+    const uint8_t* wp = wrow + min(wave, nb - 1) * 144;
+    hdr_n = *(const uint4*)wp;
 #pragma unroll
-    for (int g = 0; g < 4; g++) qs[g] = *(const uint4*)(wrow + blk * 144 + 16 + 32 * g + 16 * half);
+    for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
+  }
+  for (int blk = wave; blk < nb; blk += NW) {
     // activations: the lane's 16 int8 of each of the 8 sub-blocks (4-byte aligned 16-byte loads)
     uint4 xa4[8];
 #pragma unroll
@@ -84,14 +92,29 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
       const uint32_t* p = (const uint32_t*)(xrow + (int64_t)(blk * 8 + j) * 36);
       xa4[j] = make_uint4(p[0], p[1], p[2], p[3]);
     }
+    uint32_t dsraw[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int t = lane + 64 * i;
+      dsraw[i] = *(const uint32_t*)(xq + (int64_t)min(t >> 3, B - 1) * xrow_bytes + (int64_t)(blk * 8 + (t & 7)) * 36 + 32);
+    }
+    const uint4 hdr = hdr_n;
+    uint4 qs[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) qs[g] = qs_n[g];
+    if (PF) {
+      const uint8_t* wp = wrow + min(blk + NW, nb - 1) * 144;
+      hdr_n = *(const uint4*)wp;
+#pragma unroll
+      for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
+    }
     // scales of the 32 x 8 activation blocks of this super-block -> LDS of this wave, 4 per lane
     __builtin_amdgcn_wave_barrier();     // the previous super-block's scales have been consumed by every lane
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int t = lane + 64 * i;
-      const int b = t >> 3, j = t & 7;
-      const uint32_t ds = *(const uint32_t*)(xq + (int64_t)min(b, B - 1) * xrow_bytes + (int64_t)(blk * 8 + j) * 36 + 32);
-      lds_ds[wave][j][b] = make_double2((double)half_to_f32((uint16_t)(ds & 0xffffu)), (double)half_to_f32((uint16_t)(ds >> 16)));
+      const uint32_t ds = dsraw[i];
+      lds_ds[wave][t & 7][t >> 3] = make_double2((double)half_to_f32((uint16_t)(ds & 0xffffu)), (double)half_to_f32((uint16_t)(ds >> 16)));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -103,14 +126,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
     const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
     const uint32_t m_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
 
-    double sblk[16], mblk[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) { sblk[r] = 0.0; mblk[r] = 0.0; }
-
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const int g = j >> 1;
-      const uint4 q = qs[g];
+    const float dmin_neg = -dmin;
+    // A = activations (M = batch row), B = weights (N = weight row): result[r] = I_j[b = mfma32_row(r), n = col]
+    auto dots = [&](int j) {
+      const uint4 q = qs[j >> 1];
       i32x4_t wb;
       if (j & 1) {
         wb = (i32x4_t){(int)((q.x >> 4) & 0x0f0f0f0fu), (int)((q.y >> 4) & 0x0f0f0f0fu), (int)((q.z >> 4) & 0x0f0f0f0fu),
@@ -122,62 +141,80 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
       i32x16_t c;
 #pragma unroll
       for (int r = 0; r < 16; r++) c[r] = 0;
-      // A = activations (M = batch row), B = weights (N = weight row): c[r] = I_j[b = mfma32_row(r), n = col]
-      c = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb, c, 0, 0, 0);
-      const int sc = (int)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xffu);
-      const double mj = (double)(((j < 4 ? m_lo : m_hi) >> (8 * (j & 3))) & 0xffu);
-      // the scales of eight outputs are requested together and consumed as they arrive (LDS returns in order);
-      // without the scheduling fences the compiler pairs every read with its use and exposes the LDS latency 16 times
+      return __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb, c, 0, 0, 0);
+    };
+    // The fold runs as a pipeline over the 16 groups (sub-block j, eight of the lane's sixteen outputs): the activation
+    // scales of group g+1 are requested from LDS and the matrix instruction of sub-block j+1 is issued before group g
+    // is folded, so neither latency is exposed.  Per sub-block the lane's row contributes two factors, both exact in f32
+    // (11-bit x 6-bit): d * sc_j and -dmin * m_j; every term (d*sc_j) * (d8 * I) and (-dmin*m_j) * s8 is exact in double.
+    double2 dsa[8], dsb[8];
 #pragma unroll
-      for (int r0 = 0; r0 < 16; r0 += 8) {
-        double2 ds8[8];
+    for (int r = 0; r < 8; r++) dsa[r] = lds_ds[wave][0][mfma32_row(r, half)];
+    i32x16_t c = dots(0), cn = c;
 #pragma unroll
-        for (int r = 0; r < 8; r++) ds8[r] = lds_ds[wave][j][mfma32_row(r0 + r, half)];
-        __builtin_amdgcn_sched_barrier(0);
+    for (int g = 0; g < 16; g++) {
+      const int j = g >> 1, r0 = 8 * (g & 1);
+      double2 (&cur)[8] = (g & 1) ? dsb : dsa;
+      double2 (&nxt)[8] = (g & 1) ? dsa : dsb;
+      if (g + 1 < 16) {
 #pragma unroll
-        for (int r = 0; r < 8; r++) {
-          const int p = __mul24(sc, c[r0 + r]);                     // 6-bit x 17-bit: exact
-          sblk[r0 + r] = fma(ds8[r].x, (double)p, sblk[r0 + r]);
-          mblk[r0 + r] = fma(mj, ds8[r].y, mblk[r0 + r]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        for (int r = 0; r < 8; r++) nxt[r] = lds_ds[wave][(g + 1) >> 1][mfma32_row(8 * ((g + 1) & 1) + r, half)];
       }
-    }
-    const double dd = (double)d, dm = (double)dmin;
+      if (!(g & 1) && j + 1 < 8) cn = dots(j + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      const double dsc = (double)(d * (float)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xffu));
+      const double dmm = (double)(dmin_neg * (float)(((j < 4 ? m_lo : m_hi) >> (8 * (j & 3))) & 0xffu));
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] += dd * sblk[r] - dm * mblk[r];
+      for (int r = 0; r < 8; r++) {
+        const double t = cur[r].x * (double)c[r0 + r];            // d8 * I: 11-bit x 17-bit, exact
+        acc[r0 + r] = fma(dsc, t, acc[r0 + r]);
+        acc[r0 + r] = fma(dmm, cur[r].y, acc[r0 + r]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (g & 1) c = cn;
+    }
+    if (!PF) {
+      const uint8_t* wp = wrow + min(blk + NW, nb - 1) * 144;
+      hdr_n = *(const uint4*)wp;
+#pragma unroll
+      for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
+    }
   }
 
+  auto store = [&](int r, double total) {
+    const int b = mfma32_row(r, half);
+    if (n0 + col >= N || b >= B) return;
+    const int64_t o = (int64_t)(b0 + b) * N + n0 + col;
+    const float v = (float)total;
+    if (EPI == GEPI_F32) ((float*)out)[o] = v;
+    else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
+    else ((uint16_t*)out)[o] = f32_to_bf16(bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(res[o]));
+  };
   if (NW > 1) {
-    // partial sums meet in wave order; the last wave ends up with the totals
-    for (int w = 0; w < NW; w++) {
-      if (wave == w) {
+    // every wave leaves its 16 partial sums per lane in LDS; then wave w finishes outputs r = w*16/NW .. of every lane:
+    // the partials are added in wave order, and the conversions and stores are spread over all waves
+    double* part = (double*)lds_raw;
+    __syncthreads();                       // all waves are done with the activation scales that share the buffer
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          if (w > 0) acc[r] += lds_acc[r * 64 + lane];
-          if (w < NW - 1) lds_acc[r * 64 + lane] = acc[r];
-        }
-      }
-      if (w < NW - 1) __syncthreads();
-    }
-    if (wave != NW - 1) return;
-  }
-
-  if (n0 + col < N) {
+    for (int r = 0; r < 16; r++) part[(wave * 16 + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    constexpr int R = 16 / NW;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int b = mfma32_row(r, half);
-      if (b >= B) continue;
-      const int64_t o = (int64_t)(b0 + b) * N + n0 + col;
-      const float v = (float)acc[r];
-      if (EPI == GEPI_F32) ((float*)out)[o] = v;
-      else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
-      else ((uint16_t*)out)[o] = f32_to_bf16(bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(res[o]));
+    for (int rr = 0; rr < R; rr++) {
+      const int r = wave * R + rr;
+      double t = part[r * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < NW; w++) t += part[(w * 16 + r) * 64 + lane];
+      store(r, t);
     }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) store(r, acc[r]);
   }
 }
 
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
+int g_tune_gemm_pf = -1;     // next-block weight prefetch: 0 off, 1 on, -1 = chosen from the shape
 
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi) {
@@ -204,14 +241,24 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   int nw = g_tune_gemm_nw;
   if (nw <= 0) {
     nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
-    if (wgs <= num_cus() / 2 && A.nb >= 8) nw = 8;          // few tiles: one super-block per wave
+    if (wgs <= num_cus() + num_cus() / 4 && A.nb >= 8) nw = 8;          // about a tile per CU: one super-block per wave
     if (wgs >= 8 * num_cus() && nw > 2) nw = 2;
   }
+  nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
+  // next-block weight prefetch for waves with several super-blocks; not when the chip is full of tiles anyway
+  // (it costs 20 registers: two waves per SIMD instead of three)
+  const bool pf = g_tune_gemm_pf >= 0 ? g_tune_gemm_pf != 0 : ((A.nb + nw - 1) / nw >= 2 && wgs * nw <= 8 * num_cus());
   const dim3 grid(tiles, btiles);
-  if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8>), grid, dim3(512), 0, stream(), A);
-  else if (nw >= 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4>), grid, dim3(256), 0, stream(), A);
-  else if (nw >= 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2>), grid, dim3(128), 0, stream(), A);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1>), grid, dim3(64), 0, stream(), A);
+#define BK_GEMM_LAUNCH(NWV)                                                                                             \
+  {                                                                                                                     \
+    if (pf) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<NWV, true>), grid, dim3(64 * NWV), 0, stream(), A);           \
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<NWV, false>), grid, dim3(64 * NWV), 0, stream(), A);             \
+  }
+  if (nw == 8) BK_GEMM_LAUNCH(8)
+  else if (nw == 4) BK_GEMM_LAUNCH(4)
+  else if (nw == 2) BK_GEMM_LAUNCH(2)
+  else BK_GEMM_LAUNCH(1)
+#undef BK_GEMM_LAUNCH
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
