@@ -91,7 +91,8 @@ static int run_gemm(Kernel& k, const uint64_t* s) {
 // consumers (src/model.ts:65-73, 161-191 as one launch; the node-by-node result to the bit).
 // params: K, pro (0: x is Q8_1, 1: x is bf16, 2: x is bf16 and goes through rmsnorm with norm_w first),
 //         G matrices with N<i>, epi<i> (0: f32, 1: bf16, 2: bf16(bf16(y) + residual)), swiglu=0|1 (G=2: gate, up), batch=1
-// slots:  x, [norm_w if pro=2], then per matrix: W, [residual if epi=2], out      (swiglu: x, [norm_w], Wg, Wu, out)
+// slots:  x, [norm_w if pro=2], then per matrix: W, [residual if epi=2], out      (swiglu: x, [norm_w], Wg, Wu, out
+//         [, out as Q8_1 blocks when q8out=1: batch >= 8 only])
 // Shapes outside the fused kernel (K not 2048/4096/6144, batch >= 8) run as rmsnorm/quantize, matmuls, swiglu.
 static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   const int K = (int)k.get("K", 0), pro = (int)k.get("pro", 0), G = (int)k.get("G", 1), batch = (int)k.get("batch", 1);
@@ -110,6 +111,7 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
     out[i] = P<void>(s[si++]);
   }
   if (swiglu) out[0] = P<void>(s[si++]);
+  void* q8out = swiglu && k.get("q8out", 0) ? P<void>(s[si++]) : nullptr;      // composed path only (build_gemv_fused checks)
   if (gemv_fused_fast_path(K, batch, swiglu)) return launch_gemv_fused(pro, x, nw, K, batch, G, W, out, res, N, epi, swiglu);
   int rc;
   const void* xq = x;
@@ -125,6 +127,7 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
       if ((rc = matmul_q8_1(W[0], xq, g, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
       if ((rc = matmul_q8_1(W[1], xq, u, N[0], K, batch, DT_F32, nullptr, -1))) return rc;
     }
+    if (q8out) return launch_swiglu_q8_1(g, u, out[0], q8out, (int64_t)batch * N[0]);
     return launch_elementwise(EW_SWIGLU_OP, g, u, out[0], (int64_t)batch * N[0]);
   }
   if (batch >= GEMM_MFMA_MIN_BATCH) return matmul_group_mfma(xq, K, batch, G, W, out, res, N, epi);
@@ -153,6 +156,11 @@ static int build_gemv_fused(Kernel& k) {
     nslots += swiglu ? 1 : (e == 2 ? 3 : 2);
   }
   if (swiglu) nslots += 1;
+  if (k.get("q8out", 0)) {
+    BK_REQUIRE(swiglu && !gemv_fused_fast_path((int)K, (int)batch, true) && k.get("N0", 0) % 32 == 0,
+               "gemv_fused: q8out=1 (SwiGLU result also as Q8_1) is served by the batched path only (batch >= 8), N a multiple of 32");
+    nslots += 1;
+  }
   if ((rc = alloc_scratch(k, (size_t)(batch * (K / 32) * 36) + (swiglu ? (size_t)(2 * batch * k.get("N0", 0) * 4) : 0)))) return rc;
   k.run = run_gemv_fused; k.nslots = nslots;
   return BK_OK;
@@ -196,11 +204,13 @@ static int run_gdn(Kernel& k, const uint64_t* s) {
 }
 // ---- op: gdn_conv = conv1d_decode + gdn_delta_rule in one launch (the conv output never reaches memory)
 // slots: qkv, conv_state_in, conv_w, z, A_log, dt_bias, a_p, b_p, norm_w, s_state_in, out, conv_state_new, s_state_new
-// params: LVH (= number of key heads), batch=1
+// params: LVH (= number of key heads), batch=1, q8out=0 (1: one more slot, the output again as Q8_1 blocks [batch, ZD/32]
+//         for the out_proj matmul, written by the same threads that write the bf16 output)
 static int run_gdn_conv(Kernel& k, const uint64_t* s) {
   return launch_gdn_conv_fused(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<float>(s[4]), P<void>(s[5]),
                                P<float>(s[6]), P<float>(s[7]), P<float>(s[8]), P<float>(s[9]), P<void>(s[10]), P<void>(s[11]),
-                               P<float>(s[12]), (int)k.get("LVH", 0), (int)k.get("batch", 1));
+                               P<float>(s[12]), k.get("q8out", 0) ? P<void>(s[13]) : nullptr, (int)k.get("LVH", 0),
+                               (int)k.get("batch", 1));
 }
 // ---- ops: qnorm (q-gate buffer, w, out; NH heads, input rows 2*HD apart), knorm (k, w, out; NKV heads)
 static int run_qnorm(Kernel& k, const uint64_t* s) {
@@ -243,7 +253,7 @@ static int run_fa2(Kernel& k, const uint64_t* s) {
 // ---- op: fa2_fused = qnorm, rope, knorm, ropek, fa2_attn of src/model.ts:126-157 as three launches
 // (norm + rotation + cache append; split attention; merge with the output gate).
 // slots: qgate (q_proj output, [q | gate] per head), k, v, q_norm.weight, k_norm.weight, rope_cos, rope_sin, pos,
-//        kv_k, kv_v, out         params: HD, NH, NKV, MAX_LEN, ROT_HALF, batch=1, pos_dev=0
+//        kv_k, kv_v, out [, out as Q8_1 blocks when q8out=1]        params: HD, NH, NKV, MAX_LEN, ROT_HALF, batch=1, pos_dev=0, q8out=0
 static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   const bool dev = k.get("pos_dev", 0) != 0;
   const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0), NKV = (int)k.get("NKV", 0), batch = (int)k.get("batch", 1);
@@ -257,7 +267,7 @@ static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   if (rc) return rc;
   return launch_attn_decode(qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, pos_dev, pos, 1, max_len, P<uint16_t>(s[0]) + HD,
                             (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - (size_t)batch * NH * HD * 2,
-                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
+                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0), k.get("q8out", 0) ? P<void>(s[11]) : nullptr);
 }
 // ---- prefill ops: T consecutive tokens of ONE sequence per launch (rows of the activation buffers = tokens)
 // conv1d_prefill   slots: qkv [T, QKVD], conv_state_in [3, QKVD], weight, out [T, QKVD], conv_state_new    params: QKVD, T
@@ -324,7 +334,7 @@ static int build_kernel(Kernel& k) {
     }
     if (k.op == "gdn_delta_rule" || k.op == "gdn_conv")
       BK_REQUIRE(k.get("LKD", 128) == 128 && k.get("LVD", 128) == 128, "gdn_delta_rule: dk = dv = 128 only");
-    k.run = sp.run; k.nslots = sp.nslots;
+    k.run = sp.run; k.nslots = sp.nslots + (k.op == "gdn_conv" && k.get("q8out", 0) ? 1 : 0);
     return BK_OK;
   }
   if (k.op == "fa2_attn") {
@@ -345,7 +355,7 @@ static int build_kernel(Kernel& k) {
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
     const size_t qbytes = (size_t)batch * k.get("NH", 0) * k.get("HD", 0) * 2;
     if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(batch, NKV, splits) : 0)))) return rc;
-    k.run = run_fa2_fused; k.nslots = 11;
+    k.run = run_fa2_fused; k.nslots = 11 + (k.get("q8out", 0) ? 1 : 0);
     return BK_OK;
   }
   if (k.op == "conv1d_prefill") {

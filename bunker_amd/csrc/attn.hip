@@ -41,6 +41,7 @@ struct AttnArgs {
   const int32_t* ctx_len;     // int32 [B]; null = ctx_scalar for every sequence; ctx_add is added to either
   const uint16_t* gate;       // bf16 or null: gate of (b, head, i) at gate[b*gate_bstride + head*gate_hstride + i]
   uint16_t* out;              // bf16 [B, NH, 256]
+  uint8_t* out_q8;            // optional: the same outputs as Q8_1 blocks [B, NH*256/32] (written by the merge kernel)
   float* lse;                 // f32 [B, NH] or null
   float* part_o;              // f32 [B, NKV, splits, 16, 256] unnormalised partial outputs
   float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
@@ -276,7 +277,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
     const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
     o = __fmul_rn(o, sigmoid_f64(gv));
   }
-  A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
+  const uint16_t ob = f32_to_bf16(o);
+  A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = ob;
+  if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (((int64_t)b * A.NH + head) * (ATT_HD / 32) + (d >> 5)) * 36, d & 31);
   if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = M + logf(L);
 }
 
@@ -299,7 +302,7 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits) {
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8) {
   BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
@@ -318,7 +321,7 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   AttnArgs A{};
   A.q = (const uint16_t*)q; A.kc = (const uint16_t*)kc; A.vc = (const uint16_t*)vc;
   A.block_table = block_table; A.ctx_len = ctx_len; A.gate = (const uint16_t*)gate;
-  A.out = (uint16_t*)out; A.lse = lse;
+  A.out = (uint16_t*)out; A.lse = lse; A.out_q8 = splits > 1 ? (uint8_t*)out_q8 : nullptr;
   A.gate_bstride = gate_bstride; A.gate_hstride = gate_hstride;
   A.bt_stride = bt_stride; A.ctx_scalar = ctx_scalar; A.ctx_add = ctx_add; A.NH = NH; A.NKV = NKV; A.G = NH / NKV;
   A.splits = splits; A.pages_per_split = (pages + splits - 1) / splits;
@@ -336,6 +339,8 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
     hipLaunchKernelGGL(attn_decode_kernel<0>, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
   if (splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, batch), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
+  // a single split writes its output from the attention kernel itself; its Q8_1 copy then takes the stand-alone quantizer
+  if (splits == 1 && out_q8) return launch_quantize_q8_1(out, DT_BF16, out_q8, NH * HD, batch);
   return BK_OK;
 }
 

@@ -194,6 +194,21 @@ __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk
   return (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);
 }
 
+// Q8_1 of one 32-element block whose values sit one per lane in an aligned group of 32 lanes (all 32 active): every lane
+// stores its int8, the first lane of the group the (d, s) pair.  `blk` points at the 36-byte block, l = lane % 32.
+__device__ __forceinline__ void lane32_q8_1_store(float v, uint8_t* __restrict__ blk, int l) {
+  float amax = row16_max(fabsf(v));
+  amax = fmaxf(amax, __shfl_xor(amax, 16));
+  const double d = (double)amax / 127.0;
+  int q = q8_1_round(v, amax != 0.0f ? 127.0f / amax : 0.0f, d != 0.0 ? d : 1.0);
+  int sum = row16_sum_i32(q);
+  sum += __shfl_xor(sum, 16);
+  q = q < -128 ? -128 : (q > 127 ? 127 : q);
+  blk[l] = (uint8_t)(int8_t)q;
+  if (l == 0)
+    *(uint32_t*)(blk + 32) = (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);
+}
+
 // Block-wide sum in double for blockDim.x = 64 * NW; every thread gets the total.
 template <int NW>
 __device__ __forceinline__ double block_sum_f64(double v, double* lds) {

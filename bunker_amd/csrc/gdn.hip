@@ -36,6 +36,7 @@ struct GdnArgs {
   const float* S_in;
   float* S_out;
   uint16_t* out;            // bf16 [B, Hg*128]
+  uint8_t* out_q8;          // optional: the same outputs as Q8_1 blocks [B, Hg*128/32] for the matmul that follows
   int Hg;
   // conv mode (src/emitters.ts:48-72 folded in): q, k, v above point into the raw qkv projection and every
   // channel first goes through the 4-tap causal convolution + SiLU; its state rows are shifted in the same pass
@@ -213,7 +214,9 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   if (tid < GDN_D) {
     const float orstd = rsqrt_f64((red[0] + red[1]) / (double)GDN_D + 1e-6);
     const float zs = zin * sigmoid_f64(zin);
-    outp[tid] = f32_to_bf16(((o * orstd) * nw) * zs);
+    const uint16_t ob = f32_to_bf16(((o * orstd) * nw) * zs);
+    outp[tid] = ob;
+    if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (bh * (GDN_D / 32) + (tid >> 5)) * 36, tid & 31);
   }
 }
 
@@ -245,8 +248,9 @@ int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, co
 
 int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv_w, const void* z, const float* A_log,
                           const void* dt_bias, const float* a_p, const float* b_p, const float* norm_w, const float* S_in,
-                          void* out, void* conv_st_new, float* S_out, int Hg, int batch) {
+                          void* out, void* conv_st_new, float* S_out, void* out_q8, int Hg, int batch) {
   GdnArgs A{};
+  A.out_q8 = (uint8_t*)out_q8;
   const int KEYDIM = Hg * GDN_D;
   A.q = (const uint16_t*)qkv; A.k = A.q + KEYDIM; A.v = A.q + 2 * KEYDIM;
   A.qkv_bstride = 3 * (int64_t)KEYDIM;

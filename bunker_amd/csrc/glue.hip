@@ -138,6 +138,45 @@ int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t 
   return BK_OK;
 }
 
+// swiglu with both forms of the result: bf16 (optional) and the Q8_1 blocks the down projection consumes, so that no
+// separate quantizer pass reads the activation again.  A thread owns 8 consecutive elements, four lanes one Q8_1 block.
+__global__ __launch_bounds__(256) void swiglu_q8_1_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                          uint16_t* __restrict__ out, uint8_t* __restrict__ out_q8, int64_t n) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i >= n) return;                     // n is a multiple of 32: the four lanes of a block leave together
+  const float4 g0 = *(const float4*)(g + i), g1 = *(const float4*)(g + i + 4);
+  const float4 u0 = *(const float4*)(u + i), u1 = *(const float4*)(u + i + 4);
+  const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+  const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+  uint16_t ob[8];
+  float f[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) {
+    ob[k] = f32_to_bf16(__fmul_rn(__fmul_rn(gv[k], sigmoid_f64(gv[k])), uv[k]));
+    f[k] = bf16_to_f32(ob[k]);
+  }
+  if (out) {
+    uint4 o;
+    o.x = (uint32_t)ob[0] | ((uint32_t)ob[1] << 16); o.y = (uint32_t)ob[2] | ((uint32_t)ob[3] << 16);
+    o.z = (uint32_t)ob[4] | ((uint32_t)ob[5] << 16); o.w = (uint32_t)ob[6] | ((uint32_t)ob[7] << 16);
+    *(uint4*)(out + i) = o;
+  }
+  uint32_t pk[2];
+  const uint32_t ds = quad_q8_1(f, pk);
+  uint8_t* blk = out_q8 + (i / 32) * 36;
+  *(uint2*)(blk + (i & 31)) = make_uint2(pk[0], pk[1]);
+  if ((i & 31) == 0) *(uint32_t*)(blk + 32) = ds;
+}
+
+int launch_swiglu_q8_1(const float* g, const float* u, void* out, void* out_q8, int64_t n) {
+  BK_REQUIRE(g && u && out_q8, "swiglu_q8_1: null pointer");
+  BK_REQUIRE(n > 0 && n % 32 == 0, "swiglu_q8_1: n=%lld must be a positive multiple of 32", (long long)n);
+  hipLaunchKernelGGL(swiglu_q8_1_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, stream(), g, u, (uint16_t*)out,
+                     (uint8_t*)out_q8, n);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
 // ---------------------------------------------------------------- conv1d decode
 // src/emitters.ts:48-72: r = (w0*s0 + w1*s1) + (w2*s2 + w3*x); out = bf16(r * sigmoid(r));
 // new state rows = (s1, s2, x).  state [B, 3, C] bf16, weight [C, 4] bf16.  The new state may be

@@ -56,6 +56,7 @@ enum : int { EW_CAST_OP = 0, EW_ADD_OP = 1, EW_SWIGLU_OP = 2 };
 int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void* out, int H, int vocab, int batch);
 int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows);
 int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t n);
+int launch_swiglu_q8_1(const float* g, const float* u, void* out, void* out_q8, int64_t n);
 int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch);
 int launch_conv1d_prefill(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int T);
 int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD, int in_stride, int64_t in_bstride,
@@ -75,7 +76,7 @@ int launch_gdn_fused(const void* conv_out, const void* z, const float* A_log, co
                      const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, int Hg, int batch);
 int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv_w, const void* z, const float* A_log,
                           const void* dt_bias, const float* a_p, const float* b_p, const float* norm_w, const float* S_in,
-                          void* out, void* conv_st_new, float* S_out, int Hg, int batch);
+                          void* out, void* conv_st_new, float* S_out, void* out_q8, int Hg, int batch);
 int launch_gdn_core(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* S_in,
                     void* out, float* S_out, int Hg, int batch);
 
@@ -85,7 +86,7 @@ int attn_choose_splits(int batch, int NKV, int max_ctx);
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits);
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8 = nullptr);
 int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
                      void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size);

@@ -205,6 +205,9 @@ def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str
     return " ".join(parts)
 
 
+Q8OUT_MIN_BATCH = 8      # from this batch on producers also emit their output as Q8_1 (gemv_fused then runs its batched path)
+
+
 def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict) -> KernelPlan:
     """The fused op spec and slot list for a multi-node group (see fusedPartition)."""
     ops = tuple(n.op for n in grp)
@@ -216,6 +219,11 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         spec = f"gemv_fused K={K} pro=2 G=2 swiglu=1 N0={N} N1={N}" + bpart
         args = [norm.inputs[0].tensorName, norm.inputs[1].tensorName, gate.inputs[1].tensorName, up.inputs[1].tensorName,
                 sw.outputs[0].tensorName]
+        if batch >= Q8OUT_MIN_BATCH and N % 32 == 0:
+            # the batched path writes the activation a second time as Q8_1, and the down projection reads that
+            aux = sw.outputs[0].tensorName + ".q8_1"
+            q8_of[sw.outputs[0].tensorName] = aux
+            return KernelPlan(spec + " q8out=1", name, args + [aux], [1, 1, 1], grp, {aux: batch * (N // 32) * 36})
         return KernelPlan(spec, name, args, [1, 1, 1], grp)
     if ops[0] == "rmsnorm" and all(o == "gemm" for o in ops[1:]) and len(ops) > 1:
         norm, gemms = grp[0], grp[1:]
@@ -242,7 +250,14 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         spec = f"gdn_conv LVH={int(gd.params['LVH'])} LKD={int(gd.params['LKD'])} LVD={int(gd.params['LVD'])}" + bpart
         args = [cv.inputs[0].tensorName, cv.inputs[1].tensorName, cv.inputs[2].tensorName] + \
                [i.tensorName for i in gd.inputs[1:]] + [gd.outputs[0].tensorName, cv.outputs[1].tensorName, gd.outputs[1].tensorName]
-        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+        if batch < Q8OUT_MIN_BATCH:
+            return KernelPlan(spec, name, args, [1, 1, 1], grp)
+        # batched step: the threads that write the bf16 output also leave it as Q8_1 for out_proj (at batch 1 the
+        # projection's own prologue does it as fast, and the recurrence kernel stays shorter)
+        out, ZD = gd.outputs[0].tensorName, int(gd.params["ZD"])
+        aux = out + ".q8_1"
+        q8_of[out] = aux
+        return KernelPlan(spec + " q8out=1", name, args + [aux], [1, 1, 1], grp, {aux: batch * (ZD // 32) * 36})
     if ops == ("qnorm", "rope", "knorm", "ropek", "fa2_attn"):
         qn, rp, kn, rk, fa = grp
         P = fa.params
@@ -251,7 +266,12 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         args = [qn.inputs[0].tensorName, kn.inputs[0].tensorName, fa.inputs[2].tensorName, qn.inputs[1].tensorName,
                 kn.inputs[1].tensorName, rp.inputs[1].tensorName, rp.inputs[2].tensorName, rp.inputs[3].tensorName,
                 fa.inputs[4].tensorName, fa.inputs[5].tensorName, fa.outputs[0].tensorName]
-        return KernelPlan(spec, name, args, [1, 1, 1], grp)
+        if batch < Q8OUT_MIN_BATCH:
+            return KernelPlan(spec, name, args, [1, 1, 1], grp)
+        out, n_out = fa.outputs[0].tensorName, int(P["NH"]) * int(P["HD"])
+        aux = out + ".q8_1"
+        q8_of[out] = aux
+        return KernelPlan(spec + " q8out=1", name, args + [aux], [1, 1, 1], grp, {aux: batch * (n_out // 32) * 36})
     raise NotImplementedError(f"no fused kernel for the group {ops}")
 
 

@@ -107,6 +107,18 @@ def test_gemv_fused_swiglu(orc, dev, K, N, batch):
     for b in range(batch):
         ref = orc.swiglu(orc.gemv_q4k_q8_1(Wg, xq_rows[b], N, K), orc.gemv_q4k_q8_1(Wu, xq_rows[b], N, K))
         assert np.array_equal(got[b], ref), b
+    if batch >= 8 and N % 32 == 0:
+        # the batched path can leave the activation as Q8_1 too (what the down projection would quantize itself)
+        out2, q8 = dev.empty(batch * N * 2), dev.empty(batch * (N // 32) * 36)
+        launch(f"gemv_fused K={K} pro=2 G=2 swiglu=1 N0={N} N1={N} batch={batch} q8out=1",
+               [dev.up(x), dev.up(w), dev.up(Wg), dev.up(Wu), out2, q8])
+        assert np.array_equal(rt.from_device(out2, (batch, N), np.uint16), got)
+        gq = rt.from_device(q8, (batch, (N // 32) * 36), np.uint8)
+        for b in range(batch):
+            assert np.array_equal(gq[b], orc.pack_q8_1(f32(got[b]))), b
+    elif batch < 8:
+        with pytest.raises(rt.BunkerError, match="q8out"):
+            rt.compileAndLoad(f"gemv_fused K=2048 pro=2 G=2 swiglu=1 N0=64 N1=64 batch={batch} q8out=1")
 
 
 @pytest.mark.parametrize("Hg,B", [(16, 1), (3, 2)])
@@ -125,10 +137,14 @@ def test_gdn_conv_is_conv1d_then_delta_rule(orc, dev, Hg, B):
     norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
     S = (g.standard_normal((B, Hg, 128, 128)) * 0.02).astype(np.float32)
     dout, dS, dst = dev.empty(B * Hg * 128 * 2), dev.empty(S.nbytes), dev.up(st)
-    launch(f"gdn_conv LVH={Hg} LKD=128 LVD=128 batch={B}",
+    dq8 = dev.empty(B * Hg * 4 * 36)
+    launch(f"gdn_conv LVH={Hg} LKD=128 LVD=128 batch={B} q8out=1",
            [dev.up(qkv), dst, dev.up(cw), dev.up(z), dev.up(A_log), dev.up(dt_bias), dev.up(a_p), dev.up(b_p), dev.up(norm_w),
-            dev.up(S), dout, dst, dS])        # conv state updated in place
+            dev.up(S), dout, dst, dS, dq8])        # conv state updated in place; the output also as Q8_1
     out = rt.from_device(dout, (B, Hg * 128), np.uint16); Sn = rt.from_device(dS, S.shape, np.float32)
+    q8 = rt.from_device(dq8, (B, Hg * 4 * 36), np.uint8)
+    for b in range(B):
+        assert np.array_equal(q8[b], orc.pack_q8_1(f32(out[b]))), b
     stn = rt.from_device(dst, (B, 3, C), np.uint16)
     for b in range(B):
         conv, rs = orc.conv1d_decode(qkv[b], st[b], cw)
@@ -157,11 +173,15 @@ def test_fa2_fused_is_norm_rope_append_attend(orc, dev, batch):
     dout = dev.empty(batch * NH * HD * 2)
     spec = f"fa2_fused HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF}"
     common = [dev.up(qgate), dev.up(k), dev.up(v), dev.up(qw), dev.up(kw), dev.up(cos_t), dev.up(sin_t)]
+    dq8 = dev.empty(batch * NH * HD // 32 * 36)
     if batch == 1:
-        launch(spec, common + [pos[0], dkc, dvc, dout])
+        launch(spec + " q8out=1 splits=1", common + [pos[0], dkc, dvc, dout, dq8])        # one split: stand-alone quantizer
     else:
-        launch(spec + f" batch={batch} pos_dev=1", common + [dev.up(np.array(pos, np.int32)), dkc, dvc, dout])
+        launch(spec + f" batch={batch} pos_dev=1 q8out=1", common + [dev.up(np.array(pos, np.int32)), dkc, dvc, dout, dq8])
     out = rt.from_device(dout, (batch, NH, HD), np.uint16)
+    q8 = rt.from_device(dq8, (batch, NH * HD // 32 * 36), np.uint8)
+    for b in range(batch):
+        assert np.array_equal(q8[b], orc.pack_q8_1(f32(out[b].ravel()))), b             # Q8_1 of the bf16 output as written
     bt = np.arange(batch * ppseq, dtype=np.int32).reshape(batch, ppseq)
     qn = np.empty((batch, NH, HD), np.uint16)
     for b in range(batch):

@@ -126,6 +126,21 @@ def test_fused_partition_groups_and_specs():
     assert "gemv_fused K=2048 pro=2 G=2 swiglu=1 N0=6144 N1=6144" in specs
     assert "gemv_fused K=6144 pro=1 G=1 N0=2048 epi0=2" in specs
     assert "fa2_fused HD=256 NH=16 NKV=2 MAX_LEN=4352 ROT_HALF=32 pos_dev=1" in specs
+    # from batch 8 on gdn_conv, fa2_fused and the SwiGLU group leave their output as Q8_1 too, and the projection behind
+    # them reads that (pro=0) instead of quantizing
+    g32 = model.buildModelGraph(SYNTH, 32)
+    plans32 = runner.compilePartition(g32, runner.topoOrder(g32, runner.fusedPartition(g32)), 32, True)
+    sw = next(p for p in plans32 if "swiglu=1" in p.spec)
+    assert sw.spec == "gemv_fused K=2048 pro=2 G=2 swiglu=1 N0=6144 N1=6144 batch=32 q8out=1"
+    assert list(sw.aux.values()) == [32 * (6144 // 32) * 36]
+    down32 = next(p for p in plans32 if p.args[0] == sw.args[-1])
+    assert down32.spec == "gemv_fused K=6144 pro=0 G=1 N0=2048 epi0=2 batch=32"
+    gdn = next(p for p in plans32 if p.spec.startswith("gdn_conv"))
+    assert gdn.spec.endswith("q8out=1") and list(gdn.aux.values()) == [32 * (2048 // 32) * 36]
+    assert next(p for p in plans32 if p.args[0] == gdn.args[-1]).spec == "gemv_fused K=2048 pro=0 G=1 N0=2048 epi0=2 batch=32"
+    fa = next(p for p in plans32 if p.spec.startswith("fa2_fused"))
+    assert fa.spec.endswith("q8out=1")
+    assert next(p for p in plans32 if p.args[0] == fa.args[-1]).spec == "gemv_fused K=4096 pro=0 G=1 N0=2048 epi0=2 batch=32"
     # lm_head reads the Q8_1 row the stand-alone final norm leaves in an auxiliary buffer
     norm = next(p for p in plans if p.spec.startswith("rmsnorm_q8_1"))
     head = next(p for p in plans if "N0=151936" in p.spec)
