@@ -156,3 +156,18 @@ def test_synthetic_qwen35_decode_step_bs32(orc):
     S = synth_model.synth_state(D, batch=32, seed=8, share_kv_across_batch=True)
     starts = [(9419 + 4099 * i) % D.VOCAB for i in range(32)]
     _strict_decode(D, W, S, starts, 4096, 2, use_graph=True, check=[0, 13, 31], fused=True)
+
+
+@pytest.mark.parametrize("batch", [1, 9])
+def test_reference_dims_decode(orc, batch):
+    """The dimensions of src/model.ts:14-18 (hidden 1024, FFN 3584, 8 query heads) with 4 layers and a short vocabulary:
+    K = 1024 and 3584 are outside the fused GEMV's fast path, so the same op specs run their composed form
+    (RMSNorm -> Q8_1 kernel, generic-K GEMV at batch 1, MFMA matmul at batch 9) and must give the same bits."""
+    from dataclasses import replace
+    D = replace(model.REFERENCE, NL=4, VOCAB=4096, MAX_LEN=64)
+    print(f"reference dims, batch {batch}", flush=True)
+    W = synth_model.synth_weights(D, seed=41)
+    S = synth_model.synth_state(D, batch=batch, seed=42)
+    starts = [(113 * i + 9) % D.VOCAB for i in range(batch)]
+    toks, vals = _strict_decode(D, W, S, starts, 30, 3, use_graph=True, fused=True, check=[0, batch - 1] if batch > 1 else None)
+    assert toks.shape == (3, batch)
