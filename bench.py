@@ -131,6 +131,25 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
                       "first_generated_token": tok}
     for env in envs:
         env.close()
+    # the reference model's own dimensions (src/model.ts:14-18), random Q4_K weights, KV at 4096: batch 1 only
+    from dataclasses import replace
+    DR = replace(model.REFERENCE, MAX_LEN=4352)
+    WR = synth_model.synth_weights(DR, seed=2027)
+    SR = synth_model.device_state(synth_model.synth_state(DR, batch=1, seed=9))
+    gR = model.buildModelGraph(DR, 1)
+    envR = runner.DecodeEnv(gR, WR, SR, inplace_state=True)
+    loopR = runner.DeviceLoop(gR, envR, 1, [9419], 4096, max_steps=8 + steps_bs1, use_graph=use_graph,
+                              partition=runner.fusedPartition(gR) if fused else None)
+    loopR.step(8)
+    rt.cuSync()
+    e0, e1 = rt.Event().record(), rt.Event()
+    loopR.step(steps_bs1)
+    e1.record()
+    rt.cuSync()
+    ms = e0.elapsed_ms(e1) / steps_bs1
+    out["reference_dims"] = {"dims": "hidden 1024, FFN 3584, vocab 248320, 18 GDN + 6 attention layers (src/model.ts:14-18)",
+                             "bs1": {"tok_per_s": round(1e3 / ms, 1), "ms_per_step": round(ms, 4), "steps": steps_bs1}}
+    envR.close()
     return out
 
 

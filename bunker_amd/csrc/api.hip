@@ -93,7 +93,8 @@ static int run_gemm(Kernel& k, const uint64_t* s) {
 //         G matrices with N<i>, epi<i> (0: f32, 1: bf16, 2: bf16(bf16(y) + residual)), swiglu=0|1 (G=2: gate, up), batch=1
 // slots:  x, [norm_w if pro=2], then per matrix: W, [residual if epi=2], out      (swiglu: x, [norm_w], Wg, Wu, out
 //         [, out as Q8_1 blocks when q8out=1: batch >= 8 only])
-// Shapes outside the fused kernel (K not 2048/4096/6144, batch >= 8) run as rmsnorm/quantize, matmuls, swiglu.
+// Shapes outside the fused kernel (K other than 1024, 2048, 3584, 4096, 6144, or batch >= 8) run as rmsnorm/quantize,
+// matmuls, swiglu.
 static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   const int K = (int)k.get("K", 0), pro = (int)k.get("pro", 0), G = (int)k.get("G", 1), batch = (int)k.get("batch", 1);
   const bool swiglu = k.get("swiglu", 0) != 0;

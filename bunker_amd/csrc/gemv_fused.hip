@@ -58,26 +58,30 @@ __device__ __forceinline__ StepSel select_step(const FusedArgs& A, int s) {
   return r;
 }
 
-// ---- prologue: activation row -> Q8_1 in LDS (36-byte blocks).  K = 2048 * NR: NR passes of 256 threads x 8 elements.
+// ---- prologue: activation row -> Q8_1 in LDS (36-byte blocks).  K = 256 * KB elements in NR = ceil(KB / 8) passes of
+// 256 threads x 8 elements; in the last pass of a K that is not a multiple of 2048 the threads past the row take no part
+// (their loads are clamped, their values zero).
 // Everything the prologue reads from memory (the row and, for RMSNorm, the norm weight) is requested up front.
 // Loads return to a wave in the order they were issued, so these go out BEFORE the weight rows: the prologue then
 // waits for a few small, cache-resident loads only and runs while the weight rows are still on their way.
-template <int NR>
+template <int KB>
 struct ActRegs {
+  static constexpr int NR = (KB + 7) / 8, K = KB * 256;
   uint4 xv[NR], wv[NR];
 };
-template <int PRO, int NR>
-__device__ __forceinline__ void act_load(ActRegs<NR>& r, const uint16_t* __restrict__ xr, const uint16_t* __restrict__ w) {
+template <int PRO, int KB>
+__device__ __forceinline__ void act_load(ActRegs<KB>& r, const uint16_t* __restrict__ xr, const uint16_t* __restrict__ w) {
+  constexpr int K = ActRegs<KB>::K;
 #pragma unroll
-  for (int p = 0; p < NR; p++) {
-    const int i = threadIdx.x * 8 + p * 2048;
+  for (int p = 0; p < ActRegs<KB>::NR; p++) {
+    const int i = min((int)threadIdx.x * 8 + p * 2048, K - 8);
     r.xv[p] = *(const uint4*)(xr + i);
     if (PRO == PRO_RMSNORM) r.wv[p] = *(const uint4*)(w + i);
   }
 }
-template <int PRO, int NR>
-__device__ __forceinline__ void stage_activation(const ActRegs<NR>& regs, uint8_t* lds_xq, double* lds_red) {
-  constexpr int K = NR * 2048;
+template <int PRO, int KB>
+__device__ __forceinline__ void stage_activation(const ActRegs<KB>& regs, uint8_t* lds_xq, double* lds_red) {
+  constexpr int NR = ActRegs<KB>::NR, K = ActRegs<KB>::K;
   const uint4 (&xv)[NR] = regs.xv;
   const uint4 (&wv)[NR] = regs.wv;
   float rstd = 0.0f;
@@ -85,12 +89,15 @@ __device__ __forceinline__ void stage_activation(const ActRegs<NR>& regs, uint8_
     double ss = 0.0;
 #pragma unroll
     for (int p = 0; p < NR; p++) {
+      const bool valid = (p + 1) * 2048 <= K || (int)threadIdx.x * 8 + p * 2048 < K;
       const uint32_t u[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w};
+      double sp = 0.0;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
-        ss += (double)(a * a) + (double)(b * b);
+        sp += (double)(a * a) + (double)(b * b);
       }
+      ss += valid ? sp : 0.0;
     }
     ss = block_sum_f64<4>(ss, lds_red);
     rstd = rsqrt_f64(ss / (double)K + 1e-6);
@@ -98,6 +105,7 @@ __device__ __forceinline__ void stage_activation(const ActRegs<NR>& regs, uint8_
 #pragma unroll
   for (int p = 0; p < NR; p++) {
     const int i = threadIdx.x * 8 + p * 2048;
+    const bool valid = (p + 1) * 2048 <= K || i < K;        // whole quads (K is a multiple of 32)
     const uint32_t u[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w};
     float f[8];
     if (PRO == PRO_RMSNORM) {
@@ -118,25 +126,35 @@ __device__ __forceinline__ void stage_activation(const ActRegs<NR>& regs, uint8_
     }
     uint32_t pk[2];
     const uint32_t ds = quad_q8_1(f, pk);
-    uint8_t* ob = lds_xq + (i / 32) * 36;
-    uint32_t* oq = (uint32_t*)(ob + (i & 31));
-    oq[0] = pk[0]; oq[1] = pk[1];
-    if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+    if (valid) {
+      uint8_t* ob = lds_xq + (i / 32) * 36;
+      uint32_t* oq = (uint32_t*)(ob + (i & 31));
+      oq[0] = pk[0]; oq[1] = pk[1];
+      if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+    }
   }
   __syncthreads();
 }
 
+// Rows of KB super-blocks: 9 * KB pieces of 16 bytes each, RPI rows per wave step.
+template <int KB, int RPI>
+struct FusedStage {
+  static constexpr int PIECES = RPI * KB * 9;
+  static constexpr int LOADS = (PIECES + 63) / 64;
+  uint4 v[LOADS];
+};
+
 // ---- weight rows of one step: coalesced 16-byte pieces; with SWIGLU the second half of the tile
 // comes from the up matrix (same rows)
-template <int NR, int RPI, bool SWIGLU>
-__device__ __forceinline__ void fused_stage_load(StageRegs<NR, RPI>& g, const uint8_t* __restrict__ W0,
+template <int KB, int RPI, bool SWIGLU>
+__device__ __forceinline__ void fused_stage_load(FusedStage<KB, RPI>& g, const uint8_t* __restrict__ W0,
                                                  const uint8_t* __restrict__ W1, int row0, int N, int lane) {
-  constexpr int PIECES = StageRegs<NR, RPI>::PIECES;
-  constexpr int64_t row_bytes = (int64_t)NR * 8 * 144;
+  constexpr int PIECES = FusedStage<KB, RPI>::PIECES;
+  constexpr int64_t row_bytes = (int64_t)KB * 144;
   const int64_t last = (int64_t)N * row_bytes - 16;
   const int64_t base = (int64_t)row0 * row_bytes;
 #pragma unroll
-  for (int u = 0; u < StageRegs<NR, RPI>::LOADS; u++) {
+  for (int u = 0; u < FusedStage<KB, RPI>::LOADS; u++) {
     // every lane loads in every round (lanes past the tile re-request its last piece): the number of loads in
     // flight is then known at compile time and waits can be counted instead of draining the queue
     const int piece = min(lane + 64 * u, PIECES - 1);
@@ -146,11 +164,23 @@ __device__ __forceinline__ void fused_stage_load(StageRegs<NR, RPI>& g, const ui
     g.v[u] = load_w16(W + (off < last ? off : last));       // past the matrix: re-read its last piece
   }
 }
+template <int KB, int RPI>
+__device__ __forceinline__ void fused_stage_park(const FusedStage<KB, RPI>& g, uint4* __restrict__ tile, int lane) {
+#pragma unroll
+  for (int u = 0; u < FusedStage<KB, RPI>::LOADS; u++) {
+    const int piece = lane + 64 * u;
+    if (piece < FusedStage<KB, RPI>::PIECES) tile[piece] = g.v[u];
+  }
+}
 
-template <int NR, int RPI, int PRO, bool SWIGLU>
+// KB = super-blocks per row (K = 256 * KB).  Lane (b, c) folds super-block 8r + b in pass r; when KB is not a multiple of 8
+// the lanes past the row in the last pass read a clamped block and an all-zero activation slice, which adds exact zeros.
+template <int KB, int RPI, int PRO, bool SWIGLU>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A) {
-  constexpr int PIECES = RPI * NR * 72;
-  constexpr int K = NR * 2048;
+  constexpr int NR = (KB + 7) / 8;
+  constexpr int RP = KB * 9;                 // 16-byte pieces per row
+  constexpr int PIECES = RPI * RP;
+  constexpr int K = KB * 256;
   constexpr int ROWS_PER_STEP = SWIGLU ? RPI / 2 : RPI;
   __shared__ uint4 tiles[GEMV_WAVES][PIECES];
   __shared__ __align__(16) uint8_t lds_xq[PRO == PRO_Q8 ? 16 : (K / 32) * 36];
@@ -166,34 +196,34 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
   const int total = A.step_first[4];
   uint4* tile = tiles[wv];
 
-  ActRegs<NR> act;
-  if (PRO != PRO_Q8) act_load<PRO, NR>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
+  ActRegs<KB> act;
+  if (PRO != PRO_Q8) act_load<PRO, KB>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
 
   int s = blockIdx.x * GEMV_WAVES + wv;
   StepSel cur = select_step<ROWS_PER_STEP>(A, s < total ? s : 0);
-  StageRegs<NR, RPI> g;
+  FusedStage<KB, RPI> g;
   // unconditional (a wave without a step of its own requests step 0): with a branch around these loads the
   // prologue's first wait could not be counted and would drain the weight rows as well
-  fused_stage_load<NR, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
+  fused_stage_load<KB, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
 
   XQ x[NR];
   if (PRO == PRO_Q8) {
     const uint8_t* xq = (const uint8_t*)A.x + (int64_t)bidx * (K / 32) * 36;
 #pragma unroll
-    for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, true);
+    for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, (r + 1) * 8 <= KB || r * 8 + b < KB);
   } else {
-    stage_activation<PRO, NR>(act, lds_xq, lds_red);
+    stage_activation<PRO, KB>(act, lds_xq, lds_red);
 #pragma unroll
-    for (int r = 0; r < NR; r++) load_xq(x[r], lds_xq, r * 8 + b, c, true);
+    for (int r = 0; r < NR; r++) load_xq(x[r], lds_xq, r * 8 + b, c, (r + 1) * 8 <= KB || r * 8 + b < KB);
   }
 
   while (s < total) {
-    stage_park<NR, RPI>(g, tile, lane);
+    fused_stage_park<KB, RPI>(g, tile, lane);
     const int sn = s + nwaves;
     StepSel nxt = cur;
     if (sn < total) {
       nxt = select_step<ROWS_PER_STEP>(A, sn);
-      fused_stage_load<NR, RPI, SWIGLU>(g, nxt.W, A.g[1].W, nxt.row0, nxt.N, lane);
+      fused_stage_load<KB, RPI, SWIGLU>(g, nxt.W, A.g[1].W, nxt.row0, nxt.N, lane);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -203,7 +233,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
     for (int i = 0; i < RPI; i++) {
 #pragma unroll
       for (int r = 0; r < NR; r++) {
-        const int blk = (i * NR + r) * 72 + b * 9;
+        const int blk = i * RP + min(r * 8 + b, KB - 1) * 9;
         t.hdr[i][r] = tile[blk];
         t.q[i][r] = tile[blk + 1 + c];
       }
@@ -236,18 +266,18 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
   }
 }
 
+// Row lengths with a compiled kernel: 1024, 2048, 3584, 4096, 6144 (4, 8, 14, 16, 24 super-blocks); SwiGLU pairs for 1024 and 2048.
 bool gemv_fused_fast_path(int K, int batch, bool swiglu) {
-  if (K <= 0 || K % 2048 != 0 || K > 6144) return false;
-  if (swiglu && K != 2048) return false;
-  return batch >= 1 && batch < 8;
+  const bool k_ok = swiglu ? (K == 1024 || K == 2048) : (K == 1024 || K == 2048 || K == 3584 || K == 4096 || K == 6144);
+  return k_ok && batch >= 1 && batch < 8;
 }
 
-template <int NR, int RPI, bool SWIGLU>
+template <int KB, int RPI, bool SWIGLU>
 static void launch_fused_pro(int pro, dim3 grid, const FusedArgs& A) {
   const dim3 block(GEMV_WAVES * 64);
-  if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_Q8, SWIGLU>), grid, block, 0, stream(), A);
-  else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_BF16, SWIGLU>), grid, block, 0, stream(), A);
-  else hipLaunchKernelGGL((gemv_fused_kernel<NR, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
+  if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, SWIGLU>), grid, block, 0, stream(), A);
+  else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, SWIGLU>), grid, block, 0, stream(), A);
+  else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
 }
 
 // Fast path only (gemv_fused_fast_path says whether it applies); the caller composes the same
@@ -259,7 +289,7 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
   BK_REQUIRE(gemv_fused_fast_path(K, batch, swiglu), "gemv_fused: K=%d batch=%d is outside the fused kernel's shapes", K, batch);
   BK_REQUIRE(ngroups >= 1 && ngroups <= 4 && (!swiglu || ngroups == 2), "gemv_fused: bad number of matrices %d", ngroups);
   BK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemv_fused: activation and norm weight must be 16-byte aligned");
-  const int NR = K / 2048, RPI = NR == 1 ? 4 : 2;
+  const int KB = K / 256, RPI = KB <= 8 ? 4 : 2;
   const int rows_per_step = swiglu ? RPI / 2 : RPI;
   FusedArgs A{};
   A.ngroups = ngroups; A.x = x; A.norm_w = (const uint16_t*)norm_w;
@@ -288,10 +318,13 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
   const int cap = num_cus() * g_tune_cap;
   if (wgs > cap) wgs = cap;
   const dim3 grid(wgs, batch);
-  if (swiglu) launch_fused_pro<1, 4, true>(pro, grid, A);
-  else if (NR == 1) launch_fused_pro<1, 4, false>(pro, grid, A);
-  else if (NR == 2) launch_fused_pro<2, 2, false>(pro, grid, A);
-  else launch_fused_pro<3, 2, false>(pro, grid, A);
+  if (swiglu && KB == 4) launch_fused_pro<4, 4, true>(pro, grid, A);
+  else if (swiglu) launch_fused_pro<8, 4, true>(pro, grid, A);
+  else if (KB == 4) launch_fused_pro<4, 4, false>(pro, grid, A);
+  else if (KB == 8) launch_fused_pro<8, 4, false>(pro, grid, A);
+  else if (KB == 14) launch_fused_pro<14, 2, false>(pro, grid, A);
+  else if (KB == 16) launch_fused_pro<16, 2, false>(pro, grid, A);
+  else launch_fused_pro<24, 2, false>(pro, grid, A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -53,9 +53,11 @@ def ref_activation(orc, pro, x_bits, w_bits):
     return rows
 
 
-# K = 2048 / 4096 / 6144 run the fused kernel at batch < 8; K = 512 and batch 9 run the composed path
+# K = 1024 / 2048 / 3584 / 4096 / 6144 run the fused kernel at batch < 8 (1024 and 3584 with lanes past the row in the last
+# pass); K = 512 and batch 9 run the composed path
 @pytest.mark.parametrize("K,batch,pro", [(2048, 1, 2), (2048, 3, 2), (2048, 1, 1), (2048, 2, 0), (4096, 1, 1), (6144, 2, 1),
-                                          (6144, 1, 2), (512, 2, 2), (2048, 9, 2)])
+                                          (6144, 1, 2), (512, 2, 2), (2048, 9, 2), (1024, 1, 2), (1024, 2, 0), (1024, 3, 1),
+                                          (3584, 1, 1), (3584, 3, 2), (3584, 2, 0)])
 def test_gemv_fused_groups(orc, dev, K, batch, pro):
     print(f"gemv_fused K={K} batch={batch} pro={pro}", flush=True)
     g = synth.rng(900 + K + 10 * batch + pro)
@@ -93,7 +95,7 @@ def test_gemv_fused_groups(orc, dev, K, batch, pro):
                 assert np.array_equal(got, ref), (i, b)
 
 
-@pytest.mark.parametrize("K,N,batch", [(2048, 6144, 1), (2048, 204, 3), (512, 64, 2), (2048, 128, 8)])
+@pytest.mark.parametrize("K,N,batch", [(2048, 6144, 1), (2048, 204, 3), (512, 64, 2), (2048, 128, 8), (1024, 3584, 1), (1024, 100, 2)])
 def test_gemv_fused_swiglu(orc, dev, K, N, batch):
     print(f"gemv_fused swiglu K={K} N={N} batch={batch}", flush=True)
     g = synth.rng(950 + N + batch)
