@@ -1,0 +1,392 @@
+// Byte-level BPE tokenizer behind the C ABI the reference binds (shim/gigatoken_wrapper/src/lib.rs:19-93, used by
+// prototypes/decode.ts:78-86): gt_init(path to a Hugging Face tokenizer.json) / gt_encode / gt_free.  The reference's
+// wrapper is Rust over the gigatoken crate (a path dependency outside its tree, Cargo.toml:11); this is a C++ restatement
+// of the published algorithm those files implement:
+//   1. added tokens ("added_tokens": content -> id) are cut out of the text first, leftmost-longest;
+//   2. the rest is split by the pre-tokenizer's regular expression (the Qwen / cl100k family, matched by a hand-written
+//      scanner over code points with the Unicode general categories of unicode_tables.h);
+//   3. every piece goes through the GPT-2 byte -> printable-character map and is merged pair by pair in rank order
+//      ("merges"), lowest rank first, leftmost on ties; "ignore_merges" emits a piece that is a vocabulary entry as is.
+// Not done: Unicode normalisation (a "normalizer" of type NFC in the file is accepted; the text is taken as already
+// normalised), lstrip / rstrip / single_word flags of added tokens, case folding beyond ASCII in the contraction branch.
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "unicode_tables.h"
+
+namespace {
+
+// ------------------------------------------------------------------ minimal JSON reader (objects, arrays, strings, scalars)
+struct JValue {
+  enum Kind { NUL, BOOL, NUM, STR, ARR, OBJ } kind = NUL;
+  bool b = false;
+  double num = 0;
+  std::string str;
+  std::vector<JValue> arr;
+  std::vector<std::pair<std::string, JValue>> obj;
+  const JValue* get(const char* key) const {
+    for (const auto& kv : obj)
+      if (kv.first == key) return &kv.second;
+    return nullptr;
+  }
+};
+
+struct JParser {
+  const char* p;
+  const char* end;
+  bool ok = true;
+  void ws() { while (p < end && (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r')) p++; }
+  static void put_utf8(std::string& s, uint32_t cp) {
+    if (cp < 0x80) s += (char)cp;
+    else if (cp < 0x800) { s += (char)(0xC0 | (cp >> 6)); s += (char)(0x80 | (cp & 0x3F)); }
+    else if (cp < 0x10000) { s += (char)(0xE0 | (cp >> 12)); s += (char)(0x80 | ((cp >> 6) & 0x3F)); s += (char)(0x80 | (cp & 0x3F)); }
+    else { s += (char)(0xF0 | (cp >> 18)); s += (char)(0x80 | ((cp >> 12) & 0x3F)); s += (char)(0x80 | ((cp >> 6) & 0x3F)); s += (char)(0x80 | (cp & 0x3F)); }
+  }
+  uint32_t hex4() {
+    uint32_t v = 0;
+    for (int i = 0; i < 4 && p < end; i++, p++) {
+      const char c = *p;
+      v = v * 16 + (c >= '0' && c <= '9' ? c - '0' : c >= 'a' && c <= 'f' ? c - 'a' + 10 : c >= 'A' && c <= 'F' ? c - 'A' + 10 : (ok = false, 0));
+    }
+    return v;
+  }
+  std::string string() {
+    std::string s;
+    if (p >= end || *p != '"') { ok = false; return s; }
+    p++;
+    while (p < end && *p != '"') {
+      if (*p == '\\') {
+        p++;
+        if (p >= end) { ok = false; break; }
+        const char c = *p++;
+        switch (c) {
+          case 'n': s += '\n'; break; case 't': s += '\t'; break; case 'r': s += '\r'; break;
+          case 'b': s += '\b'; break; case 'f': s += '\f'; break;
+          case 'u': {
+            uint32_t cp = hex4();
+            if (cp >= 0xD800 && cp < 0xDC00 && p + 1 < end && p[0] == '\\' && p[1] == 'u') {   // surrogate pair
+              p += 2;
+              const uint32_t lo = hex4();
+              cp = 0x10000 + ((cp - 0xD800) << 10) + (lo - 0xDC00);
+            }
+            put_utf8(s, cp);
+            break;
+          }
+          default: s += c;      // \" \\ \/
+        }
+      } else {
+        s += *p++;
+      }
+    }
+    if (p >= end) ok = false; else p++;
+    return s;
+  }
+  JValue value() {
+    JValue v;
+    ws();
+    if (p >= end) { ok = false; return v; }
+    if (*p == '{') {
+      v.kind = JValue::OBJ; p++; ws();
+      if (p < end && *p == '}') { p++; return v; }
+      while (ok) {
+        ws();
+        std::string k = string();
+        ws();
+        if (p >= end || *p != ':') { ok = false; break; }
+        p++;
+        v.obj.emplace_back(std::move(k), value());
+        ws();
+        if (p < end && *p == ',') { p++; continue; }
+        if (p < end && *p == '}') { p++; break; }
+        ok = false;
+      }
+    } else if (*p == '[') {
+      v.kind = JValue::ARR; p++; ws();
+      if (p < end && *p == ']') { p++; return v; }
+      while (ok) {
+        v.arr.push_back(value());
+        ws();
+        if (p < end && *p == ',') { p++; continue; }
+        if (p < end && *p == ']') { p++; break; }
+        ok = false;
+      }
+    } else if (*p == '"') {
+      v.kind = JValue::STR; v.str = string();
+    } else if (!strncmp(p, "true", 4)) { v.kind = JValue::BOOL; v.b = true; p += 4; }
+    else if (!strncmp(p, "false", 5)) { v.kind = JValue::BOOL; v.b = false; p += 5; }
+    else if (!strncmp(p, "null", 4)) { v.kind = JValue::NUL; p += 4; }
+    else {
+      char* e = nullptr;
+      v.kind = JValue::NUM; v.num = strtod(p, &e);
+      if (e == p) ok = false;
+      p = e;
+    }
+    return v;
+  }
+};
+
+// ------------------------------------------------------------------ code points and classes
+bool in_ranges(const uint32_t (*t)[2], int n, uint32_t cp) {
+  int lo = 0, hi = n - 1;
+  while (lo <= hi) {
+    const int mid = (lo + hi) / 2;
+    if (cp < t[mid][0]) hi = mid - 1;
+    else if (cp > t[mid][1]) lo = mid + 1;
+    else return true;
+  }
+  return false;
+}
+bool is_letter(uint32_t cp) { return cp < 0x80 ? ((cp | 0x20) >= 'a' && (cp | 0x20) <= 'z') : in_ranges(UNI_LETTER, UNI_LETTER_count, cp); }
+bool is_number(uint32_t cp) { return cp < 0x80 ? (cp >= '0' && cp <= '9') : in_ranges(UNI_NUMBER, UNI_NUMBER_count, cp); }
+bool is_space(uint32_t cp) {       // the White_Space property (what \s means in the file's regular expression)
+  return (cp >= 0x09 && cp <= 0x0D) || cp == 0x20 || cp == 0x85 || cp == 0xA0 || cp == 0x1680 || (cp >= 0x2000 && cp <= 0x200A) ||
+         cp == 0x2028 || cp == 0x2029 || cp == 0x202F || cp == 0x205F || cp == 0x3000;
+}
+bool is_newline(uint32_t cp) { return cp == '\r' || cp == '\n'; }
+
+struct Cp { uint32_t cp; uint32_t off; };     // code point and its byte offset
+
+// UTF-8 -> code points; a malformed byte becomes one code point 0xFFFD that still covers that byte
+void decode_utf8(const uint8_t* s, size_t n, size_t base, std::vector<Cp>& out) {
+  size_t i = 0;
+  while (i < n) {
+    const uint8_t c = s[i];
+    uint32_t cp = 0xFFFD; size_t len = 1;
+    if (c < 0x80) cp = c;
+    else if ((c & 0xE0) == 0xC0 && i + 1 < n && (s[i + 1] & 0xC0) == 0x80) { cp = ((c & 0x1F) << 6) | (s[i + 1] & 0x3F); len = 2; }
+    else if ((c & 0xF0) == 0xE0 && i + 2 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80) {
+      cp = ((c & 0x0F) << 12) | ((s[i + 1] & 0x3F) << 6) | (s[i + 2] & 0x3F); len = 3;
+    } else if ((c & 0xF8) == 0xF0 && i + 3 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80 && (s[i + 3] & 0xC0) == 0x80) {
+      cp = ((c & 0x07) << 18) | ((s[i + 1] & 0x3F) << 12) | ((s[i + 2] & 0x3F) << 6) | (s[i + 3] & 0x3F); len = 4;
+    }
+    out.push_back({cp, (uint32_t)(base + i)});
+    i += len;
+  }
+}
+
+// ------------------------------------------------------------------ the pre-tokenizer's regular expression, by hand
+//   (?i:'s|'t|'re|'ve|'m|'ll|'d) | [^\r\n\p{L}\p{N}]?\p{L}+ | \p{N}{1,D} | ?[^\s\p{L}\p{N}]+[\r\n]* | \s*[\r\n]+ | \s+(?!\S) | \s+
+// Alternatives are tried in this order at every position and the first that matches wins; D = 1 (Qwen) or 3 (cl100k).
+struct Scanner {
+  int max_digits = 1;
+  // returns the number of code points of the piece that starts at c[i]
+  size_t next(const std::vector<Cp>& c, size_t i) const {
+    const size_t n = c.size();
+    auto at = [&](size_t k) { return k < n ? c[k].cp : 0u; };
+    auto lower = [](uint32_t x) { return x >= 'A' && x <= 'Z' ? x + 32 : x; };
+    if (at(i) == '\'' && i + 1 < n) {
+      const uint32_t a = lower(at(i + 1)), b = i + 2 < n ? lower(at(i + 2)) : 0;
+      if (a == 's' || a == 't') return 2;
+      if ((a == 'r' && b == 'e') || (a == 'v' && b == 'e')) return 3;
+      if (a == 'm') return 2;
+      if (a == 'l' && b == 'l') return 3;
+      if (a == 'd') return 2;
+    }
+    {   // [^\r\n\p{L}\p{N}]?\p{L}+
+      size_t k = i;
+      const uint32_t x = at(k);
+      if (!is_newline(x) && !is_letter(x) && !is_number(x) && k + 1 < n && is_letter(at(k + 1))) k++;
+      if (k < n && is_letter(at(k))) {
+        while (k < n && is_letter(at(k))) k++;
+        return k - i;
+      }
+    }
+    if (is_number(at(i))) {
+      size_t k = i;
+      while (k < n && k - i < (size_t)max_digits && is_number(at(k))) k++;
+      return k - i;
+    }
+    {   //  ?[^\s\p{L}\p{N}]+[\r\n]*
+      size_t k = i;
+      if (at(k) == ' ' && k + 1 < n) k++;
+      auto other = [&](uint32_t x) { return !is_space(x) && !is_letter(x) && !is_number(x); };
+      if (k < n && other(at(k))) {
+        while (k < n && other(at(k))) k++;
+        while (k < n && is_newline(at(k))) k++;
+        return k - i;
+      }
+    }
+    if (is_space(at(i))) {
+      size_t e = i;
+      while (e < n && is_space(at(e))) e++;
+      // \s*[\r\n]+ : up to and including the last line break of the run
+      for (size_t k = e; k > i; k--)
+        if (is_newline(at(k - 1))) return k - i;
+      // \s+(?!\S) : the whole run at the end of the text, else all but its last character
+      if (e == n) return e - i;
+      if (e - i > 1) return e - i - 1;
+      return 1;                                             // \s+
+    }
+    return 1;     // not reachable for well-formed input: every code point is a letter, number, space or "other"
+  }
+};
+
+// ------------------------------------------------------------------ the tokenizer
+struct PairHash {
+  size_t operator()(uint64_t k) const { return (size_t)(k * 0x9E3779B97F4A7C15ull >> 17); }
+};
+
+struct Tokenizer {
+  std::unordered_map<std::string, uint32_t> vocab;
+  std::unordered_map<uint64_t, std::pair<uint32_t, uint32_t>, PairHash> merges;     // (left id, right id) -> (rank, merged id)
+  std::vector<std::pair<std::string, uint32_t>> added;                              // content, id
+  uint32_t byte_id[256];          // id of the one-character token of every byte
+  std::string byte_char[256];     // the printable character (UTF-8) a byte maps to
+  bool ignore_merges = false;
+  Scanner scan;
+  std::string error;
+
+  bool load(const char* path) {
+    FILE* f = fopen(path, "rb");
+    if (!f) { error = std::string("cannot open ") + path; return false; }
+    std::string text;
+    char buf[1 << 16];
+    size_t got;
+    while ((got = fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, got);
+    fclose(f);
+    JParser jp{text.data(), text.data() + text.size()};
+    const JValue root = jp.value();
+    if (!jp.ok || root.kind != JValue::OBJ) { error = "tokenizer.json: not valid JSON"; return false; }
+    const JValue* model = root.get("model");
+    if (!model || !model->get("vocab") || !model->get("merges")) { error = "tokenizer.json: no model.vocab / model.merges"; return false; }
+    if (const JValue* t = model->get("type")) if (t->kind == JValue::STR && t->str != "BPE") { error = "tokenizer.json: model type is not BPE"; return false; }
+    if (const JValue* im = model->get("ignore_merges")) ignore_merges = im->kind == JValue::BOOL && im->b;
+    for (const auto& kv : model->get("vocab")->obj) vocab.emplace(kv.first, (uint32_t)kv.second.num);
+    // GPT-2 byte map: printable bytes map to themselves, the others to U+0100 onwards in byte order
+    int extra = 0;
+    for (int b = 0; b < 256; b++) {
+      const bool printable = (b >= 0x21 && b <= 0x7E) || (b >= 0xA1 && b <= 0xAC) || (b >= 0xAE && b <= 0xFF);
+      const uint32_t cp = printable ? (uint32_t)b : 0x100u + extra++;
+      JParser::put_utf8(byte_char[b], cp);
+      auto it = vocab.find(byte_char[b]);
+      if (it == vocab.end()) { error = "tokenizer.json: the vocabulary lacks a byte-level base token"; return false; }
+      byte_id[b] = it->second;
+    }
+    uint32_t rank = 0;
+    for (const JValue& m : model->get("merges")->arr) {
+      std::string a, b;
+      if (m.kind == JValue::ARR && m.arr.size() == 2) { a = m.arr[0].str; b = m.arr[1].str; }
+      else if (m.kind == JValue::STR) {
+        const size_t sp = m.str.find(' ');
+        if (sp == std::string::npos) { error = "tokenizer.json: malformed merge"; return false; }
+        a = m.str.substr(0, sp); b = m.str.substr(sp + 1);
+      } else { error = "tokenizer.json: malformed merge"; return false; }
+      auto ia = vocab.find(a), ib = vocab.find(b), iab = vocab.find(a + b);
+      if (ia == vocab.end() || ib == vocab.end() || iab == vocab.end()) { error = "tokenizer.json: merge of unknown tokens"; return false; }
+      merges.emplace(((uint64_t)ia->second << 32) | ib->second, std::make_pair(rank, iab->second));
+      rank++;
+    }
+    if (const JValue* at = root.get("added_tokens"))
+      for (const JValue& t : at->arr) {
+        const JValue *c = t.get("content"), *id = t.get("id");
+        if (c && id && !c->str.empty()) added.emplace_back(c->str, (uint32_t)id->num);
+      }
+    // the split pattern decides how many digits form one piece
+    if (const JValue* pt = root.get("pre_tokenizer")) {
+      std::string all;
+      collect_strings(*pt, all);
+      if (all.find("\\p{N}{1,3}") != std::string::npos) scan.max_digits = 3;
+    }
+    return true;
+  }
+  static void collect_strings(const JValue& v, std::string& out) {
+    if (v.kind == JValue::STR) { out += v.str; out += '\n'; }
+    for (const JValue& e : v.arr) collect_strings(e, out);
+    for (const auto& kv : v.obj) collect_strings(kv.second, out);
+  }
+
+  // one pre-token (raw bytes) -> ids
+  void bpe(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
+    if (n == 0) return;
+    if (ignore_merges) {
+      std::string whole;
+      for (size_t i = 0; i < n; i++) whole += byte_char[s[i]];
+      auto it = vocab.find(whole);
+      if (it != vocab.end()) { out.push_back(it->second); return; }
+    }
+    std::vector<uint32_t> sym(n);
+    for (size_t i = 0; i < n; i++) sym[i] = byte_id[s[i]];
+    // lowest rank first, leftmost on ties, until no neighbouring pair is a merge
+    while (sym.size() > 1) {
+      uint32_t best = 0xFFFFFFFFu, merged = 0; size_t at = 0;
+      for (size_t i = 0; i + 1 < sym.size(); i++) {
+        auto it = merges.find(((uint64_t)sym[i] << 32) | sym[i + 1]);
+        if (it != merges.end() && it->second.first < best) { best = it->second.first; merged = it->second.second; at = i; }
+      }
+      if (best == 0xFFFFFFFFu) break;
+      sym[at] = merged;
+      sym.erase(sym.begin() + at + 1);
+    }
+    out.insert(out.end(), sym.begin(), sym.end());
+  }
+
+  void encode_plain(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
+    std::vector<Cp> cps;
+    decode_utf8(s, n, 0, cps);
+    size_t i = 0;
+    while (i < cps.size()) {
+      const size_t len = scan.next(cps, i);
+      const size_t b0 = cps[i].off, b1 = i + len < cps.size() ? cps[i + len].off : n;
+      bpe(s + b0, b1 - b0, out);
+      i += len;
+    }
+  }
+
+  void encode(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
+    size_t start = 0, i = 0;
+    while (i < n && !added.empty()) {
+      // leftmost-longest added token at i
+      size_t best_len = 0; uint32_t best_id = 0;
+      for (const auto& a : added)
+        if (a.first.size() > best_len && a.first.size() <= n - i && (uint8_t)a.first[0] == s[i] && !memcmp(a.first.data(), s + i, a.first.size())) {
+          best_len = a.first.size(); best_id = a.second;
+        }
+      if (best_len) {
+        encode_plain(s + start, i - start, out);
+        out.push_back(best_id);
+        i += best_len;
+        start = i;
+      } else {
+        i++;
+      }
+    }
+    encode_plain(s + start, n - start, out);
+  }
+};
+
+thread_local std::string g_last_error;
+
+}  // namespace
+
+extern "C" {
+
+// shim/gigatoken_wrapper/src/lib.rs:19-33: null on failure
+__attribute__((visibility("default"))) void* gt_init(const char* path) {
+  if (!path) { g_last_error = "gt_init: null path"; return nullptr; }
+  Tokenizer* t = new Tokenizer();
+  if (!t->load(path)) { g_last_error = t->error; delete t; return nullptr; }
+  return t;
+}
+
+// lib.rs:35-46: ids of `text` into out_buf; returns the number written (at most out_max), -1 on a null argument
+__attribute__((visibility("default"))) int gt_encode(void* tok, const uint8_t* text, size_t text_len, uint32_t* out_buf, size_t out_max) {
+  if (!tok || !text || !out_buf) return -1;
+  std::vector<uint32_t> ids;
+  ids.reserve(text_len);
+  ((const Tokenizer*)tok)->encode(text, text_len, ids);
+  const size_t n = ids.size() < out_max ? ids.size() : out_max;
+  memcpy(out_buf, ids.data(), n * sizeof(uint32_t));
+  return (int)n;
+}
+
+// lib.rs:90-93
+__attribute__((visibility("default"))) void gt_free(void* tok) { delete (Tokenizer*)tok; }
+
+// why the last gt_init of this thread returned null (not in the reference's wrapper, which only returns null)
+__attribute__((visibility("default"))) const char* gt_last_error(void) { return g_last_error.c_str(); }
+
+}
