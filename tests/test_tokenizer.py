@@ -25,7 +25,8 @@ def _train(path, pattern, ignore_merges=False):
     tok.decoder = decoders.ByteLevel()
     tr = trainers.BpeTrainer(vocab_size=3000, special_tokens=SPECIAL, initial_alphabet=pre_tokenizers.ByteLevel.alphabet(),
                              show_progress=False)
-    text = open(os.path.join(ROOT, "DESIGN.md")).read() + open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, "README.md")).read() + open(os.path.join(ROOT, "bunker_amd", "runner.py")).read()
+    text += open(os.path.join(ROOT, "bunker_amd", "loader.py")).read()
     text += " 日本語のテキスト 한국어 텍스트 naïve café 12345 67 890 😀 " * 20
     tok.train_from_iterator([text[i:i + 1500] for i in range(0, len(text), 1500)], tr)
     tok.save(path)
@@ -59,7 +60,7 @@ def test_encode_equals_hugging_face(tmp_path, pattern, ignore_merges):
     path = str(tmp_path / "tokenizer.json")
     hf = _train(path, pattern, ignore_merges)
     t = tokenizer.Tokenizer(path)
-    docs = [open(os.path.join(ROOT, "README.md")).read(), open(os.path.join(ROOT, "bench.py")).read()[:20000]]
+    docs = [open(os.path.join(ROOT, "bunker_amd", "model.py")).read(), open(os.path.join(ROOT, "bench.py")).read()[:20000]]
     for s in FIXED + _fuzz(np.random.default_rng(7), 600) + docs:
         got, ref = t.encode(s).tolist(), hf.encode(s).ids
         assert got == ref, (s[:80], got[:16], ref[:16])
