@@ -280,6 +280,8 @@ static void launch_fused_pro(int pro, dim3 grid, const FusedArgs& A) {
   else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
 }
 
+int g_tune_fused_cap = 0;     // workgroups per CU of the fused GEMV (0: chosen by the launcher)
+
 // Fast path only (gemv_fused_fast_path says whether it applies); the caller composes the same
 // result from separate kernels otherwise.
 int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
@@ -315,7 +317,10 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
   for (int i = swiglu ? 1 : ngroups; i < 5; i++) A.step_first[i] = steps;
   if (swiglu) A.step_first[0] = 0;
   int wgs = (steps + GEMV_WAVES - 1) / GEMV_WAVES;
-  const int cap = num_cus() * g_tune_cap;
+  // With a prologue every workgroup repeats the RMSNorm / Q8_1 work of the row, so fewer, longer-lived workgroups win:
+  // two per CU measured best (three per CU, one step per wave: 4 % slower over the decode step; one per CU: the rows
+  // in flight no longer cover the memory latency).  Without a prologue the plain GEMV's cap applies.
+  const int cap = num_cus() * (g_tune_fused_cap > 0 ? g_tune_fused_cap : (pro != PRO_Q8 ? 2 : g_tune_cap));
   if (wgs > cap) wgs = cap;
   const dim3 grid(wgs, batch);
   if (swiglu && KB == 4) launch_fused_pro<4, 4, true>(pro, grid, A);

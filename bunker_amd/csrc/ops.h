@@ -40,6 +40,7 @@ int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, i
 int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, int K);
 
 // gemv_fused.hip   pro: 0 = x is Q8_1, 1 = x is bf16 (quantized in the kernel), 2 = rmsnorm(x, norm_w) then quantized
+extern int g_tune_fused_cap;
 bool gemv_fused_fast_path(int K, int batch, bool swiglu);
 int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
                       void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
