@@ -91,8 +91,19 @@ def test_embed_rmsnorm_cast_add_swiglu(orc, dev, batch):
     # cast, add, swiglu
     a = (g.standard_normal((batch, I)) * 3).astype(np.float32); u = g.standard_normal((batch, I)).astype(np.float32)
     dc = dev.empty(batch * I * 2)
+    # values that reach every branch of the conversion: ties, carries into the exponent, denormals, infinities, NaN
+    sp = np.array([0x3F808000, 0x3F818000, 0x3F80FFFF, 0x7F7FFFFF, 0xFF7FFFFF, 0x00000001, 0x00008000, 0x00018000, 0x807FFFFF,
+                   0x7F800000, 0xFF800000, 0x7FC00000, 0x7F800001, 0xFFA12345, 0x00000000, 0x80000000, 0x33800000, 0x477FE000],
+                  np.uint32).view(np.float32)
+    a[0, :sp.size] = sp
     launch(f"cast N={I} batch={batch}", [dev.up(a), dc])
-    assert np.array_equal(rt.from_device(dc, (batch, I), np.uint16), bf(a))
+    got = rt.from_device(dc, (batch, I), np.uint16)
+    ref = np.array([orc.lib().orc_f32_to_bf16(float(v)) if not np.isnan(v) else 0 for v in sp], np.uint16)
+    nan = np.isnan(sp)
+    assert np.array_equal(got[0, :sp.size][~nan], ref[~nan])
+    assert np.all((got[0, :sp.size][nan] & 0x7F80) == 0x7F80) and np.all((got[0, :sp.size][nan] & 0x007F) != 0)   # NaN stays NaN
+    assert np.array_equal(got[:, sp.size:], bf(a)[:, sp.size:])
+    a[0, :sp.size] = 1.0          # the checker's swiglu below is for finite inputs
     launch(f"swiglu N={I} batch={batch}", [dev.up(a), dev.up(u), dc])
     assert np.array_equal(rt.from_device(dc, (batch * I,), np.uint16), orc.swiglu(a.ravel(), u.ravel()))
     p, q = bf(a), bf(u)
