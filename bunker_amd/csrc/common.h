@@ -123,7 +123,23 @@ __device__ __forceinline__ int row16_sum_i32(int v) {
 // arithmetic uses one IEEE operation per written operation (__fmul_rn & co. keep the
 // compiler from fusing), so that these values equal a plain host computation to the bit.
 __device__ __forceinline__ float sigmoid_f64(float v) { return (float)(1.0 / (1.0 + exp(-(double)v))); }
-__device__ __forceinline__ float rsqrt_f64(double v) { return (float)(1.0 / sqrt(v)); }
+// (float)(1 / sqrt(v)) for a normal positive v: the hardware's reciprocal square root estimate (about 2^-26 relative)
+// and one third-order correction y += y * e * (1/2 + 3/8 e), e = 1 - v y^2, leave y within an ulp or so of the double
+// value of 1/sqrt(v) (2^-78 from the iteration, the rest is rounding), which is then rounded once to f32: the same float as
+// the host's correctly rounded sqrt and division give unless the double lies within ~1e-16 of an f32 rounding boundary.
+__device__ __forceinline__ float rsqrt_f64(double v) {
+  const double y = __builtin_amdgcn_rsq(v);
+  const double e = fma(-v * y, y, 1.0);
+  return (float)fma(y, e * fma(0.375, e, 0.5), y);
+}
+
+// a / 127 in double, correctly rounded, for any finite f32 value a: q1 = a * c with c = fl(1/127), the exact residual
+// r = a - 127 q1 by FMA, q = q1 + r c (checked against the division for all 2^23 significands).
+__device__ __forceinline__ double div127_f64(double a) {
+  const double c = 1.0 / 127.0;
+  const double q1 = a * c;
+  return fma(fma(-127.0, q1, a), c, q1);
+}
 
 __device__ __forceinline__ double readlane_f64(double v, int lane) {
   const long long b = __builtin_bit_cast(long long, v);
@@ -148,21 +164,22 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 }
 
 // Q8_1 rounding of one value: q = floor(fl64(f / d) + 0.5) with d = fl64(amax / 127) (bench/bench.ts:53-72,
-// ECMAScript Math.round).  The quotient is first formed in f32 (t = f * (127 / amax), off by at most 3e-5 from
+// ECMAScript Math.round).  The quotient is first formed in f32 (t = f * (127 / amax), off by less than 5e-5 from
 // the double quotient); only when t + 0.5 lies within 2e-4 of an integer — where the two could round
 // differently — is the double division carried out.  Both paths return the reference's integer.
+__device__ __forceinline__ int q8_1_round_exact(float f, double div) {
+  const double qd = (double)f / div;
+  double r = floor(qd);
+  if (qd - r >= 0.5) r += 1.0;
+  return (int)r;
+}
 __device__ __forceinline__ int q8_1_round(float f, float inv, double div) {
   const float u = f * inv + 0.5f;
-  const float fl = floorf(u);
-  const float nr = rintf(u);
-  if (fabsf(u - nr) < 2e-4f) {               // rare: decided by the double quotient (|u - exact| < 5e-5 for |u| <= 128)
-    const double qd = (double)f / div;
-    double r = floor(qd);
-    if (qd - r >= 0.5) r += 1.0;
-    return (int)r;
-  }
-  return (int)fl;
+  if (fabsf(u - rintf(u)) < 2e-4f) return q8_1_round_exact(f, div);      // rare
+  return (int)floorf(u);
 }
+// 127 / amax to within two ulps (the f32 quotient above tolerates it), 0 for an all-zero block
+__device__ __forceinline__ float q8_1_inv(float amax) { return amax != 0.0f ? 127.0f * __builtin_amdgcn_rcpf(amax) : 0.0f; }
 
 // Q8_1 of one 32-element block held by four consecutive lanes (8 values each, already rounded to
 // the activation's storage type).  d = amax/127 in double, s = trunc16(float(sum(q) * d)) with the
@@ -173,16 +190,31 @@ __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk
   for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(f[j]));
   amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
   amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
-  const double d = (double)amax / 127.0, div = d != 0.0 ? d : 1.0;
-  const float inv = amax != 0.0f ? 127.0f / amax : 0.0f;      // amax = 0: every value is 0 and so is every q
+  const double d = div127_f64((double)amax), div = d != 0.0 ? d : 1.0;
+  const float inv = q8_1_inv(amax);
+  // all eight quotients in f32 first; one test tells whether any of them sits near a rounding boundary
+  float u[8];
+  bool near = false;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    u[j] = f[j] * inv + 0.5f;
+    near = near || fabsf(u[j] - rintf(u[j])) < 2e-4f;
+  }
+  int q[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) q[j] = (int)floorf(u[j]);
+  if (near) {                                     // rare: those values are decided by the double quotient
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (fabsf(u[j] - rintf(u[j])) < 2e-4f) q[j] = q8_1_round_exact(f[j], div);
+  }
   int sum = 0;
   pk[0] = 0; pk[1] = 0;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
-    int q = q8_1_round(f[j], inv, div);
-    sum += q;
-    q = q < -128 ? -128 : (q > 127 ? 127 : q);
-    pk[j >> 2] |= (uint32_t)(q & 0xff) << (8 * (j & 3));
+    sum += q[j];
+    const int c = q[j] < -128 ? -128 : (q[j] > 127 ? 127 : q[j]);
+    pk[j >> 2] |= (uint32_t)(c & 0xff) << (8 * (j & 3));
   }
   sum += dpp_i32<DPP_QUAD_XOR1>(sum);
   sum += dpp_i32<DPP_QUAD_XOR2>(sum);
@@ -194,8 +226,8 @@ __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk
 __device__ __forceinline__ void lane32_q8_1_store(float v, uint8_t* __restrict__ blk, int l) {
   float amax = row16_max(fabsf(v));
   amax = fmaxf(amax, __shfl_xor(amax, 16));
-  const double d = (double)amax / 127.0;
-  int q = q8_1_round(v, amax != 0.0f ? 127.0f / amax : 0.0f, d != 0.0 ? d : 1.0);
+  const double d = div127_f64((double)amax);
+  int q = q8_1_round(v, q8_1_inv(amax), d != 0.0 ? d : 1.0);
   int sum = row16_sum_i32(q);
   sum += __shfl_xor(sum, 16);
   q = q < -128 ? -128 : (q > 127 ? 127 : q);

@@ -22,8 +22,8 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const void* __restri
   }
   float amax = row16_max(fabsf(v));
   amax = fmaxf(amax, __shfl_xor(amax, 16));
-  const double d = (double)amax / 127.0;
-  int q = q8_1_round(v, amax != 0.0f ? 127.0f / amax : 0.0f, d != 0.0 ? d : 1.0);
+  const double d = div127_f64((double)amax);
+  int q = q8_1_round(v, q8_1_inv(amax), d != 0.0 ? d : 1.0);
   int sum = row16_sum_i32(q);
   sum += __shfl_xor(sum, 16);
   q = q < -128 ? -128 : (q > 127 ? 127 : q);
