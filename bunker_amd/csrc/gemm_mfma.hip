@@ -4,23 +4,32 @@
 // post-scale (experiments/q4k_q81_final.ts:214-217).
 //
 // One v_mfma_i32_32x32x32_i8 consumes exactly one 32-element sub-block of K for a tile
-// of 32 activation rows (M) x 32 weight rows (N), so the matrix core produces the exact
-// int32 sub-block dots I_j[b, n].  A lane owns weight row n = lane % 32 and 16 of the 32
-// batch rows; it folds the dots with the scales in double, in the same way the GEMV does
+// of 32 weight rows (M) x 32 activation rows (N), so the matrix core produces the exact
+// int32 sub-block dots I_j[n, b].  A lane owns activation row b = lane % 32 and 16 of the 32
+// weight rows; it folds the dots with the scales in double, in the same way the GEMV does
 // (every term exact, ~1e-16 accumulation error, one rounding to f32), so the batched
 // path returns the same bits as the batch-1 path:
 //   y[b, n] = sum_blk ( d * sum_j d8_j[b] * (sc_j * I_j) - dmin * sum_j m_j * s8_j[b] )
+// The first sum is folded on the vector unit: per dot one 24-bit integer multiply by the 6-bit scale (a byte the
+// lane's 16 rows share with its half of the wave, fetched from LDS 16 at a time), one conversion and one FMA with
+// the lane's own activation scale; d comes in once per super-block.  The second sum is a small dense product over
+// the sub-blocks of K and runs on the double-precision matrix instruction (v_mfma_f64_16x16x4_f64), in its own
+// accumulators that join the others once, at the end.
+//
 // Batches of more than 32 rows are cut into 32-row tiles along blockIdx.y (one launch, every tile its own workgroup).
 // A workgroup owns one 32 x 32 output tile; its NW wavefronts split K by super-block (wave w takes
-// blocks w, w + NW, ...) and add their double partials in wave order through LDS at the end.  The
-// int8 activation operand is read straight from the Q8_1 rows (16-byte pieces, L2-resident); only
-// the activation scales of the wave's current super-block are staged in LDS, as doubles.
+// blocks w, w + NW, ...) and add their double partials in wave order through LDS at the end.
+// Each wave copies the 32 x 144 weight bytes and the 32 x 288 activation bytes of its super-block into its own
+// part of LDS with loads in which four neighbouring lanes cover 64 contiguous bytes (a lane-per-row load touches 64
+// cache lines per instruction and leaves the kernel bound by the rate of the L1's address path), one super-block
+// ahead of the arithmetic, and every operand is then read from LDS.
 #include "ops.h"
 
 namespace bk {
 
 typedef __attribute__((ext_vector_type(4))) int i32x4_t;
 typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+typedef __attribute__((ext_vector_type(4))) double f64x4_t;
 
 enum : int { GEPI_F32 = 0, GEPI_BF16 = 1, GEPI_BF16_ADD = 2 };
 
@@ -38,18 +47,31 @@ struct MfmaArgs {
   MfmaGroup g[4];
   int tile_first[5];      // first tile of each matrix; tile_first[i >= ngroups] = number of tiles
   const uint8_t* xq;
-  int nb, B;
+  int nb, B, tiles, btiles;
 };
 
-template <int NW, bool PF>
-__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
-  // one buffer, two uses: during the K loop (d8, s8) of activation block (j, b) of each wave's current super-block, as
-  // doubles [NW][8][32]; afterwards the waves' partial sums [NW][16][64]
-  constexpr int LDS_DS_BYTES = NW * 8 * 32 * 16, LDS_PART_BYTES = NW > 1 ? NW * 16 * 64 * 8 : 0;
-  __shared__ __align__(16) unsigned char lds_raw[LDS_DS_BYTES > LDS_PART_BYTES ? LDS_DS_BYTES : LDS_PART_BYTES];
-  double2 (*lds_ds)[8][32] = (double2 (*)[8][32])lds_raw;
+enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 * GW_ROW, G_WAVE_LDS = GX_BYTES + GW_BYTES + 512 };
 
-  const int tile = blockIdx.x;
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
+  // Per wave: the activation rows of the current super-block as they lie in memory (288 bytes, rows 292 apart so that
+  // the lanes of a read fall into different banks), the weight rows (144 bytes each), and 512 bytes of weight scales
+  // in the order the fold reads them (the 6-bit scales as bytes [8 sub-blocks][2 halves][16 rows], then d as doubles
+  // [2 halves][16 rows]).  After the K loop the same memory holds the waves' partial sums [NW][16][64].
+  __shared__ __align__(16) unsigned char lds_raw[NW * G_WAVE_LDS];
+  static_assert(G_WAVE_LDS >= 16 * 64 * 8 && G_WAVE_LDS % 16 == 0, "the partial sums share the staging memory");
+
+  // Workgroup -> (weight tile, batch tile).  With several batch tiles the workgroups that share a weight tile run next
+  // to each other on one XCD (consecutive workgroup ids go round the 8 XCDs), batch tile fastest: the weight tile comes
+  // from memory once and its other readers find it in that XCD's L2, where the activation rows stay resident.
+  int tile = blockIdx.x, btile = 0;
+  if (A.btiles > 1) {
+    const int per_xcd = (A.tiles * A.btiles + 7) >> 3;
+    const int v = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (v >= A.tiles * A.btiles) return;
+    tile = v / A.btiles;
+    btile = v - tile * A.btiles;
+  }
   const bool s1 = tile >= A.tile_first[1], s2 = tile >= A.tile_first[2], s3 = tile >= A.tile_first[3];
   const uint8_t* __restrict__ W = s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
   void* __restrict__ out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
@@ -57,164 +79,236 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
   const int N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
   const int EPI = s3 ? A.g[3].epi : s2 ? A.g[2].epi : s1 ? A.g[1].epi : A.g[0].epi;
   const int nb = A.nb;
-  const int b0 = blockIdx.y * 32;                     // first batch row of this tile
+  const int b0 = btile * 32;                          // first batch row of this tile
   const int B = min(32, A.B - b0);
-  const uint8_t* __restrict__ xq = A.xq + (int64_t)b0 * nb * 8 * 36;
+  const int64_t wrow_bytes = (int64_t)nb * 144, xrow_bytes = (int64_t)nb * 8 * 36;
+  const uint8_t* __restrict__ xq = A.xq + (int64_t)b0 * xrow_bytes;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int half = lane >> 5, col = lane & 31;
+  const int half = lane >> 5, col = lane & 31, q4 = lane >> 4, l16 = lane & 15;
   const int n0 = (tile - (s3 ? A.tile_first[3] : s2 ? A.tile_first[2] : s1 ? A.tile_first[1] : 0)) * 32;
-  const int n = min(n0 + col, N - 1);                 // rows past N recompute row N-1 and are not stored
-  const uint8_t* wrow = W + (int64_t)n * nb * 144;
-  const int64_t xrow_bytes = (int64_t)nb * 8 * 36;
-  // A operand: batch row `col` (rows past B re-read row B-1; their results are not stored)
-  const uint8_t* xrow = xq + (int64_t)min(col, B - 1) * xrow_bytes + 16 * half;
+  unsigned char* const ldsX = lds_raw + wave * G_WAVE_LDS;
+  unsigned char* const ldsW = ldsX + GX_BYTES;
+  unsigned char* const stage = ldsW + GW_BYTES;
+
+  // Copy maps.  Activations: instruction i = 2c + h covers bytes 64c.. of rows 16h + lane/4, 16 bytes per lane (the
+  // last chunk has 32 bytes per row: lanes 2, 3 of a quad repeat lane 1's piece and do not store).  Rows past B re-read
+  // row B-1 (their results are not stored).  Weights: piece p = lane + 64 i of the 288 16-byte pieces, row p / 9; rows
+  // past N re-read row N-1.
+  const int rq = lane >> 2, k4 = lane & 3;
+  const uint8_t* xsrc[2] = {xq + (int64_t)min(rq, B - 1) * xrow_bytes + 16 * k4, xq + (int64_t)min(16 + rq, B - 1) * xrow_bytes + 16 * k4};
+  const int xtail = 16 * min(k4, 1) - 16 * k4;                 // moves lanes 2, 3 back onto piece 17 in the last chunk
+  unsigned char* const xdst[2] = {ldsX + rq * GX_ROW + 16 * k4, ldsX + (16 + rq) * GX_ROW + 16 * k4};
+  const uint8_t* const wbase = W + (int64_t)n0 * wrow_bytes;
+  uint32_t woff[5];
+#pragma unroll
+  for (int i = 0; i < 5; i++) {
+    const int p = min(lane + 64 * i, 287), row = p / 9;
+    woff[i] = (uint32_t)((min(n0 + row, N - 1) - n0) * (int)wrow_bytes + (p - 9 * row) * 16);
+  }
+  uint4 xr[10], wr0, wr1, wr2, wr3, wr4;
+#define GM_FETCH(BLK)                                                                                                  \
+  {                                                                                                                    \
+    const int fb_ = (BLK);                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < 10; i++) {                                                                   \
+      const uint32_t* p_ = (const uint32_t*)(xsrc[i & 1] + (int64_t)fb_ * 288 + 64 * (i >> 1) + (i >= 8 ? xtail : 0)); \
+      xr[i] = make_uint4(p_[0], p_[1], p_[2], p_[3]); /* 4-byte aligned 16-byte load */                                \
+    }                                                                                                                  \
+    wr0 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[0]);                                                       \
+    wr1 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[1]);                                                       \
+    wr2 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[2]);                                                       \
+    wr3 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[3]);                                                       \
+    wr4 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[4]);                                                       \
+  }
+
+  // where the lane's own weight row sits among the rows of its half: row = 8g + 4h + v  ->  [h][4g + v]
+  const int stage_slot = ((col >> 2) & 1) * 16 + 4 * (col >> 3) + (col & 3);
+  const unsigned char* const myW = ldsW + col * GW_ROW;         // int8 operands: weight row col, batch row col,
+  const unsigned char* const myX = ldsX + col * GX_ROW;         // bytes 16*half.. of every sub-block
 
   double acc[16];
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0;
+  f64x4_t accm[2][2];
+#pragma unroll
+  for (int t = 0; t < 4; t++) accm[t >> 1][t & 1] = (f64x4_t){0.0, 0.0, 0.0, 0.0};
 
-  // weights of this lane's row: header + its half of every 32-byte nibble group.  A wave with several super-blocks
-  // requests the next one's weights (the HBM round trip) behind the current one's activation loads, so that only the
-  // first super-block waits for memory; the requests are unconditional (clamped) to keep the waits countable.
-  uint4 hdr_n, qs_n[4];
-  {
-    const uint8_t* wp = wrow + min(wave, nb - 1) * 144;
-    hdr_n = *(const uint4*)wp;
-#pragma unroll
-    for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
-  }
+  GM_FETCH(min(wave, nb - 1));          // requests are unconditional (clamped): the waits stay countable
   for (int blk = wave; blk < nb; blk += NW) {
-    // activations: the lane's 16 int8 of each of the 8 sub-blocks (4-byte aligned 16-byte loads)
-    uint4 xa4[8];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();     // the previous super-block has been consumed by every lane
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const uint32_t* p = (const uint32_t*)(xrow + (int64_t)(blk * 8 + j) * 36);
-      xa4[j] = make_uint4(p[0], p[1], p[2], p[3]);
+    for (int i = 0; i < 10; i++) {
+      uint32_t* p = (uint32_t*)(xdst[i & 1] + 64 * (i >> 1));
+      if (i < 8 || k4 < 2) { p[0] = xr[i].x; p[1] = xr[i].y; p[2] = xr[i].z; p[3] = xr[i].w; }
     }
-    uint32_t dsraw[4];
+    *(uint4*)(ldsW + lane * 16) = wr0;
+    *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
+    *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
+    *(uint4*)(ldsW + (lane + 192) * 16) = wr3;
+    if (lane < 32) *(uint4*)(ldsW + (lane + 256) * 16) = wr4;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    GM_FETCH(min(blk + NW, nb - 1));     // the next super-block's bytes travel while this one is folded
+
+    // the 6-bit scales of the lane's weight row (half 0 stages sub-blocks 0..3, half 1 sub-blocks 4..7) and its d
+    {
+      const uint4 hdr = *(const uint4*)myW;
+      const uint32_t scw = half ? ((hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4)) : (hdr.y & 0x3f3f3f3fu);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int t = lane + 64 * i;
-      dsraw[i] = *(const uint32_t*)(xq + (int64_t)min(t >> 3, B - 1) * xrow_bytes + (int64_t)(blk * 8 + (t & 7)) * 36 + 32);
-    }
-    const uint4 hdr = hdr_n;
-    uint4 qs[4];
-#pragma unroll
-    for (int g = 0; g < 4; g++) qs[g] = qs_n[g];
-    if (PF) {
-      const uint8_t* wp = wrow + min(blk + NW, nb - 1) * 144;
-      hdr_n = *(const uint4*)wp;
-#pragma unroll
-      for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
-    }
-    // scales of the 32 x 8 activation blocks of this super-block -> LDS of this wave, 4 per lane
-    __builtin_amdgcn_wave_barrier();     // the previous super-block's scales have been consumed by every lane
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int t = lane + 64 * i;
-      const uint32_t ds = dsraw[i];
-      lds_ds[wave][t & 7][t >> 3] = make_double2((double)half_to_f32((uint16_t)(ds & 0xffffu)), (double)half_to_f32((uint16_t)(ds >> 16)));
+      for (int i = 0; i < 4; i++) stage[(4 * half + i) * 32 + stage_slot] = (unsigned char)(scw >> (8 * i));
+      if (!half) ((double*)(stage + 256))[stage_slot] = (double)half_to_f32((uint16_t)(hdr.x & 0xffffu));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    const float d = half_to_f32((uint16_t)(hdr.x & 0xffffu)), dmin = half_to_f32((uint16_t)(hdr.x >> 16));
-    // all eight 6-bit scales and mins of the block, four per dword
-    const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu, m_lo = hdr.z & 0x3f3f3f3fu;
-    const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
-    const uint32_t m_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
-
-    const float dmin_neg = -dmin;
-    // A = activations (M = batch row), B = weights (N = weight row): result[r] = I_j[b = mfma32_row(r), n = col]
-    auto dots = [&](int j) {
-      const uint4 q = qs[j >> 1];
-      i32x4_t wb;
-      if (j & 1) {
-        wb = (i32x4_t){(int)((q.x >> 4) & 0x0f0f0f0fu), (int)((q.y >> 4) & 0x0f0f0f0fu), (int)((q.z >> 4) & 0x0f0f0f0fu),
-                       (int)((q.w >> 4) & 0x0f0f0f0fu)};
-      } else {
-        wb = (i32x4_t){(int)(q.x & 0x0f0f0f0fu), (int)(q.y & 0x0f0f0f0fu), (int)(q.z & 0x0f0f0f0fu), (int)(q.w & 0x0f0f0f0fu)};
-      }
-      const i32x4_t xa = (i32x4_t){(int)xa4[j].x, (int)xa4[j].y, (int)xa4[j].z, (int)xa4[j].w};
-      i32x16_t c;
-#pragma unroll
-      for (int r = 0; r < 16; r++) c[r] = 0;
-      return __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb, c, 0, 0, 0);
+    // A = weights (M = weight row), B = activations (N = batch row): result[r] = I_j[n = mfma32_row(r), b = col]
+    auto unpack = [](const uint4 q, int odd) {
+      if (odd) return (i32x4_t){(int)((q.x >> 4) & 0x0f0f0f0fu), (int)((q.y >> 4) & 0x0f0f0f0fu), (int)((q.z >> 4) & 0x0f0f0f0fu),
+                                (int)((q.w >> 4) & 0x0f0f0f0fu)};
+      return (i32x4_t){(int)(q.x & 0x0f0f0f0fu), (int)(q.y & 0x0f0f0f0fu), (int)(q.z & 0x0f0f0f0fu), (int)(q.w & 0x0f0f0f0fu)};
     };
-    // The fold runs as a pipeline over the 16 groups (sub-block j, eight of the lane's sixteen outputs): the activation
-    // scales of group g+1 are requested from LDS and the matrix instruction of sub-block j+1 is issued before group g
-    // is folded, so neither latency is exposed.  Per sub-block the lane's row contributes two factors, both exact in f32
-    // (11-bit x 6-bit): d * sc_j and -dmin * m_j; every term (d*sc_j) * (d8 * I) and (-dmin*m_j) * s8 is exact in double.
-    double2 dsa[8], dsb[8];
+    auto load_x = [&](int j) {
+      const uint32_t* xp = (const uint32_t*)(myX + j * 36 + 16 * half);
+      return (i32x4_t){(int)xp[0], (int)xp[1], (int)xp[2], (int)xp[3]};
+    };
+    auto mfma = [](i32x4_t wb, i32x4_t xa) {
+      i32x16_t z;
 #pragma unroll
-    for (int r = 0; r < 8; r++) dsa[r] = lds_ds[wave][0][mfma32_row(r, half)];
-    i32x16_t c = dots(0), cn = c;
+      for (int r = 0; r < 16; r++) z[r] = 0;
+      return __builtin_amdgcn_mfma_i32_32x32x32_i8(wb, xa, z, 0, 0, 0);
+    };
+    // The fold runs as a pipeline over the sub-blocks: the operands and scale bytes of sub-block j+1 are requested from
+    // LDS before sub-block j is folded and its matrix instruction is issued halfway through that fold, when they have
+    // arrived; the second half of the fold covers the matrix instruction's latency.  sc_j * I_j is an integer below 2^23;
+    // its product with d8_j (11 bits) is exact inside the FMA, and so is d (11 bits) times the sum over the eight
+    // sub-blocks as long as that sum has not been rounded (the terms of one activation row lie within a few binades of
+    // each other).
+    double S1[16];
+    uint4 q = *(const uint4*)(myW + 16 + 16 * half), qn = q;
+    uint4 scb = *(const uint4*)(stage + 16 * half), scn = scb;
+    uint32_t dsw = *(const uint32_t*)(myX + 32), dsn = dsw;
+    i32x4_t xn = load_x(0);
+    i32x16_t c = mfma(unpack(q, 0), xn), cn = c;
 #pragma unroll
-    for (int g = 0; g < 16; g++) {
-      const int j = g >> 1, r0 = 8 * (g & 1);
-      double2 (&cur)[8] = (g & 1) ? dsb : dsa;
-      double2 (&nxt)[8] = (g & 1) ? dsa : dsb;
-      if (g + 1 < 16) {
-#pragma unroll
-        for (int r = 0; r < 8; r++) nxt[r] = lds_ds[wave][(g + 1) >> 1][mfma32_row(8 * ((g + 1) & 1) + r, half)];
+    for (int j = 0; j < 8; j++) {
+      if (j + 1 < 8) {
+        scn = *(const uint4*)(stage + (j + 1) * 32 + 16 * half);
+        dsn = *(const uint32_t*)(myX + (j + 1) * 36 + 32);
+        xn = load_x(j + 1);
+        if (j & 1) qn = *(const uint4*)(myW + 16 + 32 * ((j + 1) >> 1) + 16 * half);
       }
-      if (!(g & 1) && j + 1 < 8) cn = dots(j + 1);
       __builtin_amdgcn_sched_barrier(0);
-      const double dsc = (double)(d * (float)(((j < 4 ? sc_lo : sc_hi) >> (8 * (j & 3))) & 0xffu));
-      const double dmm = (double)(dmin_neg * (float)(((j < 4 ? m_lo : m_hi) >> (8 * (j & 3))) & 0xffu));
+      const double d8 = (double)half_to_f32((uint16_t)(dsw & 0xffffu));
+      const uint32_t scv[4] = {scb.x, scb.y, scb.z, scb.w};
 #pragma unroll
       for (int r = 0; r < 8; r++) {
-        const double t = cur[r].x * (double)c[r0 + r];            // d8 * I: 11-bit x 17-bit, exact
-        acc[r0 + r] = fma(dsc, t, acc[r0 + r]);
-        acc[r0 + r] = fma(dmm, cur[r].y, acc[r0 + r]);
+        const double t = (double)__mul24(c[r], (int)((scv[r >> 2] >> (8 * (r & 3))) & 0xffu));
+        S1[r] = j == 0 ? d8 * t : fma(d8, t, S1[r]);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (g & 1) c = cn;
-    }
-    if (!PF) {
-      const uint8_t* wp = wrow + min(blk + NW, nb - 1) * 144;
-      hdr_n = *(const uint4*)wp;
+      if (j + 1 < 8) {
+        if (j & 1) q = qn;
+        cn = mfma(unpack(q, (j + 1) & 1), xn);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int g = 0; g < 4; g++) qs_n[g] = *(const uint4*)(wp + 16 + 32 * g + 16 * half);
+      for (int r = 8; r < 16; r++) {
+        const double t = (double)__mul24(c[r], (int)((scv[r >> 2] >> (8 * (r & 3))) & 0xffu));
+        S1[r] = j == 0 ? d8 * t : fma(d8, t, S1[r]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      c = cn; scb = scn; dsw = dsn;
     }
+    {
+      const double2* dd = (const double2*)(stage + 256 + 128 * half);
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const double2 v = dd[r >> 1];
+        acc[r] = fma(v.x, S1[r], acc[r]);
+        acc[r + 1] = fma(v.y, S1[r + 1], acc[r + 1]);
+      }
+    }
+    // min term: accm[tn][tb] += (-dmin * m_j)[16 rows x 4 sub-blocks] . s8_j[4 sub-blocks x 16 batch rows], for the
+    // sub-blocks 0..3 and then 4..7; a lane supplies row 16 t + l16 of either side at sub-blocks q4 and 4 + q4
+    double am[2][2], bm[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const uint4 hm = *(const uint4*)(ldsW + (16 * t + l16) * GW_ROW);
+      const float dmin_neg = -half_to_f32((uint16_t)(hm.x >> 16));
+      const uint32_t zb = (hm.z >> (8 * q4)) & 0xffu, wb = (hm.w >> (8 * q4)) & 0xffu;
+      am[t][0] = (double)(dmin_neg * (float)(zb & 63u));
+      am[t][1] = (double)(dmin_neg * (float)((wb >> 4) | ((zb >> 6) << 4)));
+      const unsigned char* xs = ldsX + (16 * t + l16) * GX_ROW + q4 * 36 + 34;
+      bm[t][0] = (double)half_to_f32(*(const uint16_t*)xs);
+      bm[t][1] = (double)half_to_f32(*(const uint16_t*)(xs + 144));
+    }
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+        accm[t >> 1][t & 1] = __builtin_amdgcn_mfma_f64_16x16x4f64(am[t >> 1][k], bm[t & 1][k], accm[t >> 1][t & 1], 0, 0, 0);
   }
 
-  auto store = [&](int r, double total) {
-    const int b = mfma32_row(r, half);
-    if (n0 + col >= N || b >= B) return;
-    const int64_t o = (int64_t)(b0 + b) * N + n0 + col;
+  // The min-term accumulators hold element (n = 16 tn + 4 v + q4, b = 16 tb + l16); they reach the lanes that own those
+  // outputs through this wave's part of the buffer.  Slot (r, lane) of a wave's part sits at r*64 + (lane ^ (r + 16*half)):
+  // the swizzle keeps the transposed reads of the last step free of bank conflicts.
+  double* part = (double*)lds_raw + wave * 16 * 64;
+  __syncthreads();                         // all waves are done with the scales that share the buffer
+#pragma unroll
+  for (int t = 0; t < 4; t++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int n = 16 * (t >> 1) + 4 * v + q4, b = 16 * (t & 1) + l16;
+      const int rr = 4 * (n >> 3) + (n & 3), hh = (n >> 2) & 1;
+      part[rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh))] = accm[t >> 1][t & 1][v];
+    }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] += part[r * 64 + (lane ^ (r + 16 * half))];
+
+  auto store = [&](int n_in_tile, int b, double total) {
+    const int n = n0 + n_in_tile;
+    if (n >= N || b >= B) return;
+    const int64_t o = (int64_t)(b0 + b) * N + n;
     const float v = (float)total;
     if (EPI == GEPI_F32) ((float*)out)[o] = v;
     else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
     else ((uint16_t*)out)[o] = f32_to_bf16(bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(res[o]));
   };
   if (NW > 1) {
-    // every wave leaves its 16 partial sums per lane in LDS; then wave w finishes outputs r = w*16/NW .. of every lane:
-    // the partials are added in wave order, and the conversions and stores are spread over all waves
-    double* part = (double*)lds_raw;
-    __syncthreads();                       // all waves are done with the activation scales that share the buffer
+    // every wave leaves its 16 partial sums per lane in LDS; then the threads finish the outputs with the weight row
+    // along the lanes (contiguous stores): thread (wave w, lane) takes row lane % 32 and batch rows 2 (w R + i) + lane / 32;
+    // the partials are added in wave order
+    __builtin_amdgcn_wave_barrier();       // slot (r, lane) was read above by this lane only
 #pragma unroll
-    for (int r = 0; r < 16; r++) part[(wave * 16 + r) * 64 + lane] = acc[r];
+    for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
     __syncthreads();
+    const double* all = (const double*)lds_raw;
     constexpr int R = 16 / NW;
+    const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
 #pragma unroll
-    for (int rr = 0; rr < R; rr++) {
-      const int r = wave * R + rr;
-      double t = part[r * 64 + lane];
+    for (int i = 0; i < R; i++) {
+      const int b = 2 * (wave * R + i) + half;
+      const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
+      double t = all[slot];
 #pragma unroll
-      for (int w = 1; w < NW; w++) t += part[(w * 16 + r) * 64 + lane];
-      store(r, t);
+      for (int w = 1; w < NW; w++) t += all[w * 16 * 64 + slot];
+      store(col, b, t);
     }
   } else {
 #pragma unroll
-    for (int r = 0; r < 16; r++) store(r, acc[r]);
+    for (int r = 0; r < 16; r++) store(mfma32_row(r, half), col, acc[r]);
   }
 }
 
+#undef GM_FETCH
+
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
-int g_tune_gemm_pf = -1;     // next-block weight prefetch: 0 off, 1 on, -1 = chosen from the shape
 
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi) {
@@ -235,30 +329,22 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   }
   for (int i = ngroups; i < 5; i++) A.tile_first[i] = tiles;
   // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
-  // and two ways when the tiles alone fill the chip many times over (lm_head)
+  // and not at all when the tiles alone fill the chip many times over (lm_head, prompt batches)
   const int btiles = (batch + 31) / 32;
   const int64_t wgs = (int64_t)tiles * btiles;
   int nw = g_tune_gemm_nw;
   if (nw <= 0) {
     nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
     if (wgs <= num_cus() + num_cus() / 4 && A.nb >= 8) nw = 8;          // about a tile per CU: one super-block per wave
-    if (wgs >= 8 * num_cus() && nw > 2) nw = 2;
+    if (wgs >= 8 * num_cus()) nw = 1;                                     // the tiles alone fill the chip many times over
   }
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
-  // next-block weight prefetch for waves with several super-blocks; not when the chip is full of tiles anyway
-  // (it costs 20 registers: two waves per SIMD instead of three)
-  const bool pf = g_tune_gemm_pf >= 0 ? g_tune_gemm_pf != 0 : ((A.nb + nw - 1) / nw >= 2 && wgs * nw <= 8 * num_cus());
-  const dim3 grid(tiles, btiles);
-#define BK_GEMM_LAUNCH(NWV)                                                                                             \
-  {                                                                                                                     \
-    if (pf) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<NWV, true>), grid, dim3(64 * NWV), 0, stream(), A);           \
-    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<NWV, false>), grid, dim3(64 * NWV), 0, stream(), A);             \
-  }
-  if (nw == 8) BK_GEMM_LAUNCH(8)
-  else if (nw == 4) BK_GEMM_LAUNCH(4)
-  else if (nw == 2) BK_GEMM_LAUNCH(2)
-  else BK_GEMM_LAUNCH(1)
-#undef BK_GEMM_LAUNCH
+  A.tiles = tiles; A.btiles = btiles;
+  const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
+  if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8>), grid, dim3(512), 0, stream(), A);
+  else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4>), grid, dim3(256), 0, stream(), A);
+  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2>), grid, dim3(128), 0, stream(), A);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1>), grid, dim3(64), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -46,7 +46,7 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
                       void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
 
 // gemm_mfma.hip
-extern int g_tune_gemm_nw, g_tune_gemm_pf;
+extern int g_tune_gemm_nw;
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi);
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
