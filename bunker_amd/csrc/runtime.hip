@@ -16,7 +16,9 @@ namespace bk {
 static thread_local char g_err[1024] = "";
 static bool g_inited = false;
 static int g_device = -1;
-static hipStream_t g_stream = nullptr;
+static hipStream_t g_stream = nullptr;         // the stream launches and copies go to (bk_stream_use)
+static hipStream_t g_main_stream = nullptr;    // the one bk_init made
+static std::vector<hipStream_t> g_extra_streams;
 static int g_cus = 256;
 
 int set_error(int code, const char* fmt, ...) {
@@ -27,6 +29,12 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 hipStream_t stream() { return g_stream; }
+// the host waits for every stream of the library
+static int sync_all() {
+  BK_HIP(hipStreamSynchronize(g_main_stream));
+  for (hipStream_t st : g_extra_streams) BK_HIP(hipStreamSynchronize(st));
+  return BK_OK;
+}
 int num_cus() { return g_cus; }
 bool inited() { return g_inited; }
 
@@ -52,7 +60,7 @@ int prof_end() {
 }
 std::string kernel_label(int kernel);   // api.hip
 static int prof_collect() {
-  BK_HIP(hipStreamSynchronize(g_stream));
+  if (int rc = sync_all()) return rc;
   for (auto& p : g_pending) {
     float ms = 0;
     if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
@@ -91,7 +99,8 @@ int bk_init(int device) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return set_error(BK_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
   g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  BK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  BK_HIP(hipStreamCreateWithFlags(&g_main_stream, hipStreamNonBlocking));
+  g_stream = g_main_stream;
   g_device = device;
   g_inited = true;
   return BK_OK;
@@ -99,12 +108,14 @@ int bk_init(int device) {
 
 int bk_shutdown(void) {
   if (!g_inited) return BK_OK;
-  (void)hipStreamSynchronize(g_stream);
+  (void)sync_all();
   for (auto& p : g_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto& ev : g_pool) (void)hipEventDestroy(ev);
   g_pending.clear(); g_pool.clear(); g_totals.clear();
-  (void)hipStreamDestroy(g_stream);
-  g_stream = nullptr; g_inited = false; g_device = -1;
+  for (hipStream_t st : g_extra_streams) (void)hipStreamDestroy(st);
+  g_extra_streams.clear();
+  (void)hipStreamDestroy(g_main_stream);
+  g_stream = g_main_stream = nullptr; g_inited = false; g_device = -1;
   return BK_OK;
 }
 
@@ -133,7 +144,7 @@ int bk_alloc(uint64_t bytes, uint64_t* out) {
 int bk_free(uint64_t ptr) {
   BK_NEED_INIT();
   if (!ptr) return BK_OK;
-  BK_HIP(hipStreamSynchronize(g_stream));
+  if (int rc = sync_all()) return rc;
   BK_HIP(hipFree((void*)(uintptr_t)ptr));
   return BK_OK;
 }
@@ -207,7 +218,47 @@ int bk_memset(uint64_t dst, int value, uint64_t bytes) {
 }
 int bk_sync(void) {
   BK_NEED_INIT();
-  BK_HIP(hipStreamSynchronize(g_stream));
+  return sync_all();
+}
+
+// Further streams (default priority) for work that may overlap: launches, copies and event records go to the stream
+// selected last; the order between streams is the caller's, through events.
+int bk_stream_create(uint64_t* out) {
+  BK_NEED_INIT();
+  BK_REQUIRE(out, "bk_stream_create: null out");
+  hipStream_t st;
+  BK_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+  g_extra_streams.push_back(st);
+  *out = (uint64_t)(uintptr_t)st;
+  return BK_OK;
+}
+static int find_stream(uint64_t s) {
+  for (size_t i = 0; i < g_extra_streams.size(); i++)
+    if ((uint64_t)(uintptr_t)g_extra_streams[i] == s) return (int)i;
+  return -1;
+}
+int bk_stream_use(uint64_t s) {
+  BK_NEED_INIT();
+  if (!s) { g_stream = g_main_stream; return BK_OK; }
+  const int i = find_stream(s);
+  BK_REQUIRE(i >= 0, "bk_stream_use: not a stream of bk_stream_create");
+  g_stream = g_extra_streams[i];
+  return BK_OK;
+}
+int bk_stream_wait_event(uint64_t ev) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ev, "bk_stream_wait_event: null event");
+  BK_HIP(hipStreamWaitEvent(g_stream, (hipEvent_t)(uintptr_t)ev, 0));
+  return BK_OK;
+}
+int bk_stream_destroy(uint64_t s) {
+  BK_NEED_INIT();
+  const int i = find_stream(s);
+  BK_REQUIRE(i >= 0, "bk_stream_destroy: not a stream of bk_stream_create");
+  BK_HIP(hipStreamSynchronize(g_extra_streams[i]));
+  if (g_stream == g_extra_streams[i]) g_stream = g_main_stream;
+  BK_HIP(hipStreamDestroy(g_extra_streams[i]));
+  g_extra_streams.erase(g_extra_streams.begin() + i);
   return BK_OK;
 }
 

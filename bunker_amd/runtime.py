@@ -40,6 +40,7 @@ _SIGS = {
     "bk_memset": [u64, i32, u64], "bk_sync": [],
     "bk_host_alloc": [u64, C.POINTER(u64)], "bk_host_free": [u64],
     "bk_htod_async": [u64, vp, u64], "bk_dtoh_async": [vp, u64, u64], "bk_event_sync": [u64],
+    "bk_stream_create": [C.POINTER(u64)], "bk_stream_use": [u64], "bk_stream_wait_event": [u64], "bk_stream_destroy": [u64],
     "bk_event_create": [C.POINTER(u64)], "bk_event_record": [u64],
     "bk_event_elapsed_ms": [u64, u64, C.POINTER(C.c_float)], "bk_event_destroy": [u64],
     "bk_prof_enable": [i32], "bk_prof_reset": [], "bk_prof_report": [C.c_char_p, i32],
@@ -292,6 +293,56 @@ class Event:
 
 def eventSync(ev: "Event") -> None:
     ev.sync()
+
+
+_cur_stream = 0      # handle of the selected stream (0 = the library's first)
+
+
+def _use_stream(h: int) -> None:
+    global _cur_stream
+    _check(cu().bk_stream_use(h), "bk_stream_use")
+    _cur_stream = h
+
+
+class Stream:
+    """A further stream of the library: ``with stream: ...`` sends launches, copies and event records there;
+    ``stream.wait(event)`` orders it behind an event recorded on another stream."""
+
+    def __init__(self):
+        h = u64(0)
+        _check(cu().bk_stream_create(C.byref(h)), "bk_stream_create")
+        self.h = int(h.value)
+        self._prev: list[int] = []
+
+    def __enter__(self):
+        self._prev.append(_cur_stream)
+        _use_stream(self.h)
+        return self
+
+    def __exit__(self, *exc):
+        _use_stream(self._prev.pop())
+        return False
+
+    def wait(self, ev: "Event") -> None:
+        """Work queued on this stream from now on starts after ``ev`` has happened."""
+        prev = _cur_stream
+        _use_stream(self.h)
+        try:
+            _check(cu().bk_stream_wait_event(ev.h), "bk_stream_wait_event")
+        finally:
+            _use_stream(prev)
+
+    def destroy(self):
+        if self.h:
+            if _cur_stream == self.h:
+                _use_stream(0)
+            cu().bk_stream_destroy(self.h)
+            self.h = 0
+
+
+def streamWaitEvent(ev: "Event") -> None:
+    """The stream selected now (the first one outside a ``with Stream``) waits for ``ev``."""
+    _check(cu().bk_stream_wait_event(ev.h), "bk_stream_wait_event")
 
 
 class Graph:

@@ -53,10 +53,18 @@ BK_API int bk_dtoh_async(void* dst, uint64_t src, uint64_t bytes);
 
 /* ---- timing: replaces the cuEvent* calls of src/ttir.ts:352-417 */
 BK_API int bk_event_create(uint64_t* out);
-BK_API int bk_event_record(uint64_t ev);             /* on the library's stream */
+BK_API int bk_event_record(uint64_t ev);             /* on the selected stream */
 BK_API int bk_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms);  /* waits for stop */
 BK_API int bk_event_sync(uint64_t ev);                /* host waits until the event has happened */
 BK_API int bk_event_destroy(uint64_t ev);
+/* Further streams for work that may overlap (the reference runs everything on stream 0, src/ttir.ts:321-348, and its
+ * prompt prototypes have no counterpart): after bk_stream_use(s) launches, copies and bk_event_record go to stream s
+ * (0 = the library's first stream); bk_stream_wait_event makes the selected stream wait for an event recorded on
+ * another one.  bk_sync and bk_free wait for all streams.  Single host thread, like every other call here. */
+BK_API int bk_stream_create(uint64_t* out);
+BK_API int bk_stream_use(uint64_t stream);
+BK_API int bk_stream_wait_event(uint64_t ev);
+BK_API int bk_stream_destroy(uint64_t stream);
 BK_API int bk_prof_enable(int on);                   /* BUNKER_GPU_PROF=1: an event pair around every bk_launch */
 BK_API int bk_prof_reset(void);                      /* profGpuReset, src/ttir.ts:385-388 */
 BK_API int bk_prof_report(char* buf, int cap);       /* profGpuReport, src/ttir.ts:391-417; text table */

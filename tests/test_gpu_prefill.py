@@ -168,3 +168,38 @@ def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
         toks, pos = idx, pos + 1
     assert max(ref.attn_err) <= 2e-2
     env.close()
+
+
+@pytest.mark.parametrize("n_prompt,chunk", [(61, 8), (40, 16)])
+def test_prefill_two_chunks_in_flight_equals_one(orc, n_prompt, chunk):
+    """Two chunks in flight on two streams (each layer's state hand-over ordered by events) leave the same bytes as
+    one chunk at a time: logits of the last prompt token, first token, and every state tensor."""
+    print(f"prefill overlap n={n_prompt} chunk={chunk}", flush=True)
+    D = TINY
+    B, seq = 2, 1
+    W = synth_model.synth_weights(D, seed=51)
+    S = synth_model.synth_state(D, B, seed=52)
+    prompt = synth.rng(53).integers(0, D.VOCAB, n_prompt).astype(np.int32)
+    g = model.buildModelGraph(D, B)
+    results = []
+    for overlap in (False, True, True):
+        env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+        pf = prefill.Prefill(D, env, chunk=chunk, overlap=overlap)
+        tok, val = pf.run(prompt[:n_prompt // 2], seq=seq, pos0=0)            # two runs: the second continues the first
+        tok, val = pf.run(prompt[n_prompt // 2:], seq=seq, pos0=n_prompt // 2)
+        state = {"logits": rt.from_device(pf.d_logits, (D.VOCAB,), np.float32).view(np.uint32), "tok": tok,
+                 "val": np.float32(val).view(np.uint32)}
+        for l in range(D.NL):
+            p = f"model.layers.{l}"
+            if not D.is_full_attention(l):
+                state[p + ".S"] = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32).view(np.uint32)
+                state[p + ".conv"] = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)
+            else:
+                state[p + ".k"] = env.read_state(f"{p}.kv_k", (B, D.MAX_LEN // 16, D.NKV, 16, D.HD), np.uint16)
+                state[p + ".v"] = env.read_state(f"{p}.kv_v", (B, D.MAX_LEN // 16, D.NKV, D.HD, 16), np.uint16)
+        results.append(state)
+        pf.close()
+        env.close()
+    for other in results[1:]:
+        for key, v in results[0].items():
+            assert np.array_equal(v, other[key]), key
