@@ -119,6 +119,8 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   if (pro == 2) { if ((rc = launch_rmsnorm(x, nw, nullptr, k.scratch, K, batch))) return rc; xq = k.scratch; }
   else if (pro == 1) { if ((rc = launch_quantize_q8_1(x, DT_BF16, k.scratch, K, batch))) return rc; xq = k.scratch; }
   if (swiglu) {
+    // batched and with a Q8_1 result: SwiGLU and the quantization are the matmul kernel's last step
+    if (q8out && batch >= GEMM_MFMA_MIN_BATCH) return launch_gemm_swiglu_mfma(xq, K, batch, W[0], W[1], N[0], out[0], q8out);
     float* g = (float*)((uint8_t*)k.scratch + (size_t)batch * (K / 32) * 36);
     float* u = g + (size_t)batch * N[0];
     if (batch >= GEMM_MFMA_MIN_BATCH) {

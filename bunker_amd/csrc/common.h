@@ -222,8 +222,9 @@ __device__ __forceinline__ uint32_t quad_q8_1(const float (&f)[8], uint32_t (&pk
 }
 
 // Q8_1 of one 32-element block whose values sit one per lane in an aligned group of 32 lanes (all 32 active): every lane
-// stores its int8, the first lane of the group the (d, s) pair.  `blk` points at the 36-byte block, l = lane % 32.
-__device__ __forceinline__ void lane32_q8_1_store(float v, uint8_t* __restrict__ blk, int l) {
+// stores its int8, the first lane of the group the (d, s) pair (`store` = false for a whole group: nothing is written).
+// `blk` points at the 36-byte block, l = lane % 32.
+__device__ __forceinline__ void lane32_q8_1_store(float v, uint8_t* __restrict__ blk, int l, bool store = true) {
   float amax = row16_max(fabsf(v));
   amax = fmaxf(amax, __shfl_xor(amax, 16));
   const double d = div127_f64((double)amax);
@@ -231,6 +232,7 @@ __device__ __forceinline__ void lane32_q8_1_store(float v, uint8_t* __restrict__
   int sum = row16_sum_i32(q);
   sum += __shfl_xor(sum, 16);
   q = q < -128 ? -128 : (q > 127 ? 127 : q);
+  if (!store) return;                      // the group took part in the exchanges above; nothing of it is kept
   blk[l] = (uint8_t)(int8_t)q;
   if (l == 0)
     *(uint32_t*)(blk + 32) = (uint32_t)f32_to_half_trunc((float)d) | ((uint32_t)f32_to_half_trunc((float)((double)sum * d)) << 16);

@@ -48,17 +48,21 @@ struct MfmaArgs {
   int tile_first[5];      // first tile of each matrix; tile_first[i >= ngroups] = number of tiles
   const uint8_t* xq;
   int nb, B, tiles, btiles;
+  uint8_t* out_q8;        // SwiGLU form: g[0] = gate (out = bf16 activation or null), g[1] = up; Q8_1 blocks of the activation
 };
 
 enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 * GW_ROW, G_WAVE_LDS = GX_BYTES + GW_BYTES + 512 };
 
-template <int NW>
-__global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
+// SWIGLU: the workgroup holds 2 NW waves; waves 0..NW-1 form the tile of 32 gate rows, waves NW..2NW-1 the tile of the
+// same 32 up rows, and the last step writes act = bf16(silu(g) * u) and its Q8_1 block instead of g and u.
+template <int NW, bool SWIGLU>
+__global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
+  constexpr int WAVES = NW * (SWIGLU ? 2 : 1);
   // Per wave: the activation rows of the current super-block as they lie in memory (288 bytes, rows 292 apart so that
   // the lanes of a read fall into different banks), the weight rows (144 bytes each), and 512 bytes of weight scales
   // in the order the fold reads them (the 6-bit scales as bytes [8 sub-blocks][2 halves][16 rows], then d as doubles
-  // [2 halves][16 rows]).  After the K loop the same memory holds the waves' partial sums [NW][16][64].
-  __shared__ __align__(16) unsigned char lds_raw[NW * G_WAVE_LDS];
+  // [2 halves][16 rows]).  After the K loop the same memory holds the waves' partial sums [WAVES][16][64].
+  __shared__ __align__(16) unsigned char lds_raw[WAVES * G_WAVE_LDS];
   static_assert(G_WAVE_LDS >= 16 * 64 * 8 && G_WAVE_LDS % 16 == 0, "the partial sums share the staging memory");
 
   // Workgroup -> (weight tile, batch tile).  With several batch tiles the workgroups that share a weight tile run next
@@ -72,8 +76,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
     tile = v / A.btiles;
     btile = v - tile * A.btiles;
   }
-  const bool s1 = tile >= A.tile_first[1], s2 = tile >= A.tile_first[2], s3 = tile >= A.tile_first[3];
-  const uint8_t* __restrict__ W = s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kw = SWIGLU ? wave % NW : wave;           // this wave's place in the split of K
+  const bool s1 = !SWIGLU && tile >= A.tile_first[1], s2 = !SWIGLU && tile >= A.tile_first[2], s3 = !SWIGLU && tile >= A.tile_first[3];
+  const uint8_t* __restrict__ W = SWIGLU ? A.g[wave / NW].W : s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
   void* __restrict__ out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
   const uint16_t* __restrict__ res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
   const int N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
@@ -84,7 +90,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
   const int64_t wrow_bytes = (int64_t)nb * 144, xrow_bytes = (int64_t)nb * 8 * 36;
   const uint8_t* __restrict__ xq = A.xq + (int64_t)b0 * xrow_bytes;
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = lane >> 5, col = lane & 31, q4 = lane >> 4, l16 = lane & 15;
   const int n0 = (tile - (s3 ? A.tile_first[3] : s2 ? A.tile_first[2] : s1 ? A.tile_first[1] : 0)) * 32;
   unsigned char* const ldsX = lds_raw + wave * G_WAVE_LDS;
@@ -133,8 +138,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
 #pragma unroll
   for (int t = 0; t < 4; t++) accm[t >> 1][t & 1] = (f64x4_t){0.0, 0.0, 0.0, 0.0};
 
-  GM_FETCH(min(wave, nb - 1));          // requests are unconditional (clamped): the waits stay countable
-  for (int blk = wave; blk < nb; blk += NW) {
+  GM_FETCH(min(kw, nb - 1));            // requests are unconditional (clamped): the waits stay countable
+  for (int blk = kw; blk < nb; blk += NW) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();     // the previous super-block has been consumed by every lane
 #pragma unroll
@@ -280,7 +285,32 @@ __global__ __launch_bounds__(64 * NW) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A)
     else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
     else ((uint16_t*)out)[o] = f32_to_bf16(bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(res[o]));
   };
-  if (NW > 1) {
+  if (SWIGLU) {
+    // both tiles' partials meet in LDS; thread (wave w, lane) then takes output column lane % 32 and batch rows
+    // 2 (w R + i) + lane / 32: g and u are added in wave order and rounded to f32 like the matmul's own outputs, the
+    // 32 lanes of a half hold one Q8_1 block of the activation
+    __builtin_amdgcn_wave_barrier();       // slot (r, lane) was read above by this lane only
+#pragma unroll
+    for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
+    __syncthreads();
+    const double* all = (const double*)lds_raw;
+    constexpr int R = 16 / WAVES;
+    const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
+    uint16_t* act = (uint16_t*)A.g[0].out;
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+      const int b = 2 * (wave * R + i) + half;
+      const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
+      double gd = all[slot], ud = all[NW * 16 * 64 + slot];
+#pragma unroll
+      for (int w = 1; w < NW; w++) { gd += all[w * 16 * 64 + slot]; ud += all[(NW + w) * 16 * 64 + slot]; }
+      const float g = (float)gd, u = (float)ud;
+      const uint16_t a16 = f32_to_bf16(__fmul_rn(__fmul_rn(g, sigmoid_f64(g)), u));
+      const bool valid = b < B;
+      if (valid && act) act[(int64_t)(b0 + b) * N + n0 + col] = a16;
+      lane32_q8_1_store(bf16_to_f32(a16), A.out_q8 + ((int64_t)(b0 + b) * (N / 32) + (n0 >> 5)) * 36, col, valid);
+    }
+  } else if (NW > 1) {
     // every wave leaves its 16 partial sums per lane in LDS; then the threads finish the outputs with the weight row
     // along the lanes (contiguous stores): thread (wave w, lane) takes row lane % 32 and batch rows 2 (w R + i) + lane / 32;
     // the partials are added in wave order
@@ -341,10 +371,10 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
   A.tiles = tiles; A.btiles = btiles;
   const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
-  if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8>), grid, dim3(512), 0, stream(), A);
-  else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4>), grid, dim3(256), 0, stream(), A);
-  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2>), grid, dim3(128), 0, stream(), A);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1>), grid, dim3(64), 0, stream(), A);
+  if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false>), grid, dim3(512), 0, stream(), A);
+  else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false>), grid, dim3(256), 0, stream(), A);
+  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, false>), grid, dim3(128), 0, stream(), A);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, false>), grid, dim3(64), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
@@ -356,6 +386,44 @@ int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int
   BK_REQUIRE(!(residual && out_dtype != DT_BF16), "gemm_q4k_q8_1_mfma: a residual needs bf16 output");
   const int epi = out_dtype == DT_F32 ? GEPI_F32 : (residual ? GEPI_BF16_ADD : GEPI_BF16);
   return launch_gemm_group_mfma(xq, K, batch, 1, &W, &y, &residual, &N, &epi);
+}
+
+}  // namespace bk
+
+namespace bk {
+
+// gate and up projections with the SwiGLU and the Q8_1 quantization of its result in the last step of the matmul:
+// act[b, n] = bf16(silu(g) * u) (src/fusion.ts:324-330 on the two matmuls' f32 outputs), written as bf16 (if `act` is
+// given) and as the Q8_1 blocks the down projection reads.
+int launch_gemm_swiglu_mfma(const void* xq, int K, int batch, const void* Wg, const void* Wu, int N, void* act, void* act_q8) {
+  BK_REQUIRE(xq && Wg && Wu && act_q8, "gemm_swiglu_mfma: null pointer");
+  BK_REQUIRE(K > 0 && K % 256 == 0, "gemm_swiglu_mfma: K=%d must be a positive multiple of 256", K);
+  BK_REQUIRE(N > 0 && N % 32 == 0, "gemm_swiglu_mfma: N=%d must be a positive multiple of 32", N);
+  BK_REQUIRE(batch >= 1 && batch <= 32 * 65535, "gemm_swiglu_mfma: bad batch=%d", batch);
+  BK_REQUIRE(((uintptr_t)xq & 3) == 0 && ((uintptr_t)Wg & 15) == 0 && ((uintptr_t)Wu & 15) == 0 && ((uintptr_t)act_q8 & 3) == 0,
+             "gemm_swiglu_mfma: misaligned pointer");
+  MfmaArgs A{};
+  A.xq = (const uint8_t*)xq; A.nb = K / 256; A.B = batch;
+  A.g[0].W = (const uint8_t*)Wg; A.g[0].out = act; A.g[0].N = N;
+  A.g[1].W = (const uint8_t*)Wu; A.g[1].N = N;
+  A.out_q8 = (uint8_t*)act_q8;
+  const int tiles = N / 32, btiles = (batch + 31) / 32;
+  for (int i = 0; i < 5; i++) A.tile_first[i] = i ? tiles : 0;
+  A.tiles = tiles; A.btiles = btiles;
+  const int64_t wgs = (int64_t)tiles * btiles;
+  // waves per tile as in the plain form (each workgroup holds two tiles, so at most four per tile)
+  int nw = g_tune_gemm_nw;
+  if (nw <= 0) {
+    nw = A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1);
+    if (2 * wgs >= 8 * num_cus()) nw = 1;
+  }
+  nw = nw >= 4 ? 4 : (nw >= 2 ? 2 : 1);
+  const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
+  if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, true>), grid, dim3(512), 0, stream(), A);
+  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, true>), grid, dim3(256), 0, stream(), A);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, true>), grid, dim3(128), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
 }
 
 }  // namespace bk

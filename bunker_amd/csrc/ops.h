@@ -49,6 +49,7 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
 extern int g_tune_gemm_nw;
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi);
+int launch_gemm_swiglu_mfma(const void* xq, int K, int batch, const void* Wg, const void* Wu, int N, void* act, void* act_q8);
 int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int K, int batch, int out_dtype,
                               const void* residual);
 

@@ -25,7 +25,7 @@ import numpy as np
 
 from . import runtime as rt
 from .model import Dims, L
-from .runner import DecodeEnv
+from .runner import DecodeEnv, Q8OUT_MIN_BATCH
 
 
 class _Slot:
@@ -37,7 +37,7 @@ class _Slot:
         self.buf = {name: owner._alloc(T * n * b) for name, (n, b) in {
             "x": (D.H, 2), "h": (D.H, 2), "qkv": (D.QKVD, 2), "z": (D.ZD, 2), "a": (D.LVH, 4), "b": (D.LVH, 4),
             "conv": (D.QKVD, 2), "mix": (max(D.ZD, D.NH * D.HD), 2), "qg": (D.QGATE, 2), "k": (D.KV_DIM, 2), "v": (D.KV_DIM, 2),
-            "act": (D.INTER, 2)}.items()}
+            "act": (D.INTER, 2), "act_q8": (D.INTER // 32 * 36, 1)}.items()}
         self.kernels: dict[int, dict] = {}
         self.done = [rt.Event() for _ in range(D.NL)]        # layer l's state of this slot's chunk has been written
 
@@ -102,9 +102,12 @@ class Prefill:
             "fa_in": c(f"gemv_fused K={D.H} pro=2 G=3 N0={D.QGATE} epi0=1 N1={D.KV_DIM} epi1=1 N2={D.KV_DIM} epi2=1" + bp),
             "fa": c(f"fa2_prefill HD={D.HD} NH={D.NH} NKV={D.NKV} MAX_LEN={D.MAX_LEN} ROT_HALF={D.ROT_HALF} T={T}"),
             "fa_out": c(f"gemv_fused K={D.NH * D.HD} pro=1 G=1 N0={D.H} epi0=2" + bp),
-            "mlp_in": c(f"gemv_fused K={D.H} pro=2 G=2 swiglu=1 N0={D.INTER} N1={D.INTER}" + bp),
-            "mlp_out": c(f"gemv_fused K={D.INTER} pro=1 G=1 N0={D.H} epi0=2" + bp),
         }
+        # batched form: the matmul leaves the SwiGLU result as Q8_1 blocks too and the down projection reads those
+        self_q8 = T >= Q8OUT_MIN_BATCH and D.INTER % 32 == 0
+        k["mlp_q8"] = self_q8
+        k["mlp_in"] = c(f"gemv_fused K={D.H} pro=2 G=2 swiglu=1 N0={D.INTER} N1={D.INTER}" + bp + (" q8out=1" if self_q8 else ""))
+        k["mlp_out"] = c(f"gemv_fused K={D.INTER} pro={0 if self_q8 else 1} G=1 N0={D.H} epi0=2" + bp)
         slot.kernels[T] = k
         return k
 
@@ -209,5 +212,5 @@ class Prefill:
                     self.on_attention(layer, first_index, rt.from_device(B["mix"], (T, D.NH * D.HD), np.uint16))
                 self._launch(k["fa_out"], [B["mix"], W[f"{sa}.o_proj.weight"], x, h], f"{p} o_proj")
             self._launch(k["mlp_in"], [h, W[f"{p}.post_attention_layernorm.weight"], W[f"{p}.mlp.gate_proj.weight"],
-                                       W[f"{p}.mlp.up_proj.weight"], B["act"]], f"{p} gate/up")
-            self._launch(k["mlp_out"], [B["act"], W[f"{p}.mlp.down_proj.weight"], h, x], f"{p} down")
+                                       W[f"{p}.mlp.up_proj.weight"], B["act"]] + ([B["act_q8"]] if k["mlp_q8"] else []), f"{p} gate/up")
+            self._launch(k["mlp_out"], [B["act_q8"] if k["mlp_q8"] else B["act"], W[f"{p}.mlp.down_proj.weight"], h, x], f"{p} down")

@@ -95,7 +95,8 @@ def test_gemv_fused_groups(orc, dev, K, batch, pro):
                 assert np.array_equal(got, ref), (i, b)
 
 
-@pytest.mark.parametrize("K,N,batch", [(2048, 6144, 1), (2048, 204, 3), (512, 64, 2), (2048, 128, 8), (1024, 3584, 1), (1024, 100, 2)])
+@pytest.mark.parametrize("K,N,batch", [(2048, 6144, 1), (2048, 204, 3), (512, 64, 2), (2048, 128, 8), (1024, 3584, 1), (1024, 100, 2),
+                                       (768, 96, 70), (256, 64, 33), (6144, 32, 32)])
 def test_gemv_fused_swiglu(orc, dev, K, N, batch):
     print(f"gemv_fused swiglu K={K} N={N} batch={batch}", flush=True)
     g = synth.rng(950 + N + batch)
