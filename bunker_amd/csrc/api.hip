@@ -301,7 +301,7 @@ static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
   if (rc) return rc;
   return launch_attn_decode(qn, P<void>(s[9]), P<void>(s[10]), table, 0, pos, 0, 1, max_len, P<uint16_t>(s[0]) + HD,
                             (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - (size_t)T * NH * HD * 2,
-                            T, NH, NKV, HD, 16, (int)k.get("splits", 0));
+                            T, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, k.get("pair", 0) ? 2 : 1);
 }
 
 // ---- op: argmax (src/model.ts:198-201)   slots: logits, val, idx     params: VOCAB, batch=1
@@ -378,8 +378,12 @@ static int build_kernel(Kernel& k) {
       if ((rc = need(k, p))) return rc;
     const int T = (int)k.get("T", 0), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
     BK_REQUIRE(T >= 1 && T <= 65535 && NKV >= 1 && max_len >= 1, "fa2_prefill: bad T/NKV/MAX_LEN");
+    // two consecutive tokens per workgroup where their heads fit the 16 columns of the products (pair=0 switches it off)
+    const int NHq = (int)k.get("NH", 0);
+    const int tpw = (NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
+    k.p["pair"] = tpw == 2;
     int splits = (int)k.get("splits", 0);
-    if (splits <= 0) { splits = attn_choose_splits(T, NKV, max_len); k.p["splits"] = splits; }
+    if (splits <= 0) { splits = attn_choose_splits((T + tpw - 1) / tpw, NKV, max_len); k.p["splits"] = splits; }
     const size_t qbytes = (size_t)T * k.get("NH", 0) * k.get("HD", 0) * 2;
     if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(T, NKV, splits) : 0)))) return rc;
     k.run = run_fa2_prefill; k.nslots = 12;

@@ -13,7 +13,9 @@
 //   O^T[d, head]   = sum_tok V^T[d, tok] * P^T[tok, head] v_mfma_f32_16x16x16_bf16, A = V page,
 // and P^T comes out of the first product in exactly the register layout the second
 // wants as its B operand (fed as two bf16 terms, hi + lo, so that P carries 16 bits).
-// The query heads of a KV group (<= 16) are the N dimension.
+// The query heads of a KV group (<= 16) are the N dimension; when a prompt is processed and the group has at most 8 heads,
+// two consecutive tokens of the sequence share a workgroup (columns 0..G-1 and G..2G-1, each masked to its own length),
+// so a K/V page is read once for both.
 //
 // grid = (splits, NKV, B), 4 waves per workgroup.  Each wave walks pages of its
 // split with its own running (max, sum, O^T); the four are merged through LDS in a
@@ -47,6 +49,7 @@ struct AttnArgs {
   float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
   int64_t gate_bstride, gate_hstride;
   int bt_stride, ctx_scalar, ctx_add, NH, NKV, G, splits, pages_per_split;
+  int tpw, rows;              // query rows per workgroup (1, or 2 consecutive rows of one sequence: prompt tokens), rows in all
   float scale;
 };
 
@@ -63,19 +66,27 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   __shared__ float lds_m[ATT_WAVES][16], lds_l[ATT_WAVES][16];
   __shared__ int lds_bt[ATT_MAX_PPS];           // physical page of every page of this split
 
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;     // b: workgroup's first query row is b * tpw
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, kg = lane >> 4;      // n: token (A operand) / head (B operand, C column); kg: lane group
-  const int len = (A.ctx_len ? A.ctx_len[b] : A.ctx_scalar) + A.ctx_add;
-  const int npages = (len + ATT_PAGE - 1) / ATT_PAGE;
+  // column n of the products: head n % G of query row b * tpw + n / G; a row past the last one repeats the first (not stored)
+  const int row0 = b * A.tpw;
+  const int ntk = min(A.tpw, A.rows - row0);    // query rows of this workgroup
+  const int tk_n = n / A.G;
+  const bool col_valid = tk_n < ntk;
+  const int row_n = row0 + (col_valid ? tk_n : 0);
+  const int len = (A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add;       // of this lane's column
+  int len_max = (A.ctx_len ? A.ctx_len[row0] : A.ctx_scalar) + A.ctx_add;
+  if (ntk > 1) len_max = max(len_max, A.ctx_len[row0 + 1] + A.ctx_add);
+  const int npages = (len_max + ATT_PAGE - 1) / ATT_PAGE;
   const int p_begin = split * A.pages_per_split;
   const int p_end = min(npages, p_begin + A.pages_per_split);
 
-  // Q as the B operand of the first product: lane (head n, group kg) holds dims 32*s + 8*kg .. +8
+  // Q as the B operand of the first product: lane (column n, group kg) holds dims 32*s + 8*kg .. +8
   uint4 qreg[8];
   {
-    const bool valid = n < A.G;
-    const uint16_t* qp = A.q + ((int64_t)b * A.NH + kvh * A.G + (valid ? n : 0)) * ATT_HD + 8 * kg;
+    const bool valid = col_valid;
+    const uint16_t* qp = A.q + ((int64_t)row_n * A.NH + kvh * A.G + (valid ? n % A.G : 0)) * ATT_HD + 8 * kg;
 #pragma unroll
     for (int s = 0; s < 8; s++) qreg[s] = valid ? *(const uint4*)(qp + 32 * s) : make_uint4(0, 0, 0, 0);
   }
@@ -89,7 +100,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   // The page table of the split is read once, into LDS: a table lookup in front of every page would
   // put a dependent global load (and a wait for everything in flight) between the page requests.
   for (int i = threadIdx.x; i < p_end - p_begin; i += ATT_WAVES * 64)
-    lds_bt[i] = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + p_begin + i] : b * A.bt_stride + p_begin + i;
+    lds_bt[i] = A.block_table ? A.block_table[(int64_t)row0 * A.bt_stride + p_begin + i] : row0 * A.bt_stride + p_begin + i;
   __syncthreads();
   auto load_page = [&](int pg, uint4 (&kr)[8], uint2 (&vr)[16]) {
     const int phys = lds_bt[pg - p_begin];
@@ -120,11 +131,13 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float m_new = fmaxf(m_run, tmax);        // finite: every page in range holds at least one valid token
-    const float alpha = __expf(m_run - m_new);     // exp(-inf) = 0 on the first page
+    const float m_new = fmaxf(m_run, tmax);
+    // a column whose own length ends before this page (the shorter of two rows) has seen nothing yet: keep exp() off inf - inf
+    const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float alpha = __expf(m_run - m_ref);     // exp(-inf) = 0 on the first page
     float p[4], psum = 0.0f;
 #pragma unroll
-    for (int r = 0; r < 4; r++) { p[r] = __expf(sc[r] - m_new); psum += p[r]; }
+    for (int r = 0; r < 4; r++) { p[r] = __expf(sc[r] - m_ref); psum += p[r]; }
     l_run = l_run * alpha + psum;
     m_run = m_new;
     if (alpha != 1.0f) {
@@ -210,30 +223,32 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
 
   // ---- write: thread = dim, loop over the G heads of the group
   const int d = threadIdx.x;   // 0..255
+  const int ncols = A.G * ntk;
   if (A.splits == 1) {
-    for (int h = 0; h < A.G; h++) {
-      const int head = kvh * A.G + h;
-      // M and L live in the lanes with n == h; fetch them through LDS
-      float Mh = lds_m[0][h];
-      for (int w = 1; w < ATT_WAVES; w++) Mh = fmaxf(Mh, lds_m[w][h]);
+    for (int c = 0; c < ncols; c++) {
+      const int head = kvh * A.G + c % A.G;
+      const int64_t row = row0 + c / A.G;
+      // M and L live in the lanes with n == c; fetch them through LDS
+      float Mh = lds_m[0][c];
+      for (int w = 1; w < ATT_WAVES; w++) Mh = fmaxf(Mh, lds_m[w][c]);
       float Lh = 0.0f;
       for (int w = 0; w < ATT_WAVES; w++) {
-        const float mw = lds_m[w][h];
-        Lh += (mw == -INFINITY) ? 0.0f : lds_l[w][h] * __expf(mw - Mh);
+        const float mw = lds_m[w][c];
+        Lh += (mw == -INFINITY) ? 0.0f : lds_l[w][c] * __expf(mw - Mh);
       }
-      float o = lds_o[d][h] / Lh;
+      float o = lds_o[d][c] / Lh;
       if (A.gate) {
-        const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
+        const float gv = bf16_to_f32(A.gate[row * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
         o = __fmul_rn(o, sigmoid_f64(gv));
       }
-      A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
-      if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = Mh + logf(Lh);
+      A.out[(row * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
+      if (d == 0 && A.lse) A.lse[row * A.NH + head] = Mh + logf(Lh);
     }
   } else {
     const int64_t pidx = ((int64_t)b * A.NKV + kvh) * A.splits + split;
     float* po = A.part_o + pidx * 16 * ATT_HD;
-    for (int h = 0; h < A.G; h++) po[h * ATT_HD + d] = lds_o[d][h];
-    if (kg == 0 && wave == 0 && n < A.G) {
+    for (int c = 0; c < ncols; c++) po[c * ATT_HD + d] = lds_o[d][c];
+    if (kg == 0 && wave == 0 && n < ncols) {
       A.part_ml[(pidx * 16 + n) * 2] = M;
       A.part_ml[(pidx * 16 + n) * 2 + 1] = L;
     }
@@ -246,9 +261,9 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   __shared__ float wsh[ATT_MAX_SPLITS];
   __shared__ float redm[4], redl[4];
-  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const int kvh = head / A.G, h = head % A.G;
-  const int64_t p0 = ((int64_t)b * A.NKV + kvh) * A.splits;
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;      // b: query row
+  const int kvh = head / A.G, h = (b % A.tpw) * A.G + head % A.G;     // h: the row's column in its workgroup's partials
+  const int64_t p0 = ((int64_t)(b / A.tpw) * A.NKV + kvh) * A.splits;
   const bool has = d < A.splits;
   const float ms = has ? A.part_ml[((p0 + d) * 16 + h) * 2] : -INFINITY;
   const float ls = has ? A.part_ml[((p0 + d) * 16 + h) * 2 + 1] : 0.0f;
@@ -302,7 +317,7 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8) {
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw) {
   BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
@@ -313,7 +328,11 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   BK_REQUIRE(bt_stride >= (max_ctx + ATT_PAGE - 1) / ATT_PAGE || (block_table && bt_stride == 0),
              "attn_decode: block table rows hold %d pages, context needs %d", bt_stride, (max_ctx + ATT_PAGE - 1) / ATT_PAGE);
   BK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kc & 15) == 0 && ((uintptr_t)vc & 15) == 0, "attn_decode: q, K and V must be 16-byte aligned");
-  if (splits <= 0) splits = attn_choose_splits(batch, NKV, max_ctx);
+  // tpw = 2: rows 2i and 2i+1 are consecutive tokens of one sequence (a prompt) and share a workgroup
+  BK_REQUIRE(tpw == 1 || (tpw == 2 && 2 * (NH / NKV) <= 16 && block_table && bt_stride == 0 && ctx_len),
+             "attn_decode: two rows per workgroup need a group of at most 8 heads, one shared block table and per-row lengths");
+  const int groups = (batch + tpw - 1) / tpw;
+  if (splits <= 0) splits = attn_choose_splits(groups, NKV, max_ctx);
   const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
   if (splits > pages) splits = pages;
   BK_REQUIRE(splits <= ATT_MAX_SPLITS, "attn_decode: at most %d splits", ATT_MAX_SPLITS);
@@ -325,6 +344,7 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   A.gate_bstride = gate_bstride; A.gate_hstride = gate_hstride;
   A.bt_stride = bt_stride; A.ctx_scalar = ctx_scalar; A.ctx_add = ctx_add; A.NH = NH; A.NKV = NKV; A.G = NH / NKV;
   A.splits = splits; A.pages_per_split = (pages + splits - 1) / splits;
+  A.tpw = tpw; A.rows = batch;
   A.scale = (float)(1.0 / sqrt((double)HD));
   if (splits > 1) {
     BK_REQUIRE(workspace && workspace_bytes >= attn_workspace_bytes(batch, NKV, splits),
@@ -334,9 +354,9 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   }
   // waves with three pages or more keep two pages in flight ahead of the one they work on
   if (A.pages_per_split >= 3 * ATT_WAVES)
-    hipLaunchKernelGGL(attn_decode_kernel<2>, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
+    hipLaunchKernelGGL(attn_decode_kernel<2>, dim3(splits, NKV, groups), dim3(ATT_WAVES * 64), 0, stream(), A);
   else
-    hipLaunchKernelGGL(attn_decode_kernel<0>, dim3(splits, NKV, batch), dim3(ATT_WAVES * 64), 0, stream(), A);
+    hipLaunchKernelGGL(attn_decode_kernel<0>, dim3(splits, NKV, groups), dim3(ATT_WAVES * 64), 0, stream(), A);
   if (splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, batch), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
   // a single split writes its output from the attention kernel itself; its Q8_1 copy then takes the stand-alone quantizer

@@ -70,6 +70,41 @@ def test_gdn_prefill_is_T_decode_steps(orc, Hg, T):
         rt.cuFree(p)
 
 
+@pytest.mark.parametrize("T,pos0,splits", [(6, 0, 0), (37, 12, 0), (37, 60, 3), (2, 15, 2)])
+def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits):
+    """Two consecutive tokens per workgroup (their heads side by side in the 16 columns of the products, each column
+    masked to its own length) against one token per workgroup: the same output and cache bytes."""
+    print(f"fa2_prefill pairs T={T} pos0={pos0} splits={splits}", flush=True)
+    g = synth.rng(870 + T + pos0)
+    NH, NKV, HD, HALF, MAXL = 16, 2, 256, 32, 128
+    pages = MAXL // 16
+    cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+    kc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    qgate = bf(g.standard_normal((T, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((T, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((T, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    table = g.permutation(pages).astype(np.int32)
+    pos = (pos0 + np.arange(T)).astype(np.int32)
+    ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
+    res = []
+    for pair in (0, 1):
+        dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
+        dout = rt.cuAlloc(T * NH * HD * 2)
+        rt.cuMemset(dout, 0xff, T * NH * HD * 2)
+        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} pair={pair}" + (f" splits={splits}" if splits else ""),
+                ptrs + [dkc, dvc, dout])
+        res.append((rt.from_device(dout, (T, NH, HD), np.uint16), rt.from_device(dkc, kc.shape, np.uint16),
+                    rt.from_device(dvc, (pages, NKV, HD, 16), np.uint16)))
+        for p in (dkc, dvc, dout):
+            rt.cuFree(p)
+    for a, b in zip(res[0], res[1]):
+        assert np.array_equal(a, b)
+    assert not np.any(res[1][0] == 0xffff)
+    for p in ptrs:
+        rt.cuFree(p)
+
+
 @pytest.mark.parametrize("T,pos0", [(1, 0), (5, 0), (37, 12)])
 def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0):
     print(f"fa2_prefill T={T} pos0={pos0}", flush=True)
