@@ -276,63 +276,72 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] += part[r * 64 + (lane ^ (r + 16 * half))];
 
-  auto store = [&](int n_in_tile, int b, double total) {
-    const int n = n0 + n_in_tile;
-    if (n >= N || b >= B) return;
-    const int64_t o = (int64_t)(b0 + b) * N + n;
-    const float v = (float)total;
-    if (EPI == GEPI_F32) ((float*)out)[o] = v;
-    else if (EPI == GEPI_BF16) ((uint16_t*)out)[o] = f32_to_bf16(v);
-    else ((uint16_t*)out)[o] = f32_to_bf16(bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(res[o]));
-  };
-  if (SWIGLU) {
-    // both tiles' partials meet in LDS; thread (wave w, lane) then takes output column lane % 32 and batch rows
-    // 2 (w R + i) + lane / 32: g and u are added in wave order and rounded to f32 like the matmul's own outputs, the
-    // 32 lanes of a half hold one Q8_1 block of the activation
-    __builtin_amdgcn_wave_barrier();       // slot (r, lane) was read above by this lane only
+  // Last step: every wave leaves its 16 partial sums per lane in LDS; the threads then finish the outputs with the
+  // weight row along the lanes (contiguous stores): thread (wave w, lane) takes row lane % 32 and batch rows
+  // 2 (w R + i) + lane / 32, and adds the waves' partials in wave order.
+  __builtin_amdgcn_wave_barrier();         // slot (r, lane) was read above by this lane only
 #pragma unroll
-    for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
-    __syncthreads();
-    const double* all = (const double*)lds_raw;
-    constexpr int R = 16 / WAVES;
-    const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
+  for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
+  __syncthreads();
+  const double* all = (const double*)lds_raw;
+  constexpr int R = 16 / WAVES;
+  const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
+  float y[SWIGLU ? 1 : R], u_[SWIGLU ? R : 1], g_[SWIGLU ? R : 1];
+#pragma unroll
+  for (int i = 0; i < R; i++) {
+    const int b = 2 * (wave * R + i) + half;
+    const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
+    if (SWIGLU) {
+      double gd = all[slot], ud = all[NW * 16 * 64 + slot];
+#pragma unroll
+      for (int w = 1; w < NW; w++) { gd += all[w * 16 * 64 + slot]; ud += all[(NW + w) * 16 * 64 + slot]; }
+      g_[i] = (float)gd; u_[i] = (float)ud;
+    } else {
+      double t = all[slot];
+#pragma unroll
+      for (int w = 1; w < NW; w++) t += all[w * 16 * 64 + slot];
+      y[i] = (float)t;
+    }
+  }
+  if (SWIGLU) {
+    // g and u were rounded to f32 like the matmul's own outputs; the 32 lanes of a half hold one Q8_1 block of the activation
     uint16_t* act = (uint16_t*)A.g[0].out;
 #pragma unroll
     for (int i = 0; i < R; i++) {
       const int b = 2 * (wave * R + i) + half;
-      const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
-      double gd = all[slot], ud = all[NW * 16 * 64 + slot];
-#pragma unroll
-      for (int w = 1; w < NW; w++) { gd += all[w * 16 * 64 + slot]; ud += all[(NW + w) * 16 * 64 + slot]; }
-      const float g = (float)gd, u = (float)ud;
-      const uint16_t a16 = f32_to_bf16(__fmul_rn(__fmul_rn(g, sigmoid_f64(g)), u));
+      const uint16_t a16 = f32_to_bf16(__fmul_rn(__fmul_rn(g_[i], sigmoid_f64(g_[i])), u_[i]));
       const bool valid = b < B;
       if (valid && act) act[(int64_t)(b0 + b) * N + n0 + col] = a16;
       lane32_q8_1_store(bf16_to_f32(a16), A.out_q8 + ((int64_t)(b0 + b) * (N / 32) + (n0 >> 5)) * 36, col, valid);
     }
-  } else if (NW > 1) {
-    // every wave leaves its 16 partial sums per lane in LDS; then the threads finish the outputs with the weight row
-    // along the lanes (contiguous stores): thread (wave w, lane) takes row lane % 32 and batch rows 2 (w R + i) + lane / 32;
-    // the partials are added in wave order
-    __builtin_amdgcn_wave_barrier();       // slot (r, lane) was read above by this lane only
-#pragma unroll
-    for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
-    __syncthreads();
-    const double* all = (const double*)lds_raw;
-    constexpr int R = 16 / NW;
-    const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
+    return;
+  }
+  const bool n_ok = n0 + col < N;
+  const int64_t o0 = (int64_t)b0 * N + n0 + col;
+  if (EPI == GEPI_F32) {
 #pragma unroll
     for (int i = 0; i < R; i++) {
       const int b = 2 * (wave * R + i) + half;
-      const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
-      double t = all[slot];
+      if (n_ok && b < B) ((float*)out)[o0 + (int64_t)b * N] = y[i];
+    }
+  } else if (EPI == GEPI_BF16) {
 #pragma unroll
-      for (int w = 1; w < NW; w++) t += all[w * 16 * 64 + slot];
-      store(col, b, t);
+    for (int i = 0; i < R; i++) {
+      const int b = 2 * (wave * R + i) + half;
+      if (n_ok && b < B) ((uint16_t*)out)[o0 + (int64_t)b * N] = f32_to_bf16(y[i]);
     }
   } else {
+    uint16_t rv[R];
 #pragma unroll
-    for (int r = 0; r < 16; r++) store(mfma32_row(r, half), col, acc[r]);
+    for (int i = 0; i < R; i++) {
+      const int b = 2 * (wave * R + i) + half;
+      rv[i] = (n_ok && b < B) ? res[o0 + (int64_t)b * N] : (uint16_t)0;
+    }
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+      const int b = 2 * (wave * R + i) + half;
+      if (n_ok && b < B) ((uint16_t*)out)[o0 + (int64_t)b * N] = f32_to_bf16(bf16_to_f32(f32_to_bf16(y[i])) + bf16_to_f32(rv[i]));
+    }
   }
 }
 
