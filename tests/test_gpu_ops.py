@@ -330,3 +330,26 @@ def test_fa2_attn_op_appends_and_attends(orc, dev, batch):
     kc_d = rt.from_device(dkc, kc.shape, np.uint16)
     vc_d = rt.from_device(dvc, (batch * ppseq, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
     assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
+
+
+def test_streams_order_work_through_events(orc, dev):
+    """A second stream: work queued there runs behind an event of the first stream, results are visible after cuSync,
+    and a handle that is not a stream of the library is refused."""
+    n = 1 << 20
+    a = np.arange(n, dtype=np.float32)
+    da, db, dc = dev.up(a), dev.empty(n * 4), dev.empty(n * 4)
+    st = rt.Stream()
+    rt.cuDtoD(db, da, n * 4)                       # first stream: b = a
+    ev = rt.Event().record()
+    st.wait(ev)
+    with st:
+        rt.cuDtoD(dc, db, n * 4)                   # second stream, behind the event: c = b
+        with st:                                   # nesting keeps the selection
+            pass
+        done = rt.Event().record()
+    rt.streamWaitEvent(done)                       # first stream waits for the second
+    rt.cuSync()
+    assert np.array_equal(rt.from_device(dc, (n,), np.float32), a)
+    with pytest.raises(rt.BunkerError, match="not a stream"):
+        rt._check(rt.cu().bk_stream_use(12345), "bk_stream_use")
+    st.destroy(); ev.destroy(); done.destroy()
