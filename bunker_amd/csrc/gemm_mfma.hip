@@ -374,7 +374,8 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   int nw = g_tune_gemm_nw;
   if (nw <= 0) {
     nw = A.nb >= 16 ? 8 : (A.nb >= 4 ? 4 : (A.nb >= 2 ? 2 : 1));
-    if (wgs <= num_cus() + num_cus() / 4 && A.nb >= 8) nw = 8;          // about a tile per CU: one super-block per wave
+    if (wgs <= num_cus() && A.nb >= 8) nw = 8;                            // at most a tile per CU: one super-block per wave
+    if (wgs > num_cus() && nw == 8) nw = 4;     // eight waves' LDS leaves room for one workgroup per CU: no second round for a few tiles
     if (wgs >= 8 * num_cus()) nw = 1;                                     // the tiles alone fill the chip many times over
   }
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
