@@ -277,6 +277,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   if ((d & 63) == 0) redl[d >> 6] = L;
   __syncthreads();
   L = (redl[0] + redl[1]) + (redl[2] + redl[3]);
+  // the output gate does not depend on the partials: requested and evaluated ahead of them
+  const float gsig = A.gate ? sigmoid_f64(bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d])) : 1.0f;
   const float* po = A.part_o + (p0 * 16 + h) * ATT_HD + d;
   float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
   int s = 0;
@@ -288,10 +290,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   }
   for (; s < A.splits; s++) o0 = fmaf(po[(int64_t)s * 16 * ATT_HD], wsh[s], o0);
   float o = ((o0 + o1) + (o2 + o3)) / L;
-  if (A.gate) {
-    const float gv = bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
-    o = __fmul_rn(o, sigmoid_f64(gv));
-  }
+  if (A.gate) o = __fmul_rn(o, gsig);
   const uint16_t ob = f32_to_bf16(o);
   A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = ob;
   if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (((int64_t)b * A.NH + head) * (ATT_HD / 32) + (d >> 5)) * 36, d & 31);

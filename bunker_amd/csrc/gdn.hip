@@ -124,7 +124,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
 #pragma unroll
   for (int r = 0; r < ROWS; r++) S[r] = *(const float4*)(Sp + (int64_t)(kg * ROWS + r) * GDN_D + col0);
 
-  float decay, beta;
+  float decay, beta, zs = 0.0f;     // zs: the output gate z * sigmoid(z), evaluated while S is still on its way
   if (FUSED) {
     float x;
     if (CONV) {
@@ -144,6 +144,7 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
     const float softplus = (float)log1p(exp((double)sp_in));
     decay = (float)exp(-(double)((float)exp((double)alog) * softplus));
     beta = sigmoid_f64(bp);
+    zs = zin * sigmoid_f64(zin);
   } else {
     if (tid < 128) qn[tid] = bf16_to_f32(xbits);
     else kn[tid - 128] = bf16_to_f32(xbits);
@@ -213,7 +214,6 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   __syncthreads();
   if (tid < GDN_D) {
     const float orstd = rsqrt_f64((red[0] + red[1]) / (double)GDN_D + 1e-6);
-    const float zs = zin * sigmoid_f64(zin);
     const uint16_t ob = f32_to_bf16(((o * orstd) * nw) * zs);
     outp[tid] = ob;
     if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (bh * (GDN_D / 32) + (tid >> 5)) * 36, tid & 31);
