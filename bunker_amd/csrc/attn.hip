@@ -34,6 +34,8 @@ constexpr int ATT_MAX_SPLITS = 256;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_nt;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_nt;
 
 struct AttnArgs {
   const uint16_t* q;          // bf16 [B, NH, 256]
@@ -60,7 +62,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 // PF = pages a wave requests ahead of the one it computes on (0 or 2).  Loads are issued
 // unconditionally (past its last page a wave re-requests that page), so the number of loads in
 // flight at every wait is known when the kernel is compiled and a wait covers only the page needed.
-template <int PF>
+template <int PF, bool NT>
 __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A) {
   __shared__ float lds_o2[2][ATT_HD][16];       // exchange buffers for the merge of the four waves, 2 x 16 KiB
   __shared__ float lds_m[ATT_WAVES][16], lds_l[ATT_WAVES][16];
@@ -108,11 +110,19 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
     // K page as the A operand: lane (token n, group kg) holds dims 32*s + 8*kg .. +8
     const uint16_t* kp = A.kc + base + n * ATT_HD + 8 * kg;
 #pragma unroll
-    for (int s = 0; s < 8; s++) kr[s] = *(const uint4*)(kp + 32 * s);
+    for (int s = 0; s < 8; s++) {
+      const u32x4_nt* p4 = (const u32x4_nt*)(kp + 32 * s);
+      const u32x4_nt t4 = NT ? __builtin_nontemporal_load(p4) : *p4;
+      kr[s] = make_uint4(t4[0], t4[1], t4[2], t4[3]);
+    }
     // V page as the A operand: lane (dim 16*t + n, group kg) holds tokens 4*kg .. +4
     const uint16_t* vp = A.vc + base + n * ATT_PAGE + 4 * kg;
 #pragma unroll
-    for (int t = 0; t < 16; t++) vr[t] = *(const uint2*)(vp + t * 16 * ATT_PAGE);
+    for (int t = 0; t < 16; t++) {
+      const u32x2_nt* p2 = (const u32x2_nt*)(vp + t * 16 * ATT_PAGE);
+      const u32x2_nt t2 = NT ? __builtin_nontemporal_load(p2) : *p2;
+      vr[t] = make_uint2(t2[0], t2[1]);
+    }
   };
   auto compute_page = [&](const uint4 (&kreg)[8], const uint2 (&vreg)[16], int pg) {
     f32x4_t s4 = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -297,6 +307,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = M + logf(L);
 }
 
+int g_tune_attn_nt = -1;   // K/V pages through nontemporal loads: 0 off, 1 on, -1 = from the size of the read
+
 size_t attn_workspace_bytes(int batch, int NKV, int max_splits) {
   return (size_t)batch * NKV * max_splits * 16 * (ATT_HD + 2) * sizeof(float);
 }
@@ -352,10 +364,18 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
     A.part_ml = A.part_o + (size_t)batch * NKV * splits * 16 * ATT_HD;
   }
   // waves with three pages or more keep two pages in flight ahead of the one they work on
-  if (A.pages_per_split >= 3 * ATT_WAVES)
-    hipLaunchKernelGGL(attn_decode_kernel<2>, dim3(splits, NKV, groups), dim3(ATT_WAVES * 64), 0, stream(), A);
-  else
-    hipLaunchKernelGGL(attn_decode_kernel<0>, dim3(splits, NKV, groups), dim3(ATT_WAVES * 64), 0, stream(), A);
+  // A cache read that is larger than what the memory-side cache can still hold when the next token comes round (decode
+  // at large batch x context) bypasses the caches; prompt rows re-read the same pages and keep the plain loads.
+  const bool nt = g_tune_attn_nt >= 0 ? g_tune_attn_nt != 0
+                                      : (tpw == 1 && (int64_t)batch * NKV * max_ctx * ATT_HD * 4 >= ((int64_t)128 << 20));
+  const dim3 grid(splits, NKV, groups), block(ATT_WAVES * 64);
+  if (A.pages_per_split >= 3 * ATT_WAVES) {
+    if (nt) hipLaunchKernelGGL((attn_decode_kernel<2, true>), grid, block, 0, stream(), A);
+    else hipLaunchKernelGGL((attn_decode_kernel<2, false>), grid, block, 0, stream(), A);
+  } else {
+    if (nt) hipLaunchKernelGGL((attn_decode_kernel<0, true>), grid, block, 0, stream(), A);
+    else hipLaunchKernelGGL((attn_decode_kernel<0, false>), grid, block, 0, stream(), A);
+  }
   if (splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, batch), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
   // a single split writes its output from the attention kernel itself; its Q8_1 copy then takes the stand-alone quantizer
