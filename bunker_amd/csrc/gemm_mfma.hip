@@ -55,9 +55,15 @@ enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 *
 
 // SWIGLU: the workgroup holds 2 NW waves; waves 0..NW-1 form the tile of 32 gate rows, waves NW..2NW-1 the tile of the
 // same 32 up rows, and the last step writes act = bf16(silu(g) * u) and its Q8_1 block instead of g and u.
-template <int NW, bool SWIGLU>
+// R16: the tile has 16 weight rows (rows 16..31 of the matrix instruction repeat them and are ignored), for launches with
+// so few tiles that the time is the length of one wave's instruction stream: half the fold per super-block, twice the tiles.
+template <int NW, bool SWIGLU, bool R16 = false>
 __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
+  static_assert(!(SWIGLU && R16), "the SwiGLU form quantizes 32 outputs at a time");
   constexpr int WAVES = NW * (SWIGLU ? 2 : 1);
+  constexpr int TR = R16 ? 16 : 32;        // weight rows of the tile
+  constexpr int RF = TR / 2;               // of them per lane
+  constexpr int TN = TR / 16;              // 16-row groups (min term)
   // Per wave: the activation rows of the current super-block as they lie in memory (288 bytes, rows 292 apart so that
   // the lanes of a read fall into different banks), the weight rows (144 bytes each), and 512 bytes of weight scales
   // in the order the fold reads them (the 6-bit scales as bytes [8 sub-blocks][2 halves][16 rows], then d as doubles
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   const uint8_t* __restrict__ xq = A.xq + (int64_t)b0 * xrow_bytes;
 
   const int half = lane >> 5, col = lane & 31, q4 = lane >> 4, l16 = lane & 15;
-  const int n0 = (tile - (s3 ? A.tile_first[3] : s2 ? A.tile_first[2] : s1 ? A.tile_first[1] : 0)) * 32;
+  const int n0 = (tile - (s3 ? A.tile_first[3] : s2 ? A.tile_first[2] : s1 ? A.tile_first[1] : 0)) * TR;
   unsigned char* const ldsX = lds_raw + wave * G_WAVE_LDS;
   unsigned char* const ldsW = ldsX + GX_BYTES;
   unsigned char* const stage = ldsW + GW_BYTES;
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   uint32_t woff[5];
 #pragma unroll
   for (int i = 0; i < 5; i++) {
-    const int p = min(lane + 64 * i, 287), row = p / 9;
+    const int p = min(lane + 64 * i, TR * 9 - 1), row = p / 9;
     woff[i] = (uint32_t)((min(n0 + row, N - 1) - n0) * (int)wrow_bytes + (p - 9 * row) * 16);
   }
   uint4 xr[10], wr0, wr1, wr2, wr3, wr4;
@@ -122,21 +128,24 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     wr0 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[0]);                                                       \
     wr1 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[1]);                                                       \
     wr2 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[2]);                                                       \
-    wr3 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[3]);                                                       \
-    wr4 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[4]);                                                       \
+    if (!R16) {                                                                                                        \
+      wr3 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[3]);                                                     \
+      wr4 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[4]);                                                     \
+    }                                                                                                                  \
   }
 
   // where the lane's own weight row sits among the rows of its half: row = 8g + 4h + v  ->  [h][4g + v]
-  const int stage_slot = ((col >> 2) & 1) * 16 + 4 * (col >> 3) + (col & 3);
-  const unsigned char* const myW = ldsW + col * GW_ROW;         // int8 operands: weight row col, batch row col,
+  const int wcol = col & (TR - 1);
+  const int stage_slot = ((wcol >> 2) & 1) * 16 + 4 * (wcol >> 3) + (wcol & 3);
+  const unsigned char* const myW = ldsW + wcol * GW_ROW;        // int8 operands: weight row col, batch row col,
   const unsigned char* const myX = ldsX + col * GX_ROW;         // bytes 16*half.. of every sub-block
 
-  double acc[16];
+  double acc[RF];
 #pragma unroll
-  for (int r = 0; r < 16; r++) acc[r] = 0.0;
-  f64x4_t accm[2][2];
+  for (int r = 0; r < RF; r++) acc[r] = 0.0;
+  f64x4_t accm[TN][2];
 #pragma unroll
-  for (int t = 0; t < 4; t++) accm[t >> 1][t & 1] = (f64x4_t){0.0, 0.0, 0.0, 0.0};
+  for (int t = 0; t < 2 * TN; t++) accm[t >> 1][t & 1] = (f64x4_t){0.0, 0.0, 0.0, 0.0};
 
   GM_FETCH(min(kw, nb - 1));            // requests are unconditional (clamped): the waits stay countable
   for (int blk = kw; blk < nb; blk += NW) {
@@ -149,9 +158,13 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     }
     *(uint4*)(ldsW + lane * 16) = wr0;
     *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
-    *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
-    *(uint4*)(ldsW + (lane + 192) * 16) = wr3;
-    if (lane < 32) *(uint4*)(ldsW + (lane + 256) * 16) = wr4;
+    if (R16) {
+      if (lane < 16) *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
+    } else {
+      *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
+      *(uint4*)(ldsW + (lane + 192) * 16) = wr3;
+      if (lane < 32) *(uint4*)(ldsW + (lane + 256) * 16) = wr4;
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -191,7 +204,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     // its product with d8_j (11 bits) is exact inside the FMA, and so is d (11 bits) times the sum over the eight
     // sub-blocks as long as that sum has not been rounded (the terms of one activation row lie within a few binades of
     // each other).
-    double S1[16];
+    double S1[RF];
     uint4 q = *(const uint4*)(myW + 16 + 16 * half), qn = q;
     uint4 scb = *(const uint4*)(stage + 16 * half), scn = scb;
     uint32_t dsw = *(const uint32_t*)(myX + 32), dsn = dsw;
@@ -209,7 +222,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
       const double d8 = (double)half_to_f32((uint16_t)(dsw & 0xffffu));
       const uint32_t scv[4] = {scb.x, scb.y, scb.z, scb.w};
 #pragma unroll
-      for (int r = 0; r < 8; r++) {
+      for (int r = 0; r < RF / 2; r++) {
         const double t = (double)__mul24(c[r], (int)((scv[r >> 2] >> (8 * (r & 3))) & 0xffu));
         S1[r] = j == 0 ? d8 * t : fma(d8, t, S1[r]);
       }
@@ -220,7 +233,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int r = 8; r < 16; r++) {
+      for (int r = RF / 2; r < RF; r++) {
         const double t = (double)__mul24(c[r], (int)((scv[r >> 2] >> (8 * (r & 3))) & 0xffu));
         S1[r] = j == 0 ? d8 * t : fma(d8, t, S1[r]);
       }
@@ -230,7 +243,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     {
       const double2* dd = (const double2*)(stage + 256 + 128 * half);
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
+      for (int r = 0; r < RF; r += 2) {
         const double2 v = dd[r >> 1];
         acc[r] = fma(v.x, S1[r], acc[r]);
         acc[r + 1] = fma(v.y, S1[r + 1], acc[r + 1]);
@@ -238,14 +251,16 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     }
     // min term: accm[tn][tb] += (-dmin * m_j)[16 rows x 4 sub-blocks] . s8_j[4 sub-blocks x 16 batch rows], for the
     // sub-blocks 0..3 and then 4..7; a lane supplies row 16 t + l16 of either side at sub-blocks q4 and 4 + q4
-    double am[2][2], bm[2][2];
+    double am[TN][2], bm[2][2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-      const uint4 hm = *(const uint4*)(ldsW + (16 * t + l16) * GW_ROW);
-      const float dmin_neg = -half_to_f32((uint16_t)(hm.x >> 16));
-      const uint32_t zb = (hm.z >> (8 * q4)) & 0xffu, wb = (hm.w >> (8 * q4)) & 0xffu;
-      am[t][0] = (double)(dmin_neg * (float)(zb & 63u));
-      am[t][1] = (double)(dmin_neg * (float)((wb >> 4) | ((zb >> 6) << 4)));
+      if (t < TN) {
+        const uint4 hm = *(const uint4*)(ldsW + (16 * t + l16) * GW_ROW);
+        const float dmin_neg = -half_to_f32((uint16_t)(hm.x >> 16));
+        const uint32_t zb = (hm.z >> (8 * q4)) & 0xffu, wb = (hm.w >> (8 * q4)) & 0xffu;
+        am[t][0] = (double)(dmin_neg * (float)(zb & 63u));
+        am[t][1] = (double)(dmin_neg * (float)((wb >> 4) | ((zb >> 6) << 4)));
+      }
       const unsigned char* xs = ldsX + (16 * t + l16) * GX_ROW + q4 * 36 + 34;
       bm[t][0] = (double)half_to_f32(*(const uint16_t*)xs);
       bm[t][1] = (double)half_to_f32(*(const uint16_t*)(xs + 144));
@@ -253,7 +268,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 #pragma unroll
     for (int k = 0; k < 2; k++)
 #pragma unroll
-      for (int t = 0; t < 4; t++)
+      for (int t = 0; t < 2 * TN; t++)
         accm[t >> 1][t & 1] = __builtin_amdgcn_mfma_f64_16x16x4f64(am[t >> 1][k], bm[t & 1][k], accm[t >> 1][t & 1], 0, 0, 0);
   }
 
@@ -263,7 +278,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   double* part = (double*)lds_raw + wave * 16 * 64;
   __syncthreads();                         // all waves are done with the scales that share the buffer
 #pragma unroll
-  for (int t = 0; t < 4; t++)
+  for (int t = 0; t < 2 * TN; t++)
 #pragma unroll
     for (int v = 0; v < 4; v++) {
       const int n = 16 * (t >> 1) + 4 * v + q4, b = 16 * (t & 1) + l16;
@@ -274,22 +289,26 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-  for (int r = 0; r < 16; r++) acc[r] += part[r * 64 + (lane ^ (r + 16 * half))];
+  for (int r = 0; r < RF; r++) acc[r] += part[r * 64 + (lane ^ (r + 16 * half))];
 
   // Last step: every wave leaves its 16 partial sums per lane in LDS; the threads then finish the outputs with the
   // weight row along the lanes (contiguous stores): thread (wave w, lane) takes row lane % 32 and batch rows
   // 2 (w R + i) + lane / 32, and adds the waves' partials in wave order.
   __builtin_amdgcn_wave_barrier();         // slot (r, lane) was read above by this lane only
 #pragma unroll
-  for (int r = 0; r < 16; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
+  for (int r = 0; r < RF; r++) part[r * 64 + (lane ^ (r + 16 * half))] = acc[r];
   __syncthreads();
   const double* all = (const double*)lds_raw;
-  constexpr int R = 16 / WAVES;
-  const int rr = 4 * (col >> 3) + (col & 3), hh = (col >> 2) & 1;
+  // the thread's output row fn of the tile and its batch rows fb0 + FB * (wave R + i): 32 rows -> (lane % 32, lane / 32),
+  // 16 rows -> (lane % 16, lane / 16)
+  constexpr int R = TR / 2 / WAVES > 0 ? TR / 2 / WAVES : 1, FB = 64 / TR;
+  if (wave * R * FB >= 32) return;         // (eight waves on a 16-row tile: R = 1 and all of them have a batch row)
+  const int fn = lane & (TR - 1), fb0 = lane / TR;
+  const int rr = 4 * (fn >> 3) + (fn & 3), hh = (fn >> 2) & 1;
   float y[SWIGLU ? 1 : R], u_[SWIGLU ? R : 1], g_[SWIGLU ? R : 1];
 #pragma unroll
   for (int i = 0; i < R; i++) {
-    const int b = 2 * (wave * R + i) + half;
+    const int b = FB * (wave * R + i) + fb0;
     const int slot = rr * 64 + ((b + 32 * hh) ^ (rr + 16 * hh));
     if (SWIGLU) {
       double gd = all[slot], ud = all[NW * 16 * 64 + slot];
@@ -308,7 +327,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     uint16_t* act = (uint16_t*)A.g[0].out;
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      const int b = 2 * (wave * R + i) + half;
+      const int b = FB * (wave * R + i) + fb0;
       const uint16_t a16 = f32_to_bf16(__fmul_rn(__fmul_rn(g_[i], sigmoid_f64(g_[i])), u_[i]));
       const bool valid = b < B;
       if (valid && act) act[(int64_t)(b0 + b) * N + n0 + col] = a16;
@@ -316,30 +335,30 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     }
     return;
   }
-  const bool n_ok = n0 + col < N;
-  const int64_t o0 = (int64_t)b0 * N + n0 + col;
+  const bool n_ok = n0 + fn < N;
+  const int64_t o0 = (int64_t)b0 * N + n0 + fn;
   if (EPI == GEPI_F32) {
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      const int b = 2 * (wave * R + i) + half;
+      const int b = FB * (wave * R + i) + fb0;
       if (n_ok && b < B) ((float*)out)[o0 + (int64_t)b * N] = y[i];
     }
   } else if (EPI == GEPI_BF16) {
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      const int b = 2 * (wave * R + i) + half;
+      const int b = FB * (wave * R + i) + fb0;
       if (n_ok && b < B) ((uint16_t*)out)[o0 + (int64_t)b * N] = f32_to_bf16(y[i]);
     }
   } else {
     uint16_t rv[R];
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      const int b = 2 * (wave * R + i) + half;
+      const int b = FB * (wave * R + i) + fb0;
       rv[i] = (n_ok && b < B) ? res[o0 + (int64_t)b * N] : (uint16_t)0;
     }
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      const int b = 2 * (wave * R + i) + half;
+      const int b = FB * (wave * R + i) + fb0;
       if (n_ok && b < B) ((uint16_t*)out)[o0 + (int64_t)b * N] = f32_to_bf16(bf16_to_f32(f32_to_bf16(y[i])) + bf16_to_f32(rv[i]));
     }
   }
@@ -348,6 +367,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 #undef GM_FETCH
 
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
+int g_tune_gemm_r16 = -1;    // tiles of 16 weight rows: 0 off, 1 on (single batch tile only), -1 = from the shape
 
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi) {
@@ -366,6 +386,13 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
     A.tile_first[i] = tiles;
     tiles += (N[i] + 31) / 32;
   }
+  // One batch tile and so few weight tiles that half the CUs would stay empty: tiles of 16 weight rows (twice as many
+  // workgroups, half the fold per wave).  Measured on the 64-tile shapes at batch 32.
+  const bool r16 = batch <= 32 && (g_tune_gemm_r16 >= 0 ? g_tune_gemm_r16 != 0 : (2 * tiles <= num_cus() && A.nb >= 4));
+  if (r16) {
+    tiles = 0;
+    for (int i = 0; i < ngroups; i++) { A.tile_first[i] = tiles; tiles += (N[i] + 15) / 16; }
+  }
   for (int i = ngroups; i < 5; i++) A.tile_first[i] = tiles;
   // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
   // and not at all when the tiles alone fill the chip many times over (lm_head, prompt batches)
@@ -381,7 +408,10 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
   A.tiles = tiles; A.btiles = btiles;
   const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
-  if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false>), grid, dim3(512), 0, stream(), A);
+  if (r16 && btiles == 1) {
+    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, true>), grid, dim3(512), 0, stream(), A);
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, true>), grid, dim3(256), 0, stream(), A);
+  } else if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false>), grid, dim3(512), 0, stream(), A);
   else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false>), grid, dim3(256), 0, stream(), A);
   else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, false>), grid, dim3(128), 0, stream(), A);
   else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, false>), grid, dim3(64), 0, stream(), A);

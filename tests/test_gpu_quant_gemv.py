@@ -296,7 +296,7 @@ def test_gemm_mfma_equals_gemv_and_oracle(orc, dev, N, K, B):
     assert np.array_equal(ya, orc.add_bf16(synth.f32_to_bf16(y).ravel(), res.ravel()).reshape(B, N))
 
 
-@pytest.mark.parametrize("N,K,B", [(200, 2048, 70), (96, 1280, 32)])
+@pytest.mark.parametrize("N,K,B", [(200, 2048, 70), (96, 1280, 32), (41, 3072, 19)])
 def test_gemm_mfma_every_split_of_k_returns_the_same_bits(orc, dev, N, K, B):
     """1, 2, 4 or 8 wavefronts per tile (K split by super-block, partials joined in wave order): same bits as the host loop."""
     print(f"gemm mfma splits N={N} K={K} B={B}", flush=True)
@@ -307,11 +307,14 @@ def test_gemm_mfma_every_split_of_k_returns_the_same_bits(orc, dev, N, K, B):
     ref = np.stack([orc.gemv_q4k_q8_1(W, xq[b], N, K) for b in range(B)])
     dW, dxq, dy = dev.up(W), dev.up(xq), dev.empty(B * N * 4)
     try:
-        for nw in (1, 2, 4, 8):
-            rt.tune_set("gemm_nw", nw)
-            rt.cuMemset(dy, 0xff, B * N * 4)
-            rt.gemm_q4k_q8_1(dW, dxq, dy, N, K, B)
-            y = rt.from_device(dy, (B, N), np.float32)
-            assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (nw, int((y != ref).sum()))
+        for r16 in (0, 1):                     # tiles of 32 or of 16 weight rows (the latter for a single batch tile only)
+            rt.tune_set("gemm_r16", r16)
+            for nw in (1, 2, 4, 8):
+                rt.tune_set("gemm_nw", nw)
+                rt.cuMemset(dy, 0xff, B * N * 4)
+                rt.gemm_q4k_q8_1(dW, dxq, dy, N, K, B)
+                y = rt.from_device(dy, (B, N), np.float32)
+                assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (r16, nw, int((y != ref).sum()))
     finally:
         rt.tune_set("gemm_nw", 0)
+        rt.tune_set("gemm_r16", -1)
