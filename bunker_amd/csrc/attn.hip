@@ -216,16 +216,21 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
 #pragma unroll
       for (int r = 0; r < 4; r++) lds_o2[buf][16 * t + 4 * kg + r][n] = oacc[t][r];
   };
+  // between waves a lane hands its accumulators to the same lane of the other wave: 16-byte pieces in lane order
+  // (the [dim][head] layout above is only needed for the write below)
+  f32x4_t (*xch)[16][64] = (f32x4_t (*)[16][64])lds_o2;
+  auto hand = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < 16; t++) xch[buf][t][lane] = oacc[t];
+  };
   auto add = [&](int buf) {
 #pragma unroll
-    for (int t = 0; t < 16; t++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) oacc[t][r] += lds_o2[buf][16 * t + 4 * kg + r][n];
+    for (int t = 0; t < 16; t++) oacc[t] += xch[buf][t][lane];
   };
-  if (wave & 1) put(wave >> 1);           // waves 1 and 3 hand over
+  if (wave & 1) hand(wave >> 1);          // waves 1 and 3 hand over
   __syncthreads();
   if (!(wave & 1)) add(wave >> 1);        // 0 += 1 (buffer 0), 2 += 3 (buffer 1)
-  if (wave == 2) put(1);                  // buffer 1 was read by wave 2 alone, so it can take the sum straight away
+  if (wave == 2) hand(1);                 // buffer 1 was read by wave 2 alone, so it can take the sum straight away
   __syncthreads();
   if (wave == 0) { add(1); put(0); }      // (0 + 1) + (2 + 3), then out for the transposed write (buffer 0: wave 0 was its only reader)
   __syncthreads();
