@@ -80,7 +80,10 @@ BK_API int bk_capture_end(uint64_t* graph);
 BK_API int bk_graph_launch(uint64_t graph);
 BK_API int bk_graph_destroy(uint64_t graph);
 
-/* Launch-shape knobs for experiments ("gemv_rpi", "gemv_cap"); defaults are the tuned values. */
+/* Launch-shape knobs for experiments and tests; the defaults (0, or -1 = chosen from the shape) are the tuned values:
+ * "gemv_rpi", "gemv_cap", "gemv_impl", "fused_cap" (GEMV rows per wave step, workgroups per CU, kernel variant),
+ * "gemm_nw" (waves per matmul tile: 1, 2, 4, 8), "gemm_r16" (tiles of 16 weight rows), "gdn_cs" (column slabs of the
+ * GDN core op), "gdn_nt" / "attn_nt" (state / cache pages through nontemporal accesses).  No counterpart in the reference. */
 BK_API int bk_tune_set(const char* key, int value);
 
 /* ---- per-op launch surface: replaces compileAndLoad + cuLaunch
