@@ -1,4 +1,4 @@
-// Batched decode matmul: C[B, N] = Xq[B, K] . W[N, K]^T for B <= 32 activation rows in
+// Batched decode matmul: C[B, N] = Xq[B, K] . W[N, K]^T for tiles of up to 32 activation rows in
 // Q8_1 and W in Q4_K, on the int8 matrix cores.  Precedent in the reference:
 // int8MatmulTTIR (src/kernel.ts:397-417), i8 x i8 -> i32 exact, and its documented
 // post-scale (experiments/q4k_q81_final.ts:214-217).
@@ -16,7 +16,7 @@
 // the sub-blocks of K and runs on the double-precision matrix instruction (v_mfma_f64_16x16x4_f64), in its own
 // accumulators that join the others once, at the end.
 //
-// Batches of more than 32 rows are cut into 32-row tiles along blockIdx.y (one launch, every tile its own workgroup).
+// Batches of more than 32 rows are cut into 32-row tiles (one launch, every (weight tile, batch tile) its own workgroup).
 // A workgroup owns one 32 x 32 output tile; its NW wavefronts split K by super-block (wave w takes
 // blocks w, w + NW, ...) and add their double partials in wave order through LDS at the end.
 // Each wave copies the 32 x 144 weight bytes and the 32 x 288 activation bytes of its super-block into its own
