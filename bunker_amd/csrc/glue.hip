@@ -366,7 +366,7 @@ int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* 
 // stage 2 walks the partials in index order with a strict ">", so the lowest index
 // wins ties; the running maximum starts at -FLT_MAX and NaN never wins.
 constexpr float ARGMAX_INIT = -3.40282347e38f;
-constexpr int ARGMAX_TILE = 4096;
+constexpr int ARGMAX_TILE = 1024;     // one 16-byte load per thread: a short instruction stream on many CUs (the op is latency-bound)
 
 __device__ __forceinline__ void argmax_merge(float& v, int& i, float ov, int oi) {
   // (ov, oi) beats (v, i) when larger, or equal with a lower index
@@ -382,16 +382,26 @@ __device__ __forceinline__ void argmax_wave(float& v, int& i) {
 }
 
 __global__ __launch_bounds__(256) void argmax_stage1_kernel(const float* __restrict__ logits, float* __restrict__ pv,
-                                                            int32_t* __restrict__ pi, int n, int ntiles) {
+                                                            int32_t* __restrict__ pi, int n, int ntiles, bool vec4) {
   __shared__ float sv[4];
   __shared__ int si[4];
   const int b = blockIdx.y, tile = blockIdx.x;
   const float* L = logits + (int64_t)b * n;
   float v = ARGMAX_INIT; int idx = 0x7fffffff;
   const int base = tile * ARGMAX_TILE;
-  for (int j = threadIdx.x; j < ARGMAX_TILE; j += 256) {
-    const int e = base + j;
-    if (e < n) { const float x = L[e]; if (x > v) { v = x; idx = e; } }
+  const int e0 = base + threadIdx.x * 4;
+  if (vec4 && e0 + 3 < n) {
+    const float4 x = *(const float4*)(L + e0);          // elements in index order, strict >: the lowest index wins a tie
+    if (x.x > v) { v = x.x; idx = e0; }
+    if (x.y > v) { v = x.y; idx = e0 + 1; }
+    if (x.z > v) { v = x.z; idx = e0 + 2; }
+    if (x.w > v) { v = x.w; idx = e0 + 3; }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int e = e0 + j;
+      if (e < n) { const float x = L[e]; if (x > v) { v = x; idx = e; } }
+    }
   }
   argmax_wave(v, idx);
   if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = v; si[threadIdx.x >> 6] = idx; }
@@ -423,7 +433,8 @@ int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace
   const int ntiles = (n + ARGMAX_TILE - 1) / ARGMAX_TILE;
   float* pv = (float*)workspace;
   int32_t* pi = (int32_t*)(pv + (size_t)batch * ntiles);
-  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(ntiles, batch), dim3(256), 0, stream(), logits, pv, pi, n, ntiles);
+  const bool vec4 = n % 4 == 0 && ((uintptr_t)logits & 15) == 0;      // every row then starts on a 16-byte boundary
+  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(ntiles, batch), dim3(256), 0, stream(), logits, pv, pi, n, ntiles, vec4);
   hipLaunchKernelGGL(argmax_stage2_kernel, dim3(batch), dim3(64), 0, stream(), pv, pi, val, idx, ntiles);
   BK_LAUNCH_CHECK();
   return BK_OK;
