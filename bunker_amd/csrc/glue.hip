@@ -33,15 +33,20 @@ int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void*
 // workgroup per row, 8 elements per thread per pass.  With `xq` set the bf16 result
 // is also quantized to Q8_1 in the same pass (four lanes share one 32-element block),
 // which is what the following matmuls consume.
-template <bool QUANT>
+// ONE: the row has at most 2048 elements: a thread's 8 values and weights stay in registers between the two passes
+// (one memory round trip instead of two).
+template <bool QUANT, bool ONE>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                       uint16_t* __restrict__ out, uint8_t* __restrict__ xq, int N) {
   __shared__ double lds[4];
   const int row = blockIdx.x;
   const uint16_t* xr = x + (int64_t)row * N;
   double ss = 0.0;     // squares of bf16 values are exact in f32; their sum is carried in double
+  uint4 keep = make_uint4(0, 0, 0, 0), keepw = keep;
+  if (ONE && threadIdx.x * 8 < N) keepw = *(const uint4*)(w + threadIdx.x * 8);
   for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
     const uint4 v = *(const uint4*)(xr + i);
+    if (ONE) keep = v;
     const uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -52,8 +57,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
   ss = block_sum_f64<4>(ss, lds);
   const float rstd = rsqrt_f64(ss / (double)N + 1e-6);
   for (int i = threadIdx.x * 8; i < N; i += 256 * 8) {
-    const uint4 v = *(const uint4*)(xr + i);
-    const uint4 wv = *(const uint4*)(w + i);
+    const uint4 v = ONE ? keep : *(const uint4*)(xr + i);
+    const uint4 wv = ONE ? keepw : *(const uint4*)(w + i);
     const uint32_t u[4] = {v.x, v.y, v.z, v.w}, uw[4] = {wv.x, wv.y, wv.z, wv.w};
     uint32_t o[4];
     float f[8];
@@ -82,12 +87,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
 int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows) {
   BK_REQUIRE(x && w && (out || xq), "rmsnorm: null pointer");
   BK_REQUIRE(N > 0 && N % 32 == 0 && rows > 0, "rmsnorm: N=%d must be a positive multiple of 32 (rows=%d)", N, rows);
-  if (xq)
-    hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
-                       (uint16_t*)out, (uint8_t*)xq, N);
-  else
-    hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
-                       (uint16_t*)out, (uint8_t*)nullptr, N);
+  const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
+  const bool one = N <= 2048;
+  if (xq && one) hipLaunchKernelGGL((rmsnorm_kernel<true, true>), dim3(rows), dim3(256), 0, stream(), xp, wp, (uint16_t*)out, (uint8_t*)xq, N);
+  else if (xq) hipLaunchKernelGGL((rmsnorm_kernel<true, false>), dim3(rows), dim3(256), 0, stream(), xp, wp, (uint16_t*)out, (uint8_t*)xq, N);
+  else if (one) hipLaunchKernelGGL((rmsnorm_kernel<false, true>), dim3(rows), dim3(256), 0, stream(), xp, wp, (uint16_t*)out, (uint8_t*)nullptr, N);
+  else hipLaunchKernelGGL((rmsnorm_kernel<false, false>), dim3(rows), dim3(256), 0, stream(), xp, wp, (uint16_t*)out, (uint8_t*)nullptr, N);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
