@@ -433,6 +433,7 @@ int bk_tune_set(const char* key, int value) {
   else if (!strcmp(key, "gdn_cs")) bk::g_tune_gdn_cs = value;
   else if (!strcmp(key, "fused_cap")) bk::g_tune_fused_cap = value;
   else if (!strcmp(key, "attn_nt")) bk::g_tune_attn_nt = value;
+  else if (!strcmp(key, "attn_bal")) bk::g_tune_attn_bal = value;
   else if (!strcmp(key, "gemm_r16")) bk::g_tune_gemm_r16 = value;
   else if (!strcmp(key, "gdn_nt")) bk::g_tune_gdn_nt = value;
   else if (!strcmp(key, "gemm_nw")) bk::g_tune_gemm_nw = value;

@@ -21,6 +21,18 @@
 // split with its own running (max, sum, O^T); the four are merged through LDS in a
 // fixed order; with more than one split the workgroup partials go to a workspace
 // and a second kernel merges them, again in a fixed order.
+//
+// Lengths that live in device memory (a captured decode step, a ragged batch): the host cannot size the splits, and
+// cutting every sequence into equal page ranges of the LONGEST context the cache allows leaves the workgroups behind a
+// short context without work.  Two forms, chosen on the host from the bound alone:
+//  - relative: every workgroup divides its own sequence's pages by the number of splits (one division after the length
+//    has arrived); all workgroups of a sequence work, long sequences take longer than short ones;
+//  - balanced (large shares, where the page loop and not the start-up decides the time): the batch's workgroup slots
+//    (B * splits, grid = (slots, NKV)) are handed out in proportion to the lengths.  Every workgroup derives the plan
+//    from the B lengths itself (sums and a prefix sum in the lanes, no extra launch) and takes at most
+//    ceil(total pages / slots) pages, up to a rounding allowance; the first workgroup of a sequence leaves (first slot,
+//    splits) for the merge kernel.
+// With every length at the bound both give the page ranges of the plain form and the same bits.
 #include "ops.h"
 
 namespace bk {
@@ -49,14 +61,57 @@ struct AttnArgs {
   float* lse;                 // f32 [B, NH] or null
   float* part_o;              // f32 [B, NKV, splits, 16, 256] unnormalised partial outputs
   float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
+  int2* plan;                 // balanced form: (first slot, number of splits) of every sequence, behind the partials
   int64_t gate_bstride, gate_hstride;
   int bt_stride, ctx_scalar, ctx_add, NH, NKV, G, splits, pages_per_split;
   int tpw, rows;              // query rows per workgroup (1, or 2 consecutive rows of one sequence: prompt tokens), rows in all
+  int max_pages;              // pages of the longest context the caller allows
+  int rel;                    // 1: lengths in device memory, every sequence cuts its own pages into `splits` equal ranges
+  int slots;                  // > 0: balanced form, this many workgroup slots per KV head shared by the rows (rows <= 64)
   float scale;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+// ceil(a / b) for 0 <= a < 2^24, b >= 1, inv_b ~ 1 / b: the float quotient is off by less than one, the remainder settles it
+__device__ __forceinline__ int ceil_div_rcp(int a, int b, float inv_b) {
+  int q = (int)((float)a * inv_b);
+  int r = a - q * b;
+  if (r < 0) { q -= 1; r += b; }
+  if (r >= b) { q += 1; r -= b; }
+  return q + (r > 0 ? 1 : 0);
+}
+
+// Balanced plan, computed by every wave for itself: lane i < rows holds sequence i's pages `np`, its number of splits
+// `ns` and the first slot `first` of its splits.  The page budget of a slot is ceil(total / slots); when the round-up
+// of the sequences' split counts does not fit the slots, it is taken for rows - 1 slots fewer, which always fits
+// (sum ceil(np_i / t) <= total / t + rows - rows / t).  Sums and the prefix sum stay in the lanes (DPP), no LDS.
+__device__ __forceinline__ void attn_balanced_plan(const AttnArgs& A, int lane, int& np, int& ns, int& first) {
+  // a length outside 1 .. max_ctx (the caller's mistake) still plans inside the block table and the slots
+  np = lane < A.rows ? min(max((A.ctx_len[lane] + A.ctx_add + ATT_PAGE - 1) / ATT_PAGE, 1), A.max_pages) : 0;
+  const int t16 = row16_sum_i32(np);
+  const int total = (__builtin_amdgcn_readlane(t16, 0) + __builtin_amdgcn_readlane(t16, 16)) +
+                    (__builtin_amdgcn_readlane(t16, 32) + __builtin_amdgcn_readlane(t16, 48));
+  int incl = 0;
+  for (int attempt = 0; attempt < 2; attempt++) {
+    const int over = attempt ? A.slots - (A.rows - 1) : A.slots;
+    const int budget = ceil_div_rcp(total, over, __builtin_amdgcn_rcpf((float)over));
+    ns = ceil_div_rcp(np, budget, __builtin_amdgcn_rcpf((float)budget));
+    // inclusive prefix sum: inside each row of 16 lanes by row shifts (lanes without a source read 0), then the rows before
+    int v = ns;
+    v += dpp_i32<0x111>(v);      // row_shr:1
+    v += dpp_i32<0x112>(v);      // row_shr:2
+    v += dpp_i32<0x114>(v);      // row_shr:4
+    v += dpp_i32<0x118>(v);      // row_shr:8
+    const int r0 = __builtin_amdgcn_readlane(v, 15), r1 = __builtin_amdgcn_readlane(v, 31), r2 = __builtin_amdgcn_readlane(v, 47);
+    const int row = lane >> 4;
+    incl = v + (row == 0 ? 0 : row == 1 ? r0 : row == 2 ? r0 + r1 : r0 + r1 + r2);
+    const int used = r0 + r1 + r2 + __builtin_amdgcn_readlane(v, 63);
+    if (used <= A.slots) break;
+  }
+  first = incl - ns;
 }
 
 // PF = pages a wave requests ahead of the one it computes on (0 or 2).  Loads are issued
@@ -68,8 +123,22 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   __shared__ float lds_m[ATT_WAVES][16], lds_l[ATT_WAVES][16];
   __shared__ int lds_bt[ATT_MAX_PPS];           // physical page of every page of this split
 
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;     // b: workgroup's first query row is b * tpw
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int split = blockIdx.x, b = blockIdx.z;       // b: workgroup's first query row is b * tpw
+  const int kvh = blockIdx.y;
+  int pps = A.pages_per_split;
+  if (A.slots > 0) {                            // balanced form: slot blockIdx.x belongs to the sequence whose range holds it
+    int np, ns, first;
+    attn_balanced_plan(A, lane, np, ns, first);
+    const unsigned long long own = __ballot((int)blockIdx.x >= first && (int)blockIdx.x < first + ns);
+    if (own == 0) return;                       // a slot past the last one in use (the whole workgroup leaves)
+    b = __ffsll(own) - 1;
+    split = blockIdx.x - __builtin_amdgcn_readlane(first, b);
+    const int nsb = __builtin_amdgcn_readlane(ns, b);
+    pps = ceil_div_rcp(__builtin_amdgcn_readlane(np, b), nsb, __builtin_amdgcn_rcpf((float)nsb));
+    // the merge kernel finds the sequence's partials through this pair
+    if (split == 0 && kvh == 0 && threadIdx.x == 0) A.plan[b] = make_int2(blockIdx.x, nsb);
+  }
   const int n = lane & 15, kg = lane >> 4;      // n: token (A operand) / head (B operand, C column); kg: lane group
   // column n of the products: head n % G of query row b * tpw + n / G; a row past the last one repeats the first (not stored)
   const int row0 = b * A.tpw;
@@ -80,9 +149,10 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   const int len = (A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add;       // of this lane's column
   int len_max = (A.ctx_len ? A.ctx_len[row0] : A.ctx_scalar) + A.ctx_add;
   if (ntk > 1) len_max = max(len_max, A.ctx_len[row0 + 1] + A.ctx_add);
-  const int npages = (len_max + ATT_PAGE - 1) / ATT_PAGE;
-  const int p_begin = split * A.pages_per_split;
-  const int p_end = min(npages, p_begin + A.pages_per_split);
+  const int npages = min((len_max + ATT_PAGE - 1) / ATT_PAGE, A.max_pages);
+  if (A.rel) pps = ceil_div_rcp(npages, A.splits, __builtin_amdgcn_rcpf((float)A.splits));   // equal parts of its own context
+  const int p_begin = split * pps;
+  const int p_end = min(npages, p_begin + pps);
 
   // Q as the B operand of the first product: lane (column n, group kg) holds dims 32*s + 8*kg .. +8
   uint4 qreg[8];
@@ -260,7 +330,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
       if (d == 0 && A.lse) A.lse[row * A.NH + head] = Mh + logf(Lh);
     }
   } else {
-    const int64_t pidx = ((int64_t)b * A.NKV + kvh) * A.splits + split;
+    const int64_t pidx = A.slots > 0 ? (int64_t)kvh * A.slots + blockIdx.x : ((int64_t)b * A.NKV + kvh) * A.splits + split;
     float* po = A.part_o + pidx * 16 * ATT_HD;
     for (int c = 0; c < ncols; c++) po[c * ATT_HD + d] = lds_o[d][c];
     if (kg == 0 && wave == 0 && n < ncols) {
@@ -278,8 +348,14 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   __shared__ float redm[4], redl[4];
   const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;      // b: query row
   const int kvh = head / A.G, h = (b % A.tpw) * A.G + head % A.G;     // h: the row's column in its workgroup's partials
-  const int64_t p0 = ((int64_t)(b / A.tpw) * A.NKV + kvh) * A.splits;
-  const bool has = d < A.splits;
+  int64_t p0 = ((int64_t)(b / A.tpw) * A.NKV + kvh) * A.splits;
+  int nsplit = A.splits;
+  if (A.slots > 0) {
+    const int2 pl = A.plan[b];
+    nsplit = pl.y;
+    p0 = (int64_t)kvh * A.slots + pl.x;
+  }
+  const bool has = d < nsplit;
   const float ms = has ? A.part_ml[((p0 + d) * 16 + h) * 2] : -INFINITY;
   const float ls = has ? A.part_ml[((p0 + d) * 16 + h) * 2 + 1] : 0.0f;
   float M = wave_max(ms);
@@ -297,13 +373,16 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   const float* po = A.part_o + (p0 * 16 + h) * ATT_HD + d;
   float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
   int s = 0;
-  for (; s + 4 <= A.splits; s += 4) {
+  for (; s + 4 <= nsplit; s += 4) {
     o0 = fmaf(po[(int64_t)(s + 0) * 16 * ATT_HD], wsh[s + 0], o0);
     o1 = fmaf(po[(int64_t)(s + 1) * 16 * ATT_HD], wsh[s + 1], o1);
     o2 = fmaf(po[(int64_t)(s + 2) * 16 * ATT_HD], wsh[s + 2], o2);
     o3 = fmaf(po[(int64_t)(s + 3) * 16 * ATT_HD], wsh[s + 3], o3);
   }
-  for (; s < A.splits; s++) o0 = fmaf(po[(int64_t)s * 16 * ATT_HD], wsh[s], o0);
+  // the last one to three splits keep their own accumulators, so that splits without pages behind them change nothing
+  if (s < nsplit) o0 = fmaf(po[(int64_t)s * 16 * ATT_HD], wsh[s], o0);
+  if (s + 1 < nsplit) o1 = fmaf(po[(int64_t)(s + 1) * 16 * ATT_HD], wsh[s + 1], o1);
+  if (s + 2 < nsplit) o2 = fmaf(po[(int64_t)(s + 2) * 16 * ATT_HD], wsh[s + 2], o2);
   float o = ((o0 + o1) + (o2 + o3)) / L;
   if (A.gate) o = __fmul_rn(o, gsig);
   const uint16_t ob = f32_to_bf16(o);
@@ -313,9 +392,10 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
 }
 
 int g_tune_attn_nt = -1;   // K/V pages through nontemporal loads: 0 off, 1 on, -1 = from the size of the read
+int g_tune_attn_bal = -1;  // lengths in device memory: 0 = plain splits of the bound, 1 = balanced plan wherever it can run, 2 = relative, -1 = by share
 
 size_t attn_workspace_bytes(int batch, int NKV, int max_splits) {
-  return (size_t)batch * NKV * max_splits * 16 * (ATT_HD + 2) * sizeof(float);
+  return (size_t)batch * NKV * max_splits * 16 * (ATT_HD + 2) * sizeof(float) + 64 * sizeof(int2);
 }
 
 int attn_choose_splits(int batch, int NKV, int max_ctx) {
@@ -349,7 +429,8 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
              "attn_decode: two rows per workgroup need a group of at most 8 heads, one shared block table and per-row lengths");
   const int groups = (batch + tpw - 1) / tpw;
   if (splits <= 0) splits = attn_choose_splits(groups, NKV, max_ctx);
-  const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
+  // a context the host knows sizes the splits itself; lengths in device memory leave only their bound
+  const int pages = ((ctx_len ? max_ctx : ctx_scalar + ctx_add) + ATT_PAGE - 1) / ATT_PAGE;
   if (splits > pages) splits = pages;
   BK_REQUIRE(splits <= ATT_MAX_SPLITS, "attn_decode: at most %d splits", ATT_MAX_SPLITS);
   BK_REQUIRE((pages + splits - 1) / splits <= ATT_MAX_PPS, "attn_decode: %d pages in %d splits exceed %d pages per split", pages, splits, ATT_MAX_PPS);
@@ -361,19 +442,33 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   A.bt_stride = bt_stride; A.ctx_scalar = ctx_scalar; A.ctx_add = ctx_add; A.NH = NH; A.NKV = NKV; A.G = NH / NKV;
   A.splits = splits; A.pages_per_split = (pages + splits - 1) / splits;
   A.tpw = tpw; A.rows = batch;
+  // lengths in device memory: balanced plan where a workgroup's share of the bound is long (64 pages and up: below that
+  // start-up and merge decide the time and the plan's own cost of about a microsecond is not won back), else relative
+  // splits; the rows of a prompt keep the plain form (paired and single rows must cut alike).
+  // balanced: the batch shares batch * splits slots; a slot's page budget is largest when rows - 1 slots are held back
+  A.slots = 0; A.rel = 0; A.max_pages = pages;
+  const bool prompt_rows = block_table && bt_stride == 0;
+  if (ctx_len && tpw == 1 && !prompt_rows && splits > 1 && g_tune_attn_bal != 0) {
+    const bool can_balance = batch <= 64 && batch * splits <= ATT_MAX_SPLITS && (int64_t)batch * pages < (1 << 24) &&
+        ((int64_t)batch * pages + (batch * splits - batch)) / (batch * splits - batch + 1) <= ATT_MAX_PPS;
+    const bool want_balance = g_tune_attn_bal == 1 || (g_tune_attn_bal < 0 && A.pages_per_split >= 64);
+    if (can_balance && want_balance) A.slots = batch * splits;
+    else if (pages < (1 << 24)) A.rel = 1;
+  }
   A.scale = (float)(1.0 / sqrt((double)HD));
   if (splits > 1) {
     BK_REQUIRE(workspace && workspace_bytes >= attn_workspace_bytes(batch, NKV, splits),
                "attn_decode: workspace of %zu bytes needed for %d splits", attn_workspace_bytes(batch, NKV, splits), splits);
     A.part_o = (float*)workspace;
     A.part_ml = A.part_o + (size_t)batch * NKV * splits * 16 * ATT_HD;
+    A.plan = (int2*)(A.part_ml + (size_t)batch * NKV * splits * 16 * 2);
   }
   // waves with three pages or more keep two pages in flight ahead of the one they work on
   // A cache read that is larger than what the memory-side cache can still hold when the next token comes round (decode
   // at large batch x context) bypasses the caches; prompt rows re-read the same pages and keep the plain loads.
   const bool nt = g_tune_attn_nt >= 0 ? g_tune_attn_nt != 0
                                       : (tpw == 1 && (int64_t)batch * NKV * max_ctx * ATT_HD * 4 >= ((int64_t)128 << 20));
-  const dim3 grid(splits, NKV, groups), block(ATT_WAVES * 64);
+  const dim3 grid(A.slots > 0 ? A.slots : splits, NKV, A.slots > 0 ? 1 : groups), block(ATT_WAVES * 64);
   if (A.pages_per_split >= 3 * ATT_WAVES) {
     if (nt) hipLaunchKernelGGL((attn_decode_kernel<2, true>), grid, block, 0, stream(), A);
     else hipLaunchKernelGGL((attn_decode_kernel<2, false>), grid, block, 0, stream(), A);

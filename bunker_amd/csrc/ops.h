@@ -46,7 +46,7 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
                       void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
 
 // gemm_mfma.hip
-extern int g_tune_gemm_nw, g_tune_gemm_r16, g_tune_gdn_nt, g_tune_attn_nt;
+extern int g_tune_gemm_nw, g_tune_gemm_r16, g_tune_gdn_nt, g_tune_attn_nt, g_tune_attn_bal;
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi);
 int launch_gemm_swiglu_mfma(const void* xq, int K, int batch, const void* Wg, const void* Wu, int N, void* act, void* act_q8);

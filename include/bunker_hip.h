@@ -83,7 +83,9 @@ BK_API int bk_graph_destroy(uint64_t graph);
 /* Launch-shape knobs for experiments and tests; the defaults (0, or -1 = chosen from the shape) are the tuned values:
  * "gemv_rpi", "gemv_cap", "gemv_impl", "fused_cap" (GEMV rows per wave step, workgroups per CU, kernel variant),
  * "gemm_nw" (waves per matmul tile: 1, 2, 4, 8), "gemm_r16" (tiles of 16 weight rows), "gdn_cs" (column slabs of the
- * GDN core op), "gdn_nt" / "attn_nt" (state / cache pages through nontemporal accesses).  No counterpart in the reference. */
+ * GDN core op), "gdn_nt" / "attn_nt" (state / cache pages through nontemporal accesses), "attn_bal" (attention splits
+ * under lengths in device memory: 0 = equal ranges of max_ctx, 2 = of each sequence's own length, 1 = the batch's
+ * workgroups shared out by length, -1 = 1 for long ranges, else 2).  No counterpart in the reference. */
 BK_API int bk_tune_set(const char* key, int value);
 
 /* ---- per-op launch surface: replaces compileAndLoad + cuLaunch
@@ -170,7 +172,9 @@ BK_API int bk_gdn_core(uint64_t q, uint64_t k, uint64_t v, uint64_t g, uint64_t 
  * ctx_len int32 [batch].  gate: 0, or bf16 with the gate of (b, head, i) at
  * gate[b*gate_bstride + head*gate_hstride + i] (output *= sigmoid(gate)).
  * splits: 0 = let the library choose; with more than one split the caller passes
- * a workspace of bk_attn_workspace_bytes(). */
+ * a workspace of the size bk_attn_plan() returns.  max_ctx bounds the lengths (and the
+ * block table); the page ranges of the splits follow the lengths found in ctx_len
+ * at run time, so a bound far above the contexts costs nothing. */
 BK_API int bk_attn_plan(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes);
 BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride,
                           uint64_t ctx_len, int max_ctx, uint64_t gate, int64_t gate_bstride,

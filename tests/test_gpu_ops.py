@@ -298,6 +298,50 @@ def test_attn_decode_invariants(orc, dev):
     assert np.array_equal(out_p, outs[2][0]) and np.array_equal(lse_p, outs[2][1])
 
 
+def test_attn_decode_splits_follow_lengths_in_device_memory(orc, dev):
+    """Lengths in device memory: relative splits (tune attn_bal = 2: every sequence cuts its own pages) and the balanced
+    plan (1: the batch's workgroup slots handed out in proportion to the lengths) against the plain splits of the
+    bound (0).  With every length at the bound all three cut alike (same bits, also where some splits stay empty);
+    ragged lengths stay within the tolerance, whether the first page budget of the plan fits the slots or not."""
+    g = synth.rng(620)
+    try:
+        B, L = 4, 4100                          # 257 pages: the plain form leaves splits without pages
+        kc, vc, bt, ctx = synth.paged_kv_random(g, B, L)
+        ctx[:] = L
+        q = bf(g.standard_normal((B, 16, 256)).astype(np.float32))
+        rt.tune_set("attn_bal", 0)
+        out0, lse0, s0 = _run_attn(dev, q, kc, vc, bt, ctx, B, L)
+        assert s0 > 1
+        for mode in (1, 2, -1):
+            rt.tune_set("attn_bal", mode)
+            out1, lse1, s1 = _run_attn(dev, q, kc, vc, bt, ctx, B, L)
+            assert s0 == s1
+            assert np.array_equal(out0, out1) and np.array_equal(lse0.view(np.uint32), lse1.view(np.uint32)), mode
+        # ragged: one token, one page, a page and a token, long ones; many rows; a bound far above the contexts
+        for B, L, lens in ((8, 8192, [1, 16, 17, 5000, 8192, 33, 4096, 8191]),
+                           (64, 1024, list(g.integers(1, 1025, 64))),
+                           (2, 20000, [20000, 3]),
+                           (3, 32768, [900, 2100, 1500]),
+                           (1, 9000, [4700])):
+            print(f"attn, lengths on the device: B={B} L={L}", flush=True)
+            kc, vc, bt, ctx = synth.paged_kv_random(g, B, L)
+            ctx[:] = lens
+            q = bf(g.standard_normal((B, 16, 256)).astype(np.float32))
+            ro, rl = orc.attn_decode_paged(q, kc, vc, bt, ctx, B, 16, 2, 256, 16)
+            rt.tune_set("attn_bal", 0)
+            outp, lsep, _ = _run_attn(dev, q, kc, vc, bt, ctx, B, L)
+            for mode in (1, 2, -1):
+                rt.tune_set("attn_bal", mode)
+                out, lse, s = _run_attn(dev, q, kc, vc, bt, ctx, B, L)
+                assert s > 1
+                assert np.abs(f32(out).astype(np.float64) - f32(ro)).max() <= 2e-2, mode
+                assert np.all(np.abs(lse - rl) <= 1e-4 * np.maximum(1, np.abs(rl))), mode
+                assert np.abs(f32(out).astype(np.float64) - f32(outp)).max() <= 1e-2, mode
+                assert np.allclose(lse, lsep, rtol=1e-5, atol=1e-5), mode
+    finally:
+        rt.tune_set("attn_bal", -1)
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 def test_fa2_attn_op_appends_and_attends(orc, dev, batch):
     """The graph's fa2_attn node: slots (q, k, v, qgate, kv_k_in, kv_v_in, pos, out, kv_k_new, kv_v_new)."""
