@@ -35,11 +35,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant GEMV kernel (average over its three shapes), from two rocprofv3 --pmc runs of
+# HBM bytes per launch of the dominant GEMV kernel (gemv_q4k_q8_1_lds_kernel<1,0,4>: the lm_head shape), from two rocprofv3 --pmc runs of
 # `bench.py --sections gemv,calib` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter
 # reads for memcopy_kernel of 175030272 bytes (FETCH_SIZE reads 0.50006 of the bytes: factor 1.99979; WRITE_SIZE factor 1.0).
 # The summary with the per-shape counters is profiles/gemv_q4k_q8_1_decode_shapes.md.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 65721604
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 175699681
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
 ROTATION_BYTES = 600e6  # every shape rotates through copies of its matrix that add up to at least this much
 
@@ -420,12 +420,19 @@ def main():
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # dominant kernel: gemv_q4k_q8_1_kernel<1,0> serves every K=2048 shape (qkv, gate_up, lm_head)
-    dom = [n for n, _, K in SHAPES if K == 2048]
+    # dominant kernel: the instantiation with the largest share of the step.  Rows of 2048 run as
+    # gemv_q4k_q8_1_lds_kernel<1,0,RPI> with RPI = 2 rows per wave step up to 16384 rows and 4 above (lm_head);
+    # rows of 6144 as <3,0,2>.
+    def kernel_of(N, K):
+        return f"gemv_q4k_q8_1_lds_kernel<{K // 2048},0,{4 if (K == 2048 and N > 16384) else 2}>"
+    by_kernel = {}
+    for n, N, K in SHAPES:
+        by_kernel.setdefault(kernel_of(N, K), []).append(n)
+    dom_kernel, dom = max(by_kernel.items(), key=lambda kv: sum(per_shape[n]["us_per_launch"] for n in kv[1]))
     dom_bytes = sum(per_shape[n]["bytes"] for n in dom) / len(dom)
     dom_us = sum(per_shape[n]["us_per_launch"] for n in dom) / len(dom)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemv_q4k_q8_1_lds_kernel<1,0,4>", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": dom_kernel, "shapes": dom, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH}
 

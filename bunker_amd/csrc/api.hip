@@ -427,6 +427,10 @@ extern "C" {
 // "gemv_cap" (workgroups per CU), "gemm_nw" (waves per MFMA tile), "memread_*" (calibration read kernel).
 int bk_tune_set(const char* key, int value) {
   BK_REQUIRE(key, "bk_tune_set: null key");
+  // values that size a grid are checked here: the launchers divide by them
+  if (!strcmp(key, "gemv_cap") || !strcmp(key, "memread_cap"))
+    BK_REQUIRE(value >= 1 && value <= 1024, "bk_tune_set: %s=%d outside 1..1024", key, value);
+  if (!strcmp(key, "gemv_rpi")) BK_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4, "bk_tune_set: gemv_rpi=%d (0, 1, 2 or 4)", value);
   if (!strcmp(key, "gemv_rpi")) bk::g_tune_rpi = value;
   else if (!strcmp(key, "gemv_cap")) bk::g_tune_cap = value;
   else if (!strcmp(key, "gemv_impl")) bk::g_tune_gemv_impl = value;

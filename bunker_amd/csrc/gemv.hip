@@ -187,7 +187,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
 
 int g_tune_gemv_impl = 2;               // 2: rows staged through LDS when K is a multiple of 2048 (else as 0),
                                         // 0: direct loads in the (block, chunk) mapping
-int g_tune_rpi = 4, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows per wave step, workgroups per CU
+int g_tune_rpi = 0, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows per wave step (0: from the shape), workgroups per CU
 
 static int gemv_grid(int N, int rows_per_wg) {
   int wgs = (N + rows_per_wg - 1) / rows_per_wg;
@@ -197,7 +197,7 @@ static int gemv_grid(int N, int rows_per_wg) {
 
 template <int NR, int EPI>
 static void launch_q8_1_rpi(dim3 block, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int nb, int batch) {
-  const int rpi = g_tune_rpi;
+  const int rpi = (g_tune_rpi == 1 || g_tune_rpi == 2) ? g_tune_rpi : 4;
   dim3 grid(gemv_grid(N, GEMV_WAVES * rpi), batch);
   if (rpi == 1) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 1>), grid, block, 0, stream(), w, x, y, r, N, nb);
   else if (rpi == 2) hipLaunchKernelGGL((gemv_q4k_q8_1_kernel<NR, EPI, 2>), grid, block, 0, stream(), w, x, y, r, N, nb);
@@ -206,7 +206,9 @@ static void launch_q8_1_rpi(dim3 block, const uint8_t* w, const uint8_t* x, void
 
 template <int NR, int EPI>
 static void launch_q8_1_lds(dim3 block, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int batch) {
-  const int rpi = NR == 1 ? (g_tune_rpi == 2 ? 2 : 4) : 2;
+  // rows of 2048: two rows per wave step while the matrix is small (twice the workgroups in flight: qkv 3.95 -> 3.65 us,
+  // gate+up 4.8 -> 4.7), four for a long one (lm_head: 29.8 us against 33 with two)
+  const int rpi = NR == 1 ? ((g_tune_rpi == 2 || (g_tune_rpi == 0 && N <= 16384)) ? 2 : 4) : 2;
   dim3 grid(gemv_grid(N, GEMV_WAVES * rpi), batch);
   if (NR == 1 && rpi == 4) hipLaunchKernelGGL((gemv_q4k_q8_1_lds_kernel<NR, EPI, (NR == 1 ? 4 : 2)>), grid, block, 0, stream(), w, x, y, r, N);
   else hipLaunchKernelGGL((gemv_q4k_q8_1_lds_kernel<NR, EPI, 2>), grid, block, 0, stream(), w, x, y, r, N);

@@ -158,14 +158,14 @@ def test_gemv_variants_return_the_same_bits(orc, dev, N, K):
     ref = orc.gemv_q4k_q8_1(W, xq, N, K)
     dW, dxq, dy = dev.up(W), dev.up(xq), dev.empty(N * 4)
     try:
-        for impl, rpi, cap in [(2, 4, 16), (2, 2, 1), (0, 1, 16), (0, 2, 2), (0, 4, 1), (0, 4, 64)]:
+        for impl, rpi, cap in [(2, 0, 16), (2, 4, 16), (2, 2, 1), (0, 1, 16), (0, 2, 2), (0, 4, 1), (0, 4, 64)]:
             rt.tune_set("gemv_impl", impl); rt.tune_set("gemv_rpi", rpi); rt.tune_set("gemv_cap", cap)
             rt.cuMemset(dy, 0xCD, N * 4)
             rt.gemv_q4k_q8_1(dW, dxq, dy, N, K)
             y = rt.from_device(dy, (N,), np.float32)
             assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (impl, rpi, cap, int((y != ref).sum()))
     finally:
-        rt.tune_set("gemv_impl", 2); rt.tune_set("gemv_rpi", 4); rt.tune_set("gemv_cap", 16)
+        rt.tune_set("gemv_impl", 2); rt.tune_set("gemv_rpi", 0); rt.tune_set("gemv_cap", 16)
 
 
 @pytest.mark.parametrize("N,K", [(64, 256), (33, 768), (100, 1792), (128, 4096), (77, 8192), (5, 2048)])
