@@ -60,6 +60,25 @@ def bf16_close(got_bits, ref_bits, ulps=1.0, atol=1e-6):
 
 
 # ------------------------------------------------------------------ glue
+@pytest.mark.parametrize("N", [32, 1024, 2016, 2048, 2080, 4096, 6144])
+def test_rmsnorm_row_lengths(orc, dev, N):
+    """Rows that fit a workgroup's registers (up to 2048 elements, also with idle threads) and rows that take the loop."""
+    print(f"rmsnorm N={N}", flush=True)
+    g = synth.rng(430 + N)
+    rows = 3
+    x = bf((g.standard_normal((rows, N)) * np.exp(g.standard_normal((rows, 1)))).astype(np.float32))
+    w = bf((g.standard_normal(N) * 0.1).astype(np.float32))
+    ref = np.stack([orc.rmsnorm(r, w) for r in x])
+    dx, dw, dn, dxq = dev.up(x), dev.up(w), dev.empty(rows * N * 2), dev.empty(rows * N // 32 * 36)
+    launch(f"rmsnorm N={N} batch={rows}", [dx, dw, dn])
+    assert np.array_equal(rt.from_device(dn, (rows, N), np.uint16), ref)
+    rt.cuMemset(dn, 0xff, rows * N * 2)
+    launch(f"rmsnorm_q8_1 N={N} batch={rows}", [dx, dw, dn, dxq])
+    assert np.array_equal(rt.from_device(dn, (rows, N), np.uint16), ref)
+    xq = rt.from_device(dxq, (rows, N // 32 * 36), np.uint8)
+    assert np.array_equal(xq, np.stack([orc.pack_q8_1(f32(r)) for r in ref]))
+
+
 @pytest.mark.parametrize("batch", [1, 4])
 def test_embed_rmsnorm_cast_add_swiglu(orc, dev, batch):
     print(f"glue batch={batch}", flush=True)
