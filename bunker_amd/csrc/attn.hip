@@ -115,7 +115,7 @@ __device__ __forceinline__ void attn_balanced_plan(const AttnArgs& A, int lane, 
 }
 
 // PF = pages a wave requests ahead of the one it computes on (0 or 2).  Loads are issued
-// unconditionally (past its last page a wave re-requests that page), so the number of loads in
+// unconditionally (past its last page a wave requests a few fixed, cached lines instead), so the number of loads in
 // flight at every wait is known when the kernel is compiled and a wait covers only the page needed.
 template <int PF, bool NT>
 __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A) {
@@ -174,11 +174,15 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   for (int i = threadIdx.x; i < p_end - p_begin; i += ATT_WAVES * 64)
     lds_bt[i] = A.block_table ? A.block_table[(int64_t)row0 * A.bt_stride + p_begin + i] : row0 * A.bt_stride + p_begin + i;
   __syncthreads();
-  auto load_page = [&](int pg, uint4 (&kr)[8], uint2 (&vr)[16]) {
-    const int phys = lds_bt[pg - p_begin];
-    const int64_t base = ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
+  // A request past the wave's last page (issued only to keep the number of loads in flight fixed; its registers are
+  // never computed on) goes to the first bytes of the cache with every lane on the same address: a handful of cache
+  // lines instead of a second and third trip of the last page through memory, which nontemporal loads would make.
+  auto load_page = [&](int pg, int last_pg, uint4 (&kr)[8], uint2 (&vr)[16]) {
+    const bool real = pg <= last_pg;
+    const int phys = lds_bt[min(pg, last_pg) - p_begin];
+    const int64_t base = real ? ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD) : 0;
     // K page as the A operand: lane (token n, group kg) holds dims 32*s + 8*kg .. +8
-    const uint16_t* kp = A.kc + base + n * ATT_HD + 8 * kg;
+    const uint16_t* kp = A.kc + base + (real ? n * ATT_HD + 8 * kg : 0);
 #pragma unroll
     for (int s = 0; s < 8; s++) {
       const u32x4_nt* p4 = (const u32x4_nt*)(kp + 32 * s);
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
       kr[s] = make_uint4(t4[0], t4[1], t4[2], t4[3]);
     }
     // V page as the A operand: lane (dim 16*t + n, group kg) holds tokens 4*kg .. +4
-    const uint16_t* vp = A.vc + base + n * ATT_PAGE + 4 * kg;
+    const uint16_t* vp = A.vc + base + (real ? n * ATT_PAGE + 4 * kg : 0);
 #pragma unroll
     for (int t = 0; t < 16; t++) {
       const u32x2_nt* p2 = (const u32x2_nt*)(vp + t * 16 * ATT_PAGE);
@@ -246,19 +250,19 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
     if (PF == 0) {
       for (; pg < p_end; pg += ATT_WAVES) {
         uint4 kr[8]; uint2 vr[16];
-        load_page(pg, kr, vr);
+        load_page(pg, pg, kr, vr);
         compute_page(kr, vr, pg);
       }
     } else if (pg < p_end) {
       const int last = pg + ((p_end - 1 - pg) / ATT_WAVES) * ATT_WAVES;      // this wave's last page
       uint4 k0[8], k1[8], k2[8];
       uint2 v0[16], v1[16], v2[16];
-      load_page(pg, k0, v0);
-      load_page(min(pg + ATT_WAVES, last), k1, v1);
+      load_page(pg, last, k0, v0);
+      load_page(pg + ATT_WAVES, last, k1, v1);
       while (true) {
-        load_page(min(pg + 2 * ATT_WAVES, last), k2, v2); compute_page(k0, v0, pg); pg += ATT_WAVES; if (pg > last) break;
-        load_page(min(pg + 2 * ATT_WAVES, last), k0, v0); compute_page(k1, v1, pg); pg += ATT_WAVES; if (pg > last) break;
-        load_page(min(pg + 2 * ATT_WAVES, last), k1, v1); compute_page(k2, v2, pg); pg += ATT_WAVES; if (pg > last) break;
+        load_page(pg + 2 * ATT_WAVES, last, k2, v2); compute_page(k0, v0, pg); pg += ATT_WAVES; if (pg > last) break;
+        load_page(pg + 2 * ATT_WAVES, last, k0, v0); compute_page(k1, v1, pg); pg += ATT_WAVES; if (pg > last) break;
+        load_page(pg + 2 * ATT_WAVES, last, k1, v1); compute_page(k2, v2, pg); pg += ATT_WAVES; if (pg > last) break;
       }
     }
   }
