@@ -40,6 +40,13 @@ struct Kernel {
 
 static std::vector<Kernel> g_kernels;
 
+// bk_shutdown: every handle's workspace goes back to the device and the handles become invalid
+void kernels_release_all() {
+  for (Kernel& k : g_kernels)
+    if (k.scratch) (void)hipFree(k.scratch);
+  g_kernels.clear();
+}
+
 std::string kernel_label(int kernel) {
   if (kernel < 0 || kernel >= (int)g_kernels.size()) return "?";
   return g_kernels[kernel].spec;
@@ -246,7 +253,7 @@ static int run_fa2(Kernel& k, const uint64_t* s) {
   const int32_t* pos_dev = dev ? P<int32_t>(s[6]) : nullptr;
   const int pos = dev ? 0 : (int)(int32_t)s[6];
   if (!dev) BK_REQUIRE(pos >= 0 && pos < max_len, "fa2_attn: pos=%d outside the cache (MAX_LEN=%d)", pos, max_len);
-  int rc = launch_kv_append(P<void>(s[1]), P<void>(s[2]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, batch, NKV, HD, 16);
+  int rc = launch_kv_append(P<void>(s[1]), P<void>(s[2]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, max_len, batch, NKV, HD, 16);
   if (rc) return rc;
   // the context of each sequence is its pos + 1
   return launch_attn_decode(P<void>(s[0]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, 1, max_len,
@@ -309,10 +316,11 @@ static int run_argmax(Kernel& k, const uint64_t* s) {
   return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
 }
 
-// ---- op: advance   slots: argmax idx, argmax val, token ids, positions, history, counter    params: batch, max_steps
+// ---- op: advance   slots: argmax idx, argmax val, token ids, positions, history, counter    params: batch, max_steps, max_pos
+// (max_pos = the cache capacity MAX_LEN: positions are not advanced past it, and the cache writers skip a position that reached it)
 static int run_advance(Kernel& k, const uint64_t* s) {
   return launch_advance(P<int32_t>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), P<int32_t>(s[3]), P<int32_t>(s[4]), P<int32_t>(s[5]),
-                        (int)k.get("batch", 1), (int)k.get("max_steps", 0));
+                        (int)k.get("batch", 1), (int)k.get("max_steps", 0), (int)k.get("max_pos", 0));
 }
 
 static int build_kernel(Kernel& k) {
@@ -335,6 +343,7 @@ static int build_kernel(Kernel& k) {
     if (k.op == "rope" || k.op == "ropek") {
       if ((rc = need(k, "ROT_HALF")) || (rc = need(k, "MAX_LEN"))) return rc;
     }
+    if (k.op == "advance" && (rc = need(k, "max_pos"))) return rc;
     if (k.op == "gdn_delta_rule" || k.op == "gdn_conv")
       BK_REQUIRE(k.get("LKD", 128) == 128 && k.get("LVD", 128) == 128, "gdn_delta_rule: dk = dv = 128 only");
     k.run = sp.run; k.nslots = sp.nslots + (k.op == "gdn_conv" && k.get("q8out", 0) ? 1 : 0);
@@ -344,6 +353,7 @@ static int build_kernel(Kernel& k) {
     if ((rc = need(k, "HD")) || (rc = need(k, "NH")) || (rc = need(k, "NKV")) || (rc = need(k, "MAX_LEN"))) return rc;
     const int batch = (int)k.get("batch", 1), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
     BK_REQUIRE(batch >= 1 && NKV >= 1 && max_len >= 1, "fa2_attn: bad batch/NKV/MAX_LEN");
+    BK_REQUIRE(max_len % 16 == 0, "fa2_attn: MAX_LEN=%d must be a multiple of the 16-token page (a sequence owns MAX_LEN/16 pages)", max_len);
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
     if (splits > 1 && (rc = alloc_scratch(k, attn_workspace_bytes(batch, NKV, splits)))) return rc;
@@ -354,6 +364,7 @@ static int build_kernel(Kernel& k) {
     if ((rc = need(k, "HD")) || (rc = need(k, "NH")) || (rc = need(k, "NKV")) || (rc = need(k, "MAX_LEN")) || (rc = need(k, "ROT_HALF"))) return rc;
     const int batch = (int)k.get("batch", 1), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
     BK_REQUIRE(batch >= 1 && NKV >= 1 && max_len >= 1 && k.get("NH", 0) >= 1 && k.get("HD", 0) >= 1, "fa2_fused: bad batch/NH/NKV/HD/MAX_LEN");
+    BK_REQUIRE(max_len % 16 == 0, "fa2_fused: MAX_LEN=%d must be a multiple of the 16-token page (a sequence owns MAX_LEN/16 pages)", max_len);
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
     const size_t qbytes = (size_t)batch * k.get("NH", 0) * k.get("HD", 0) * 2;
@@ -377,7 +388,7 @@ static int build_kernel(Kernel& k) {
     for (const char* p : {"HD", "NH", "NKV", "MAX_LEN", "ROT_HALF", "T"})
       if ((rc = need(k, p))) return rc;
     const int T = (int)k.get("T", 0), NKV = (int)k.get("NKV", 0), max_len = (int)k.get("MAX_LEN", 0);
-    BK_REQUIRE(T >= 1 && T <= 65535 && NKV >= 1 && max_len >= 1, "fa2_prefill: bad T/NKV/MAX_LEN");
+    BK_REQUIRE(T >= 1 && T <= 65535 && NKV >= 1 && max_len >= 1 && max_len % 16 == 0, "fa2_prefill: bad T/NKV/MAX_LEN (MAX_LEN a multiple of 16)");
     // two consecutive tokens per workgroup where their heads fit the 16 columns of the products (pair=0 switches it off)
     const int NHq = (int)k.get("NH", 0);
     const int tpw = (NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
@@ -478,6 +489,7 @@ int bk_launch(int kernel, const uint64_t* slots, int nslots) {
   BK_NEED_INIT();
   if (kernel < 0 || kernel >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "bk_launch: unknown kernel handle %d", kernel);
   Kernel& k = g_kernels[kernel];
+  if (!k.run) return set_error(BK_ERR_STATE, "bk_launch: kernel handle %d has been destroyed", kernel);
   BK_REQUIRE(slots, "bk_launch: null slots");
   BK_REQUIRE(nslots >= k.nslots, "bk_launch: '%s' takes %d argument slots, got %d", k.op.c_str(), k.nslots, nslots);
   if (prof_on()) {
@@ -488,6 +500,20 @@ int bk_launch(int kernel, const uint64_t* slots, int nslots) {
     return rc ? rc : rc2;
   }
   return k.run(k, slots);
+}
+
+int bk_kernel_destroy(int kernel) {
+  BK_NEED_INIT();
+  if (kernel < 0 || kernel >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "bk_kernel_destroy: unknown kernel handle %d", kernel);
+  Kernel& k = g_kernels[kernel];
+  if (!k.run) return BK_OK;                       // destroyed before
+  if (k.scratch) {
+    BK_HIP(hipDeviceSynchronize());               // launches that still use the workspace finish first
+    BK_HIP(hipFree(k.scratch));
+  }
+  k.scratch = nullptr; k.scratch_bytes = 0; k.run = nullptr;     // the slot stays, so later handles keep their numbers
+  k.spec += " [destroyed]";
+  return BK_OK;
 }
 
 int bk_kernel_describe(int kernel, char* buf, int cap) {
@@ -568,12 +594,12 @@ int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, i
                             max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse), P<void>(workspace),
                             (size_t)workspace_bytes, batch, NH, NKV, HD, page_size, splits);
 }
-int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t pos, int batch,
-                 int NKV, int HD, int page_size) {
+int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t pos, int max_len,
+                 int batch, int NKV, int HD, int page_size) {
   BK_NEED_INIT();
   BK_REQUIRE(pos, "bk_kv_append: pos is required");
   return launch_kv_append(P<void>(k), P<void>(v), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride, P<int32_t>(pos), 0,
-                          batch, NKV, HD, page_size);
+                          max_len, batch, NKV, HD, page_size);
 }
 
 }  // extern "C"

@@ -325,13 +325,14 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
         const float mw = lds_m[w][c];
         Lh += (mw == -INFINITY) ? 0.0f : lds_l[w][c] * __expf(mw - Mh);
       }
-      float o = lds_o[d][c] / Lh;
+      // a sequence without context (length <= 0 found in device memory) has no weights: zeros and lse = -inf
+      float o = Lh > 0.0f ? lds_o[d][c] / Lh : 0.0f;
       if (A.gate) {
         const float gv = bf16_to_f32(A.gate[row * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
         o = __fmul_rn(o, sigmoid_f64(gv));
       }
       A.out[(row * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
-      if (d == 0 && A.lse) A.lse[row * A.NH + head] = Mh + logf(Lh);
+      if (d == 0 && A.lse) A.lse[row * A.NH + head] = Lh > 0.0f ? Mh + logf(Lh) : -INFINITY;
     }
   } else {
     const int64_t pidx = A.slots > 0 ? (int64_t)kvh * A.slots + blockIdx.x : ((int64_t)b * A.NKV + kvh) * A.splits + split;
@@ -387,12 +388,12 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs A) {
   if (s < nsplit) o0 = fmaf(po[(int64_t)s * 16 * ATT_HD], wsh[s], o0);
   if (s + 1 < nsplit) o1 = fmaf(po[(int64_t)(s + 1) * 16 * ATT_HD], wsh[s + 1], o1);
   if (s + 2 < nsplit) o2 = fmaf(po[(int64_t)(s + 2) * 16 * ATT_HD], wsh[s + 2], o2);
-  float o = ((o0 + o1) + (o2 + o3)) / L;
+  float o = L > 0.0f ? ((o0 + o1) + (o2 + o3)) / L : 0.0f;      // no context at all: zeros, lse = -inf
   if (A.gate) o = __fmul_rn(o, gsig);
   const uint16_t ob = f32_to_bf16(o);
   A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = ob;
   if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (((int64_t)b * A.NH + head) * (ATT_HD / 32) + (d >> 5)) * 36, d & 31);
-  if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = M + logf(L);
+  if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = L > 0.0f ? M + logf(L) : -INFINITY;
 }
 
 int g_tune_attn_nt = -1;   // K/V pages through nontemporal loads: 0 off, 1 on, -1 = from the size of the read
@@ -501,15 +502,20 @@ struct PrepArgs {
   const int32_t* pos_dev; int pos_scalar;
   uint16_t *qout, *kc, *vc;
   const int32_t* block_table; int bt_stride;
-  int NH, NKV, half;
+  int NH, NKV, half, max_len;
 };
 
 __global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs A) {
   __shared__ uint16_t sh[ATT_HD];
   const int role = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
-  const int pos = A.pos_dev ? A.pos_dev[b] : A.pos_scalar;
+  // A position read from device memory cannot be checked by the host: one outside the cache (a loop replayed past its
+  // capacity) writes nothing, like the masked store of src/emitters.ts:203-205, and reads the tables at the nearest row.
+  const int pos_raw = A.pos_dev ? A.pos_dev[b] : A.pos_scalar;
+  const int pos = min(max(pos_raw, 0), A.max_len - 1);
+  const bool in_cache = pos == pos_raw;
   const int pg = pos / ATT_PAGE, slot = pos % ATT_PAGE;
   const bool is_q = role < A.NH, is_k = !is_q && role < A.NH + A.NKV;
+  if (!is_q && !in_cache) return;
   const int kvh = is_q ? 0 : (is_k ? role - A.NH : role - A.NH - A.NKV);
   const int phys = A.block_table ? A.block_table[(int64_t)b * A.bt_stride + pg] : b * A.bt_stride + pg;
   const int64_t base = ((int64_t)phys * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
@@ -555,13 +561,15 @@ int launch_attn_prep(const void* qg, const void* k, const void* v, const void* q
   BK_REQUIRE(qg && k && v && qw && kw && cos_t && sin_t && qout && kc && vc, "attn_prep: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_prep: head_dim 256 and 16-token pages only");
   BK_REQUIRE(batch > 0 && batch <= 65535 && NH > 0 && NKV > 0 && half > 0 && 2 * half <= HD, "attn_prep: bad shape");
+  BK_REQUIRE(max_len >= 1 && (bt_stride == 0 || (max_len + ATT_PAGE - 1) / ATT_PAGE <= bt_stride),
+             "attn_prep: max_len=%d exceeds the %d pages of a block table row", max_len, bt_stride);
   BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len && pos_scalar / ATT_PAGE < bt_stride),
              "attn_prep: pos=%d outside the cache (max_len=%d)", pos_scalar, max_len);
   PrepArgs A{};
   A.qg = (const uint16_t*)qg; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v; A.qw = (const uint16_t*)qw; A.kw = (const uint16_t*)kw;
   A.cos_t = cos_t; A.sin_t = sin_t; A.pos_dev = pos_dev; A.pos_scalar = pos_scalar;
   A.qout = (uint16_t*)qout; A.kc = (uint16_t*)kc; A.vc = (uint16_t*)vc; A.block_table = block_table; A.bt_stride = bt_stride;
-  A.NH = NH; A.NKV = NKV; A.half = half;
+  A.NH = NH; A.NKV = NKV; A.half = half; A.max_len = max_len;
   hipLaunchKernelGGL(attn_prep_kernel, dim3(NH + 2 * NKV, batch), dim3(64), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
@@ -573,9 +581,11 @@ int launch_attn_prep(const void* qg, const void* k, const void* v, const void* q
 __global__ __launch_bounds__(256) void kv_append_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
                                                         uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
                                                         const int32_t* __restrict__ block_table, int bt_stride,
-                                                        const int32_t* __restrict__ pos_dev, int pos_scalar, int NKV) {
+                                                        const int32_t* __restrict__ pos_dev, int pos_scalar, int NKV,
+                                                        int max_len) {
   const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  if (pos < 0 || pos >= max_len) return;      // outside the cache: nothing is written (src/emitters.ts:203-205 masks the same store)
   const int pg = pos / ATT_PAGE, slot = pos % ATT_PAGE;
   const int phys = block_table ? block_table[(int64_t)b * bt_stride + pg] : b * bt_stride + pg;
   const int64_t base = ((int64_t)phys * NKV + kvh) * (ATT_PAGE * ATT_HD);
@@ -585,13 +595,15 @@ __global__ __launch_bounds__(256) void kv_append_kernel(const uint16_t* __restri
 }
 
 int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
-                     const int32_t* pos_dev, int pos_scalar, int batch, int NKV, int HD, int page_size) {
+                     const int32_t* pos_dev, int pos_scalar, int max_len, int batch, int NKV, int HD, int page_size) {
   BK_REQUIRE(k && v && kc && vc, "kv_append: null pointer");
+  BK_REQUIRE(max_len >= 1 && (max_len + ATT_PAGE - 1) / ATT_PAGE <= bt_stride, "kv_append: max_len=%d exceeds the %d pages of a block table row",
+             max_len, bt_stride);
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "kv_append: head_dim 256 and 16-token pages only");
   BK_REQUIRE(batch > 0 && batch <= 65535 && NKV > 0 && NKV <= 65535, "kv_append: bad shape");
-  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar / ATT_PAGE < bt_stride), "kv_append: pos=%d outside the block table", pos_scalar);
+  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len), "kv_append: pos=%d outside the cache (max_len=%d)", pos_scalar, max_len);
   hipLaunchKernelGGL(kv_append_kernel, dim3(NKV, batch), dim3(256), 0, stream(), (const uint16_t*)k, (const uint16_t*)v,
-                     (uint16_t*)kc, (uint16_t*)vc, block_table, bt_stride, pos_dev, pos_scalar, NKV);
+                     (uint16_t*)kc, (uint16_t*)vc, block_table, bt_stride, pos_dev, pos_scalar, NKV, max_len);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(64) void headnorm_kernel(const uint16_t* __restrict
                                                       uint16_t* __restrict__ out, int nheads, int HD, int in_stride,
                                                       int64_t in_bstride, const float* __restrict__ cos_t,
                                                       const float* __restrict__ sin_t, const int32_t* __restrict__ pos_dev,
-                                                      int pos_scalar, int half) {
+                                                      int pos_scalar, int half, int max_len) {
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const uint16_t* xh = x + (int64_t)b * in_bstride + (int64_t)h * in_stride;
   uint16_t* oh = out + ((int64_t)b * nheads + h) * HD;
@@ -310,7 +310,8 @@ __global__ __launch_bounds__(64) void headnorm_kernel(const uint16_t* __restrict
     for (int i = lane; i < HD; i += 64) oh[i] = normed(i);
     return;
   }
-  const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  // a position from device memory is held inside the table (the host checks only scalar positions)
+  const int pos = min(max(pos_dev ? pos_dev[b] : pos_scalar, 0), max_len - 1);
   for (int i = lane; i < HD; i += 64) {
     if (i >= 2 * half) {
       oh[i] = normed(i);
@@ -330,10 +331,10 @@ int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD,
   BK_REQUIRE(nheads > 0 && HD > 0 && in_stride >= HD && batch > 0 && batch <= 65535, "headnorm: bad shape");
   if (cos_t) {
     BK_REQUIRE(sin_t && half > 0 && 2 * half <= HD, "headnorm+rope: bad tables / half=%d", half);
-    BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
+    BK_REQUIRE(max_len >= 1 && (pos_dev || (pos_scalar >= 0 && pos_scalar < max_len)), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
   }
   hipLaunchKernelGGL(headnorm_kernel, dim3(nheads, batch), dim3(64), 0, stream(), (const uint16_t*)x, (const uint16_t*)w,
-                     (uint16_t*)out, nheads, HD, in_stride, in_bstride, cos_t, sin_t, pos_dev, pos_scalar, half);
+                     (uint16_t*)out, nheads, HD, in_stride, in_bstride, cos_t, sin_t, pos_dev, pos_scalar, half, max_len);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
@@ -341,12 +342,12 @@ int launch_headnorm(const void* x, const void* w, void* out, int nheads, int HD,
 // src/emitters.ts:150-183 emitRoPE / emitRoPEK: in place on bf16 [B, nheads, HD].
 __global__ __launch_bounds__(256) void rope_kernel(uint16_t* __restrict__ x, const float* __restrict__ cos_t,
                                                    const float* __restrict__ sin_t, const int32_t* __restrict__ pos_dev,
-                                                   int pos_scalar, int nheads, int HD, int half) {
+                                                   int pos_scalar, int nheads, int HD, int half, int max_len) {
   const int b = blockIdx.y;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= nheads * half) return;
   const int h = t / half, i = t % half;
-  const int pos = pos_dev ? pos_dev[b] : pos_scalar;
+  const int pos = min(max(pos_dev ? pos_dev[b] : pos_scalar, 0), max_len - 1);     // device positions are held inside the table
   uint16_t* p1 = x + ((int64_t)b * nheads + h) * HD + i;
   uint16_t* p2 = p1 + half;
   const float x1 = bf16_to_f32(*p1), x2 = bf16_to_f32(*p2);
@@ -359,9 +360,9 @@ int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* 
                 int HD, int half, int max_len, int batch) {
   BK_REQUIRE(x && cos_t && sin_t, "rope: null pointer");
   BK_REQUIRE(nheads > 0 && half > 0 && 2 * half <= HD && batch > 0 && batch <= 65535, "rope: bad shape");
-  BK_REQUIRE(pos_dev || (pos_scalar >= 0 && pos_scalar < max_len), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
+  BK_REQUIRE(max_len >= 1 && (pos_dev || (pos_scalar >= 0 && pos_scalar < max_len)), "rope: pos=%d outside the table (max_len=%d)", pos_scalar, max_len);
   hipLaunchKernelGGL(rope_kernel, dim3((nheads * half + 255) / 256, batch), dim3(256), 0, stream(), (uint16_t*)x, cos_t, sin_t,
-                     pos_dev, pos_scalar, nheads, HD, half);
+                     pos_dev, pos_scalar, nheads, HD, half, max_len);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
@@ -452,7 +453,7 @@ int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace
 __global__ __launch_bounds__(256) void advance_kernel(const int32_t* __restrict__ idx, const float* __restrict__ val,
                                                       int32_t* __restrict__ ids, int32_t* __restrict__ pos,
                                                       int32_t* __restrict__ hist, int32_t* __restrict__ counter, int batch,
-                                                      int max_steps) {
+                                                      int max_steps, int max_pos) {
   const int c = counter[0];
   __syncthreads();
   for (int b = threadIdx.x; b < batch; b += 256) {
@@ -461,16 +462,18 @@ __global__ __launch_bounds__(256) void advance_kernel(const int32_t* __restrict_
       hist[((int64_t)c * batch + b) * 2 + 1] = __float_as_int(val[b]);
     }
     ids[b] = idx[b];
-    pos[b] += 1;
+    // positions stop at max_pos (the cache capacity): a replay past it finds pos == max_pos, which the cache writers skip
+    const int p = pos[b];
+    if (p < max_pos) pos[b] = p + 1;
   }
   if (threadIdx.x == 0) counter[0] = c + 1;
 }
 
 int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
-                   int max_steps) {
+                   int max_steps, int max_pos) {
   BK_REQUIRE(idx && val && ids && pos && hist && counter, "advance: null pointer");
-  BK_REQUIRE(batch > 0 && max_steps > 0, "advance: bad batch=%d max_steps=%d", batch, max_steps);
-  hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(256), 0, stream(), idx, val, ids, pos, hist, counter, batch, max_steps);
+  BK_REQUIRE(batch > 0 && max_steps > 0 && max_pos > 0, "advance: bad batch=%d max_steps=%d max_pos=%d", batch, max_steps, max_pos);
+  hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(256), 0, stream(), idx, val, ids, pos, hist, counter, batch, max_steps, max_pos);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -70,7 +70,7 @@ size_t argmax_workspace_bytes(int n, int batch);
 int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch);
 
 int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
-                   int max_steps);
+                   int max_steps, int max_pos);
 
 // gdn.hip
 extern int g_tune_gdn_cs;
@@ -93,6 +93,6 @@ int launch_attn_prep(const void* qg, const void* k, const void* v, const void* q
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
                      void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size);
 int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
-                     const int32_t* pos_dev, int pos_scalar, int batch, int NKV, int HD, int page_size);
+                     const int32_t* pos_dev, int pos_scalar, int max_len, int batch, int NKV, int HD, int page_size);
 
 }  // namespace bk

@@ -59,6 +59,7 @@ int prof_end() {
   return BK_OK;
 }
 std::string kernel_label(int kernel);   // api.hip
+void kernels_release_all();             // api.hip
 static int prof_collect() {
   if (int rc = sync_all()) return rc;
   for (auto& p : g_pending) {
@@ -109,6 +110,7 @@ int bk_init(int device) {
 int bk_shutdown(void) {
   if (!g_inited) return BK_OK;
   (void)sync_all();
+  kernels_release_all();
   for (auto& p : g_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto& ev : g_pool) (void)hipEventDestroy(ev);
   g_pending.clear(); g_pool.clear(); g_totals.clear();

@@ -58,6 +58,11 @@ class Dims:
     def is_full_attention(self, layer: int) -> bool:
         return layer % self.FAI == self.FAI - 1
 
+    def __post_init__(self):
+        # a sequence owns MAX_LEN/16 whole pages of the cache; the kernels size block-table rows from it
+        if self.MAX_LEN < 16 or self.MAX_LEN % 16 != 0:
+            raise ValueError(f"Dims: MAX_LEN={self.MAX_LEN} must be a positive multiple of the 16-token page")
+
 
 SYNTH = Dims()
 # src/model.ts:14-18

@@ -477,6 +477,12 @@ class DecodeEnv:
 
 
 # ---------------------------------------------------------------- device-resident loop
+def cache_capacity(graph: Graph):
+    """Tokens a sequence's KV cache (and the rope tables) hold: MAX_LEN of the graph's attention nodes, None without any."""
+    caps = [int(n.params["MAX_LEN"]) for n in graph.nodes if "MAX_LEN" in n.params]
+    return min(caps) if caps else None
+
+
 class DeviceLoop:
     """Greedy decode with token ids and positions in device memory and the step in a HIP graph.
 
@@ -489,11 +495,21 @@ class DeviceLoop:
                  partition: Partition | None = None, use_graph: bool = True):
         if not env.inplace:
             raise ValueError("DeviceLoop needs DecodeEnv(inplace_state=True)")
+        ids = np.asarray(start_tokens, np.int32).reshape(batch)
+        pos = np.broadcast_to(np.asarray(start_pos, np.int32), (batch,)).copy()
+        # Positions advance on the device, where no launcher can check them: the whole run must fit the cache before
+        # anything is launched.  (The kernels skip a cache write past the capacity, but the tokens would be wrong.)
+        max_len = cache_capacity(graph)
+        if max_steps < 1:
+            raise ValueError(f"DeviceLoop: max_steps={max_steps} must be at least 1")
+        if int(pos.min()) < 0:
+            raise ValueError(f"DeviceLoop: negative start position {int(pos.min())}")
+        if max_len is not None and int(pos.max()) + max_steps > max_len:
+            raise ValueError(f"DeviceLoop: start position {int(pos.max())} + {max_steps} steps exceeds the KV capacity "
+                             f"MAX_LEN={max_len}")
         self.graph, self.env, self.batch, self.max_steps = graph, env, batch, max_steps
         self.compiled = compileStep(graph, partition or choosePartition(graph), batch, device_scalars=True)
         env.bind(self.compiled)
-        ids = np.asarray(start_tokens, np.int32).reshape(batch)
-        pos = np.broadcast_to(np.asarray(start_pos, np.int32), (batch,)).copy()
         self.d_ids = rt.to_device(ids)
         self.d_pos = rt.to_device(pos)
         self.d_hist = rt.cuAlloc(max_steps * batch * 8)
@@ -501,7 +517,7 @@ class DeviceLoop:
         argmax = next(n for n in graph.nodes if n.op == "argmax")
         self.idx_ptr = env.resolve(argmax.outputs[1].tensorName)
         self.val_ptr = env.resolve(argmax.outputs[0].tensorName)
-        self.k_adv = rt.compileAndLoad(f"advance batch={batch} max_steps={max_steps}")
+        self.k_adv = rt.compileAndLoad(f"advance batch={batch} max_steps={max_steps} max_pos={max_len if max_len is not None else 2**31 - 1}")
         self.launches = []
         for plan, k in self.compiled.schedule:
             args = [self.d_ids if a == "token_id" else self.d_pos if a == "pos" else env.resolve(a) for a in plan.args]
@@ -521,6 +537,8 @@ class DeviceLoop:
         for _ in range(n):
             if self.steps_done >= self.max_steps:
                 raise RuntimeError("DeviceLoop: history is full")
+            if not self.launches:
+                raise RuntimeError("DeviceLoop: closed")
             if self.graph_exec is not None:
                 self.graph_exec.launch()
             else:
@@ -532,6 +550,24 @@ class DeviceLoop:
                         self._enqueue()
                     self.graph_exec = gr
             self.steps_done += 1
+
+    def close(self):
+        """Release what the loop owns on the device: the recorded graph, the kernel handles with their workspaces and
+        the four small buffers.  The DecodeEnv (weights, state) is the caller's."""
+        rt.cuSync()
+        if self.graph_exec is not None:
+            self.graph_exec.destroy()
+            self.graph_exec = None
+        seen = set()
+        for k, _, _ in self.launches:
+            if k.fn not in seen:
+                seen.add(k.fn)
+                rt.unloadKernel(k)
+        self.launches = []
+        for p in (self.d_ids, self.d_pos, self.d_hist, self.d_count):
+            if p:
+                rt.cuFree(p)
+        self.d_ids = self.d_pos = self.d_hist = self.d_count = 0
 
     def tokens(self):
         """(tokens int32 [steps, batch], logits f32 [steps, batch]) generated so far."""

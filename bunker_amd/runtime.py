@@ -47,7 +47,7 @@ _SIGS = {
     "bk_capture_begin": [], "bk_capture_end": [C.POINTER(u64)], "bk_graph_launch": [u64],
     "bk_graph_destroy": [u64],
     "bk_tune_set": [C.c_char_p, i32],
-    "bk_kernel_create": [C.c_char_p], "bk_launch": [i32, C.POINTER(u64), i32],
+    "bk_kernel_create": [C.c_char_p], "bk_launch": [i32, C.POINTER(u64), i32], "bk_kernel_destroy": [i32],
     "bk_kernel_describe": [i32, C.c_char_p, i32],
     "bk_memread": [u64, i64, u64], "bk_memcopy": [u64, u64, i64],
     "bk_quantize_q8_1": [u64, i32, u64, i32, i32],
@@ -61,7 +61,7 @@ _SIGS = {
     "bk_gdn_core": [u64, u64, u64, u64, u64, u64, u64, u64, i32, i32],
     "bk_attn_plan": [i32, i32, i32, C.POINTER(i32), C.POINTER(u64)],
     "bk_attn_decode": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, u64, u64, i32, i32, i32, i32, i32, i32],
-    "bk_kv_append": [u64, u64, u64, u64, u64, i32, u64, i32, i32, i32, i32],
+    "bk_kv_append": [u64, u64, u64, u64, u64, i32, u64, i32, i32, i32, i32, i32],
 }
 
 
@@ -227,6 +227,11 @@ def compileAndLoad(spec: str, funcName: str | None = None, numWarps: int = 4, la
     """
     h = _check(cu().bk_kernel_create(spec.encode()), f"compileAndLoad({spec!r})")
     return LoadedKernel(module=0, fn=h, shmem=0, label=label or spec)
+
+
+def unloadKernel(k: LoadedKernel) -> None:
+    """Give the handle's device workspace back (cuModuleUnload is the reference's nearest call); the handle is invalid afterwards."""
+    _check(cu().bk_kernel_destroy(k.fn), "bk_kernel_destroy")
 
 
 def cuLaunch(k: LoadedKernel, grid: Sequence[int], block: Sequence[int], args: Sequence[int]) -> int:
@@ -446,9 +451,10 @@ def attn_decode(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_
            "bk_attn_decode")
 
 
-def kv_append(k: int, v: int, kc: int, vc: int, block_table: int, bt_stride: int, pos: int, batch: int, NKV: int = 2,
-              HD: int = 256, page_size: int = 16) -> None:
-    _check(cu().bk_kv_append(k, v, kc, vc, block_table, bt_stride, pos, batch, NKV, HD, page_size), "bk_kv_append")
+def kv_append(k: int, v: int, kc: int, vc: int, block_table: int, bt_stride: int, pos: int, max_len: int, batch: int,
+              NKV: int = 2, HD: int = 256, page_size: int = 16) -> None:
+    """``max_len``: capacity of a sequence in tokens; a position outside 0..max_len-1 writes nothing."""
+    _check(cu().bk_kv_append(k, v, kc, vc, block_table, bt_stride, pos, max_len, batch, NKV, HD, page_size), "bk_kv_append")
 
 
 def v_pages_to_device_layout(vc) -> "np.ndarray":

@@ -13,8 +13,13 @@
  *   - every function returns int32: 0 = ok, < 0 = error; bk_last_error() then
  *     returns a message owned by the library (thread-local, never freed by the
  *     caller);
- *   - one HIP stream per process; launches are asynchronous, bk_sync() waits;
- *   - single-threaded use, like the reference (one JS thread, one context).
+ *   - launches are asynchronous on the selected stream of the library (its first
+ *     stream unless bk_stream_use chose another); bk_sync() waits for all of them;
+ *   - single-threaded use, like the reference (one JS thread, one context): the
+ *     selected stream, an open capture, the kernel handles and the profiler table
+ *     are state of the process, not of a thread.  A host with several threads
+ *     must call the library from one of them (or under one lock); only
+ *     bk_last_error()'s message is kept per thread.
  */
 #ifndef BUNKER_HIP_H
 #define BUNKER_HIP_H
@@ -97,6 +102,11 @@ BK_API int bk_tune_set(const char* key, int value);
  * scalars in the low 4 bytes); grid and block are the kernel's own business. */
 BK_API int bk_kernel_create(const char* spec);
 BK_API int bk_launch(int kernel, const uint64_t* slots, int nslots);
+/* Handles of ops with intermediate results (gemm, gemv_fused, fa2_*, argmax, gdn_prefill) own a device workspace,
+ * allocated by bk_kernel_create.  bk_kernel_destroy waits for the device, returns the workspace and makes the handle
+ * invalid (later handles keep their numbers); bk_shutdown does the same for every handle.  cuModuleUnload is the
+ * reference's nearest counterpart (its kernels own no device memory, src/ttir.ts:488-491). */
+BK_API int bk_kernel_destroy(int kernel);
 BK_API int bk_kernel_describe(int kernel, char* buf, int cap);
 
 /* Calibration kernels: a plain streaming read (16 bytes per lane, result discarded into the
@@ -174,7 +184,10 @@ BK_API int bk_gdn_core(uint64_t q, uint64_t k, uint64_t v, uint64_t g, uint64_t 
  * splits: 0 = let the library choose; with more than one split the caller passes
  * a workspace of the size bk_attn_plan() returns.  max_ctx bounds the lengths (and the
  * block table); the page ranges of the splits follow the lengths found in ctx_len
- * at run time, so a bound far above the contexts costs nothing. */
+ * at run time, so a bound far above the contexts costs nothing.
+ * Lengths live in device memory, so the host cannot check them: a length above max_ctx is
+ * read as max_ctx (no page beyond the block table row is touched); a length <= 0 gives
+ * an all-zero output row and lse = -inf. */
 BK_API int bk_attn_plan(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes);
 BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride,
                           uint64_t ctx_len, int max_ctx, uint64_t gate, int64_t gate_bstride,
@@ -182,9 +195,13 @@ BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_t
                           uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size,
                           int splits);
 /* The cache write of emitFA2Attn (src/emitters.ts:202-205): k, v bf16 [batch, NKV, 256]
- * of this step go to token pos[b] of every sequence (pos int32 [batch] on the device). */
+ * of this step go to token pos[b] of every sequence (pos int32 [batch] on the device).
+ * max_len is the capacity of a sequence in tokens (at most 16 * bt_stride): a position
+ * outside 0 .. max_len-1 writes nothing, as the reference's store is masked
+ * (boundaryCheck, src/emitters.ts:203-205). */
 BK_API int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table,
-                        int bt_stride, uint64_t pos, int batch, int NKV, int HD, int page_size);
+                        int bt_stride, uint64_t pos, int max_len, int batch, int NKV, int HD,
+                        int page_size);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,49 @@ def test_header_symbols_are_exported():
     assert set(rt._SIGS) | {"bk_last_error"} == set(names)
 
 
+_CTYPE = {
+    "int": rt.i32, "int64_t": rt.i64, "uint64_t": rt.u64,
+    "const char*": C.c_char_p, "char*": C.c_char_p, "const void*": rt.vp, "void*": rt.vp,
+    "uint64_t*": C.POINTER(rt.u64), "const uint64_t*": C.POINTER(rt.u64), "int*": C.POINTER(rt.i32),
+    "float*": C.POINTER(C.c_float),
+}
+
+
+def _header_prototypes():
+    """name -> list of C parameter types, parsed from the BK_API lines of include/bunker_hip.h."""
+    import re
+
+    text = open(rt.HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    protos = {}
+    for ret, name, args in re.findall(r"BK_API\s+([\w\s\*]+?)\b(bk_\w+)\s*\(([^)]*)\)\s*;", text):
+        params = []
+        args = " ".join(args.split())
+        if args and args != "void":
+            for a in args.split(","):
+                toks = a.strip().replace("*", " * ").split()
+                # the last identifier is the parameter name; pointer stars belong to the type
+                if toks[-1] != "*":
+                    toks = toks[:-1]
+                params.append(" ".join(toks).replace(" *", "*"))
+        protos[name] = (" ".join(ret.split()), params)
+    return protos
+
+
+def test_binding_signatures_match_the_header():
+    """Argument count and type of every ctypes signature against the C declaration (ctypes itself checks nothing)."""
+    protos = _header_prototypes()
+    assert set(protos) == set(rt.declared_symbols())
+    for name, sig in rt._SIGS.items():
+        ret, params = protos[name]
+        assert ret == "int", (name, ret)
+        assert len(params) == len(sig), f"{name}: header has {len(params)} parameters {params}, binding {len(sig)}"
+        for i, (ct, py) in enumerate(zip(params, sig)):
+            assert ct in _CTYPE, f"{name}: parameter {i} has a type this check does not know: {ct!r}"
+            assert _CTYPE[ct] is py or _CTYPE[ct] == py, f"{name}: parameter {i} is {ct!r} in the header, {py} in the binding"
+    assert protos["bk_last_error"] == ("const char*", [])
+
+
 def test_calls_before_init_fail_with_message():
     lib = _lib_or_skip()
     out = C.c_uint64(0)

@@ -148,3 +148,47 @@ def test_fused_partition_groups_and_specs():
     # residual of the fused matmul + cast + add is the add's other input
     down = next(p for p in plans if p.spec.startswith("gemv_fused K=6144"))
     assert g.t(down.args[2]).producer.op == "add" and g.t(down.args[3]).producer.op == "add"
+
+
+class _NoDeviceEnv:
+    """Stands in for a DecodeEnv in checks that must fail before anything touches the device."""
+    inplace = True
+
+
+def test_device_loop_refuses_runs_past_the_cache():
+    """Positions advance on the device, so the capacity is checked on the host before any launch
+    (the reference masks the same store, src/emitters.ts:203-205).  TINY holds 64 tokens."""
+    import pytest
+
+    from bunker_amd import model, runner
+
+    gr = model.buildModelGraph(model.TINY, 2)
+    assert runner.cache_capacity(gr) == model.TINY.MAX_LEN == 64
+    env = _NoDeviceEnv()
+    with pytest.raises(ValueError, match="exceeds the KV capacity"):
+        runner.DeviceLoop(gr, env, 2, [1, 2], [10, 60], max_steps=5)        # 60 + 5 > 64
+    with pytest.raises(ValueError, match="exceeds the KV capacity"):
+        runner.DeviceLoop(gr, env, 2, [1, 2], 64, max_steps=1)
+    with pytest.raises(ValueError, match="negative start position"):
+        runner.DeviceLoop(gr, env, 2, [1, 2], [-1, 3], max_steps=2)
+    with pytest.raises(ValueError, match="max_steps"):
+        runner.DeviceLoop(gr, env, 2, [1, 2], 0, max_steps=0)
+    # a run that fits passes the checks and only then needs the device
+    try:
+        runner.DeviceLoop(gr, env, 2, [1, 2], [10, 60], max_steps=4)
+    except ValueError as e:       # pragma: no cover
+        raise AssertionError(f"a run that fits was refused: {e}")
+    except Exception:
+        pass                      # no device here (or the stand-in env): anything but the capacity check
+
+
+def test_dims_refuse_a_capacity_that_is_not_whole_pages():
+    import pytest
+
+    from bunker_amd import model
+
+    with pytest.raises(ValueError, match="multiple of the 16-token page"):
+        model.with_context(model.TINY, 100)
+    with pytest.raises(ValueError, match="multiple of the 16-token page"):
+        model.Dims(MAX_LEN=0)
+    assert model.with_context(model.TINY, 128).MAX_LEN == 128
