@@ -594,6 +594,15 @@ int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, i
                             max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse), P<void>(workspace),
                             (size_t)workspace_bytes, batch, NH, NKV, HD, page_size, splits);
 }
+int bk_attn_decode_noalloc(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t ctx_len, int max_ctx,
+                           uint64_t gate, int64_t gate_bstride, int64_t gate_hstride, uint64_t out, uint64_t lse, int batch, int NH,
+                           int NKV, int HD, int page_size, int splits) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ctx_len, "bk_attn_decode_noalloc: ctx_len is required");
+  return launch_attn_decode_noalloc(current_device(), P<void>(q), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride,
+                                    P<int32_t>(ctx_len), max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse),
+                                    batch, NH, NKV, HD, page_size, splits);
+}
 int bk_kv_append(uint64_t k, uint64_t v, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t pos, int max_len,
                  int batch, int NKV, int HD, int page_size) {
   BK_NEED_INIT();

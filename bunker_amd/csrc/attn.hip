@@ -488,6 +488,54 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   return BK_OK;
 }
 
+// ---------------------------------------------------------------- split-K attention that allocates nothing
+// For callers that cannot allocate (code under graph capture, tight serving loops): the partial results of the splits go
+// to a fixed array in device memory instead of a caller's workspace.  Every GPU the library runs on holds its own copy
+// of the array at its own address, which the host learns once per device from hipGetSymbolAddress; in host code the
+// array's name is not a device address and is never passed to a kernel or a copy.
+constexpr int NOALLOC_MAX_PARTIALS = 1024;        // batch * NKV * splits workgroup partials of 16 x (256 + 2) floats
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)NOALLOC_MAX_PARTIALS * 16 * (ATT_HD + 2) * sizeof(float) + 64 * sizeof(int2);
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];      // 16.1 MiB per GPU, for the life of the process
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// called by bk_init with `device` current: the address of this device's copy of `scratch`
+int attn_noalloc_setup(int device) {
+  BK_REQUIRE(device >= 0 && device < NOALLOC_MAX_DEVICES, "attn_noalloc_setup: device %d beyond the %d this build keeps an address for", device,
+             NOALLOC_MAX_DEVICES);
+  void* p = nullptr;
+  BK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  BK_REQUIRE(p != nullptr, "attn_noalloc_setup: no device address for the scratch array");
+  g_scratch_ptr[device] = p;
+  return BK_OK;
+}
+void attn_noalloc_teardown(int device) {
+  if (device >= 0 && device < NOALLOC_MAX_DEVICES) g_scratch_ptr[device] = nullptr;
+}
+
+// The arguments of launch_attn_decode without the workspace.  Nothing in the array has to start at zero: every
+// partial a merge reads was written by the attention kernel of the same call (also for splits without pages).
+int launch_attn_decode_noalloc(int device, const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
+                               const int32_t* ctx_len, int max_ctx, const void* gate, int64_t gate_bstride, int64_t gate_hstride,
+                               void* out, float* lse, int batch, int NH, int NKV, int HD, int page_size, int splits) {
+  BK_REQUIRE(device >= 0 && device < NOALLOC_MAX_DEVICES && g_scratch_ptr[device], "attn_decode_noalloc: bk_init has not set up device %d", device);
+  BK_REQUIRE(batch > 0 && NKV > 0 && max_ctx >= 1, "attn_decode_noalloc: bad batch=%d NKV=%d max_ctx=%d", batch, NKV, max_ctx);
+  const int64_t groups = (int64_t)batch * NKV;
+  if (splits <= 0) {
+    // the library's own choice, held to what the array takes (one split needs no partials at all)
+    splits = attn_choose_splits(batch, NKV, max_ctx);
+    if (groups * splits > NOALLOC_MAX_PARTIALS) splits = (int)(NOALLOC_MAX_PARTIALS / groups);
+    if (splits < 1) splits = 1;
+  }
+  const int pages = (max_ctx + ATT_PAGE - 1) / ATT_PAGE;
+  if (splits > pages) splits = pages;
+  BK_REQUIRE(splits == 1 || groups * splits <= NOALLOC_MAX_PARTIALS,
+             "attn_decode_noalloc: batch %d x %d KV heads x %d splits = %lld partial results exceed the %d of the built-in scratch "
+             "(use fewer splits, or bk_attn_decode with a workspace)", batch, NKV, splits, (long long)(groups * splits), NOALLOC_MAX_PARTIALS);
+  return launch_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, 0, 0, max_ctx, gate, gate_bstride, gate_hstride, out, lse,
+                            g_scratch_ptr[device], NOALLOC_SCRATCH_BYTES, batch, NH, NKV, HD, page_size, splits);
+}
+
 // ---------------------------------------------------------------- per-head norm + RoPE + cache append in one launch
 // qnorm -> rope, knorm -> ropek and the cache write (src/emitters.ts:123-183, 202-205) as one kernel:
 // one wavefront per (role, head, sequence).  Query heads go to `qout` (bf16 [B, NH, 256]); the

@@ -10,6 +10,7 @@ enum : int { DT_F32 = 0, DT_BF16 = 1 };
 
 // runtime.hip
 bool inited();
+int current_device();
 bool prof_on();
 int prof_begin(int kernel);
 int prof_end();
@@ -89,6 +90,11 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
                        int NH, int NKV, int HD, int page_size, int splits, void* out_q8 = nullptr, int tpw = 1);
+int attn_noalloc_setup(int device);
+void attn_noalloc_teardown(int device);
+int launch_attn_decode_noalloc(int device, const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
+                               const int32_t* ctx_len, int max_ctx, const void* gate, int64_t gate_bstride, int64_t gate_hstride,
+                               void* out, float* lse, int batch, int NH, int NKV, int HD, int page_size, int splits);
 int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
                      void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size);

@@ -37,6 +37,7 @@ static int sync_all() {
 }
 int num_cus() { return g_cus; }
 bool inited() { return g_inited; }
+int current_device() { return g_device; }
 
 // ---- profiler: an event pair around every bk_launch, summed per kernel label
 struct ProfPending { hipEvent_t a, b; int kernel; };
@@ -100,6 +101,7 @@ int bk_init(int device) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return set_error(BK_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
   g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  if (int rc = attn_noalloc_setup(device)) return rc;      // with `device` current: the address of its built-in scratch array
   BK_HIP(hipStreamCreateWithFlags(&g_main_stream, hipStreamNonBlocking));
   g_stream = g_main_stream;
   g_device = device;
@@ -117,6 +119,7 @@ int bk_shutdown(void) {
   for (hipStream_t st : g_extra_streams) (void)hipStreamDestroy(st);
   g_extra_streams.clear();
   (void)hipStreamDestroy(g_main_stream);
+  attn_noalloc_teardown(g_device);
   g_stream = g_main_stream = nullptr; g_inited = false; g_device = -1;
   return BK_OK;
 }

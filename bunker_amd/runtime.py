@@ -61,6 +61,7 @@ _SIGS = {
     "bk_gdn_core": [u64, u64, u64, u64, u64, u64, u64, u64, i32, i32],
     "bk_attn_plan": [i32, i32, i32, C.POINTER(i32), C.POINTER(u64)],
     "bk_attn_decode": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, u64, u64, i32, i32, i32, i32, i32, i32],
+    "bk_attn_decode_noalloc": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, i32, i32, i32, i32, i32, i32],
     "bk_kv_append": [u64, u64, u64, u64, u64, i32, u64, i32, i32, i32, i32, i32],
 }
 
@@ -449,6 +450,14 @@ def attn_decode(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_
     _check(cu().bk_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, max_ctx, gate, gate_bstride, gate_hstride,
                                out, lse, workspace, workspace_bytes, batch, NH, NKV, HD, page_size, splits),
            "bk_attn_decode")
+
+
+def attn_decode_noalloc(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_len: int, max_ctx: int, out: int,
+                        lse: int, batch: int, NH: int = 16, NKV: int = 2, HD: int = 256, page_size: int = 16, splits: int = 0,
+                        gate: int = 0, gate_bstride: int = 0, gate_hstride: int = 0) -> None:
+    """``attn_decode`` without a workspace: split partials go to the library's fixed per-GPU array (batch * NKV * splits <= 1024)."""
+    _check(cu().bk_attn_decode_noalloc(q, kc, vc, block_table, bt_stride, ctx_len, max_ctx, gate, gate_bstride, gate_hstride,
+                                       out, lse, batch, NH, NKV, HD, page_size, splits), "bk_attn_decode_noalloc")
 
 
 def kv_append(k: int, v: int, kc: int, vc: int, block_table: int, bt_stride: int, pos: int, max_len: int, batch: int,

@@ -194,6 +194,17 @@ BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_t
                           int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
                           uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size,
                           int splits);
+/* bk_attn_decode for callers that cannot allocate device memory or bring a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and same
+ * results (bit for bit, for the same number of splits) as bk_attn_decode, without workspace / workspace_bytes: the
+ * partial results of the splits go to a fixed 16.1 MiB array that each GPU holds from library load to process end.
+ * Limit: batch * NKV * splits <= 1024 partial results; splits = 0 lets the library choose within that limit, an
+ * explicit split count beyond it is refused with an error.  The call allocates and frees nothing.  All calls on a GPU
+ * share the one array: two calls that overlap on that GPU (different streams) race, calls on one stream do not. */
+BK_API int bk_attn_decode_noalloc(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride,
+                                  uint64_t ctx_len, int max_ctx, uint64_t gate, int64_t gate_bstride,
+                                  int64_t gate_hstride, uint64_t out, uint64_t lse, int batch, int NH, int NKV,
+                                  int HD, int page_size, int splits);
 /* The cache write of emitFA2Attn (src/emitters.ts:202-205): k, v bf16 [batch, NKV, 256]
  * of this step go to token pos[b] of every sequence (pos int32 [batch] on the device).
  * max_len is the capacity of a sequence in tokens (at most 16 * bt_stride): a position
