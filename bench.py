@@ -35,11 +35,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant GEMV kernel (gemv_q4k_q8_1_lds_kernel<1,0,4>: the lm_head shape), from two rocprofv3 --pmc runs of
-# `bench.py --sections gemv,calib` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter
-# reads for memcopy_kernel of 175030272 bytes (FETCH_SIZE reads 0.50006 of the bytes: factor 1.99979; WRITE_SIZE factor 1.0).
-# The summary with the per-shape counters is profiles/gemv_q4k_q8_1_decode_shapes.md.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 175699681
+# HBM bytes per launch of every profiled kernel, from rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch,
+# each scaled by what the same counter reads for a plain copy of known size).  One line per kernel and shape:
+# `kernel | shape | traffic bytes per launch | algorithmic bytes per launch`; the summaries beside it give the commands.
+TRAFFIC_TABLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic_per_launch.txt")
+
+
+def measured_traffic(kernel: str, shape: str):
+    """Measured HBM bytes per launch of `kernel` at `shape`, or None when no counter run covers that pair."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                cols = [c.strip() for c in line.split("|")]
+                if len(cols) >= 4 and not line.startswith("#") and cols[0].replace(" ", "") == kernel.replace(" ", "") and cols[1] == shape:
+                    return int(cols[2])
+    except OSError:
+        pass
+    return None
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
 ROTATION_BYTES = 600e6  # every shape rotates through copies of its matrix that add up to at least this much
 
@@ -48,31 +60,128 @@ def gemv_bytes(N, K, batch=1):
     return N * K * 144 // 256 + batch * (K // 32) * 36 + batch * N * 4
 
 
-def cpu_baseline(seconds_target=12.0):
-    """Time the CPU oracle's Q4_K x Q8_1 GEMV (OpenMP) on a bounded sample of the workload."""
+def _host_info():
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"cpu_model": model, "os_cpu_count": os.cpu_count(), "usable_cpus": usable}
+
+
+def _timed(fn, seconds, max_reps=1_000_000):
+    """Repeat fn() for about `seconds`; returns (repetitions, elapsed seconds)."""
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds or reps >= max_reps:
+            return reps, dt
+
+
+def cpu_baseline(decode_inputs=None, seconds_per_op=1.5):
+    """The CPU restatement of the path's ops (the C oracle: the reference's host loops of bench/bench.ts:10-72,
+    prototypes/gdn_gated.ts:67-88, prototypes/fa2_vllm.ts:114-139) timed on this machine's host cores, on bounded samples
+    of the workload: one decode shape or one configuration per op, about `seconds_per_op` seconds each.  A reported
+    baseline, not a target.  The full decode step of the checker is timed on the same run that compares its tokens with the GPU's."""
     from oracle import oracle as orc
     from bunker_amd import synth
 
     orc.build()
-    threads = min(16, os.cpu_count() or 1)
-    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
-    threads = int(os.environ["OMP_NUM_THREADS"])
-    name, N, K = SHAPES[1]
+    host = _host_info()
+    # all-core legs use the CPUs this process may run on, capped by OMP_NUM_THREADS when the machine sets it
+    all_threads = host["usable_cpus"]
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        all_threads = min(all_threads, int(os.environ["OMP_NUM_THREADS"]))
+    host["threads_all_core_legs"] = all_threads
+    bf = synth.f32_to_bf16
     g = synth.rng(1)
+    ops = {}
+
+    # Q8_1 quantizer (packQ8_1, bench/bench.ts:53-72): scalar loop, one thread
+    K = 6144
+    x = g.standard_normal(K * 64).astype(np.float32)            # 64 activation rows of the down projection
+    orc.set_threads(1)
+    reps, dt = _timed(lambda: orc.pack_q8_1(x), seconds_per_op)
+    ops["quantize_q8_1"] = {"threads": 1, "value": round(reps * x.size / dt / 1e6, 1), "unit": "M elements/s",
+                            "GBps_in": round(reps * x.nbytes / dt / 1e9, 3), "sample": f"{reps} x {x.size} f32 values in {dt:.1f} s"}
+
+    # Q4_K x Q8_1 GEMV (qmm, bench/bench.ts:10-38 on super-blocks): gate_up shape, one thread and all cores
+    name, N, K = SHAPES[1]
     W = synth.q4k_random(g, N, K)
     xq = orc.pack_q8_1(g.standard_normal(K).astype(np.float32))
-    orc.gemv_q4k_q8_1(W, xq, N, K, acc64=False)
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        orc.gemv_q4k_q8_1(W, xq, N, K, acc64=False)
-        reps += 1
+    gemv = {}
+    for label, th in (("1_thread", 1), ("all_cores", all_threads)):
+        orc.set_threads(th)
+        reps, dt = _timed(lambda: orc.gemv_q4k_q8_1(W, xq, N, K, acc64=False), seconds_per_op * (2 if th > 1 else 1))
+        gemv[label] = {"threads": th, "value": round(reps * gemv_bytes(N, K) / dt / 1e9, 3), "unit": "GB/s",
+                       "sample": f"{reps} x {name} GEMV (N={N}, K={K}, batch 1) in {dt:.1f} s"}
+    ops["gemv_q4k_q8_1"] = gemv
+    del W
+
+    # gated-DeltaNet step (refGDN, prototypes/gdn_gated.ts:67-88 at T=1): BASELINE configs[2], batch 1, 32 heads
+    Hg = 32
+    S = (g.standard_normal((Hg, 128, 128), dtype=np.float32) * np.float32(0.02))
+    q = bf(g.standard_normal((Hg, 128), dtype=np.float32) / np.float32(11.3)); k = bf(g.standard_normal((Hg, 128), dtype=np.float32) / np.float32(11.3))
+    v = bf(g.standard_normal((Hg, 128), dtype=np.float32))
+    gl = (-np.log1p(np.exp(g.standard_normal(Hg))) * 0.1).astype(np.float32); beta = (1 / (1 + np.exp(-g.standard_normal(Hg)))).astype(np.float32)
+    gdn_bytes = Hg * (2 * 128 * 128 * 4 + 3 * 128 * 2 + 128 * 2 + 8)
+    orc.set_threads(all_threads)
+    reps, dt = _timed(lambda: orc.gdn_core(q, k, v, gl, beta, S, Hg), seconds_per_op)
+    ops["gdn_step"] = {"threads": all_threads, "value": round(reps * gdn_bytes / dt / 1e9, 3), "unit": "GB/s",
+                       "us_per_step": round(dt / reps * 1e6, 1), "sample": f"{reps} x core recurrence, batch 1, 32 heads of 128x128, in {dt:.1f} s"}
+
+    # paged decode attention (refAttn, prototypes/fa2_vllm.ts:114-139 for one query row): BASELINE configs[3], batch 1, L = 4096
+    B, L, NH, NKV, HD = 1, 4096, 16, 2, 256
+    kc, vc, bt, ctx = synth.paged_kv_random(g, B, L)
+    qa = bf(g.standard_normal((B, NH, HD)).astype(np.float32))
+    att_bytes = int(2 * NKV * int(ctx[0]) * HD * 2 + NH * HD * 2 * 2 + NH * 4)
+    reps, dt = _timed(lambda: orc.attn_decode_paged(qa, kc, vc, bt, ctx, B, NH, NKV, HD, 16), seconds_per_op)
+    ops["attn_decode"] = {"threads": all_threads, "value": round(reps * att_bytes / dt / 1e9, 3), "unit": "GB/s",
+                          "us_per_call": round(dt / reps * 1e6, 1), "sample": f"{reps} x batch 1, context {int(ctx[0])} of 4096, 16 q / 2 KV heads, in {dt:.1f} s"}
+
+    out = {"value": gemv["all_cores"]["value"], "unit": "GB/s", "cores": all_threads, "kind": "port",
+           "sample": gemv["all_cores"]["sample"] + f" with the C oracle on {all_threads} OpenMP threads",
+           "host": host, "ops": ops}
+    if decode_inputs:
+        out["decode_step"], parity = decode_parity(decode_inputs, all_threads)
+        return out, parity
+    return out, None
+
+
+def decode_parity(decode_inputs, threads):
+    """The checker decodes the same sequences on its own (timed: the CPU's tok/s for the full step) and its tokens are
+    compared with the GPU's free run.  Every op but attention is equal bit for bit, so a token can differ only where the
+    checker's top-1/top-2 margin is below the logit noise that one-ulp bf16 differences of the attention outputs leave;
+    the step-by-step check that continues from the GPU's attention outputs (tests/test_gpu_model.py) demands equality."""
+    from oracle import oracle as orc
+    from oracle.model_ref import RefModel, free_run_report
+
+    orc.set_threads(threads)
+    D, W = decode_inputs["D"], decode_inputs["W"]
+    timing, parity = {}, {}
+    for key, (S, starts, pos0, toks, vals) in decode_inputs["runs"].items():
+        ref = RefModel(D, W, S, batch=len(starts))
+        steps = toks.shape[0]
+        t0 = time.perf_counter()
+        rt_, rv = ref.decode(starts, pos0, steps)
         dt = time.perf_counter() - t0
-        if dt > seconds_target or reps >= 50000:
-            break
-    gbs = reps * gemv_bytes(N, K) / dt / 1e9
-    return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} x {name} GEMV (N={N}, K={K}, batch 1) with the C oracle, "
-                      f"{dt:.1f} s on {threads} OpenMP threads of the host CPU"}
+        rep = free_run_report(toks, vals, rt_, rv, np.array(ref.margins))
+        rep["mode"] = "free run of both sides; strict step-by-step equality is tests/test_gpu_model.py"
+        parity[key] = rep
+        timing[key] = {"threads": threads, "value": round(steps * len(starts) / dt, 3), "unit": "tok/s",
+                       "sample": f"{steps} steps x {len(starts)} sequence(s) of the synthetic model with the C oracle in {dt:.1f} s"}
+    return timing, parity
 
 
 def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=True):
@@ -84,9 +193,15 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     out = {}
     dev_w = None
     envs = []
+    parity_runs = {}
+    PARITY = {1: ([0], 32), 32: ([0, 13, 31], 16)}       # sequences and steps the checker decodes again on the CPU
     weight_bytes = sum(v.nbytes for k, v in W.items() if v.dtype == np.uint8)
     for B, steps in ((1, steps_bs1), (32, steps_bs32)):
-        S = synth_model.device_state(synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True))
+        S_host = synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True)
+        chk, nchk = PARITY[B]
+        S_chk = {k: np.array(np.asarray(v)[chk], copy=True) for k, v in S_host.items()}
+        S = synth_model.device_state(S_host)
+        del S_host
         g = model.buildModelGraph(D, B)
         env = runner.DecodeEnv(g, W, S, inplace_state=True, device_weights=dev_w)
         envs.append(env)
@@ -105,7 +220,9 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
         rt.cuSync()
         wall = time.perf_counter() - t0
         ms = e0.elapsed_ms(e1) / steps
-        toks, _ = loop.tokens()
+        toks, vals = loop.tokens()
+        nchk = min(nchk, toks.shape[0])
+        parity_runs[f"bs{B}"] = (S_chk, [starts[i] for i in chk], 4096, toks[:nchk][:, chk].copy(), vals[:nchk][:, chk].copy())
         # bytes one step must move: every Q4_K weight once, GDN state read+write, the KV prefix of the FA layers
         n_gdn = sum(1 for l in range(D.NL) if not D.is_full_attention(l))
         n_fa = D.NL - n_gdn
@@ -150,7 +267,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     out["reference_dims"] = {"dims": "hidden 1024, FFN 3584, vocab 248320, 18 GDN + 6 attention layers (src/model.ts:14-18)",
                              "bs1": {"tok_per_s": round(1e3 / ms, 1), "ms_per_step": round(ms, 4), "steps": steps_bs1}}
     envR.close()
-    return out
+    return out, {"D": D, "W": W, "runs": parity_runs}
 
 
 def bench_load(rt, synth):
@@ -434,7 +551,8 @@ def main():
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dom_kernel, "shapes": dom, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH}
+                "avg_launch_us": round(dom_us, 3), "bytes_per_launch": int(dom_bytes),
+                "traffic": measured_traffic(dom_kernel, "+".join(dom))}
 
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak); synthetic Qwen3.5 decode tok/s at bs=1/32",
@@ -466,8 +584,11 @@ def main():
         rt.cuSync()
         rt.cuFree(a); rt.cuFree(b)
         out["calib"] = {"kernel": "memcopy_kernel", "bytes_read": nb, "bytes_written": nb, "launches": 10}
+    decode_inputs = None
     if "decode" in sections:
-        out["decode"] = bench_decode(rt, synth, use_graph=not args.no_graph, fused=not args.unfused)
+        out["decode"], decode_inputs = bench_decode(rt, synth, use_graph=not args.no_graph, fused=not args.unfused)
+        if args.no_cpu_baseline:
+            decode_inputs = None
     if "kernels" in sections:
         out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
     if "gemm" in sections:
@@ -475,7 +596,9 @@ def main():
     if "load" in sections:
         out["weights_path"] = bench_load(rt, synth)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"], parity = cpu_baseline(decode_inputs)
+        for key, rep in (parity or {}).items():
+            out["decode"][key]["argmax_parity"] = rep
     print(json.dumps(out))
 
 

@@ -122,3 +122,31 @@ class RefModel:
             hist_t.append(idx); hist_v.append(val)
             toks, pos = idx, pos + 1
         return np.stack(hist_t), np.stack(hist_v)
+
+
+def free_run_report(got_tokens, got_vals, ref_tokens, ref_vals, margins) -> dict:
+    """Two independent greedy decodes side by side: ``got`` from the implementation under test, ``ref`` and the
+    top-1/top-2 ``margins`` from ``RefModel.decode``.  Arrays are [steps, sequences].
+
+    A sequence is compared up to its first differing token (afterwards the two runs decode different texts).
+    ``noise`` is |winning logit of the implementation - winning logit of the checker| on the compared steps."""
+    got_tokens, ref_tokens = np.asarray(got_tokens), np.asarray(ref_tokens)
+    margins = np.asarray(margins, np.float64).reshape(ref_tokens.shape)
+    noise = np.abs(np.asarray(got_vals, np.float64) - np.asarray(ref_vals, np.float64))
+    steps, nseq = ref_tokens.shape
+    matched, first_div, worst = 0, None, None
+    max_noise, min_margin = 0.0, float("inf")
+    for b in range(nseq):
+        for s in range(steps):
+            if got_tokens[s, b] != ref_tokens[s, b]:
+                seen = float(noise[:s, b].max()) if s else 0.0
+                if first_div is None or s < first_div["step"]:
+                    first_div = {"step": s, "sequence": b, "margin": float(margins[s, b]), "noise_before": seen}
+                break
+            matched += 1
+            max_noise = max(max_noise, float(noise[s, b]))
+            min_margin = min(min_margin, float(margins[s, b]))
+    return {"argmax_match": f"{matched}/{steps * nseq}", "matched": matched, "compared": steps * nseq, "steps": steps,
+            "sequences": nseq, "first_divergence": first_div,
+            "min_margin_on_matched_steps": None if min_margin == float("inf") else round(min_margin, 6),
+            "max_logit_noise_on_matched_steps": round(max_noise, 6)}

@@ -44,11 +44,16 @@
  *   orc_argmax                      prototypes/test_argmax.ts:33-44 vector + ties
  */
 #include <math.h>
+#include <omp.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
 #define ORC_API __attribute__((visibility("default")))
+
+/* Threads the row / head loops below run on (the benchmark's CPU-baseline leg times one thread and all cores). */
+ORC_API void orc_set_threads(int n) { if (n >= 1) omp_set_num_threads(n); }
+ORC_API int orc_max_threads(void) { return omp_get_max_threads(); }
 
 /* ------------------------------------------------------------------ */
 /* scalar conversions                                                   */

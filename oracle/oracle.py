@@ -49,6 +49,15 @@ def lib():
     return _lib
 
 
+def set_threads(n: int) -> None:
+    """OpenMP threads of the row / head loops from now on."""
+    lib().orc_set_threads(int(n))
+
+
+def max_threads() -> int:
+    return int(lib().orc_max_threads())
+
+
 def _p(a):
     return a.ctypes.data_as(C.c_void_p) if a is not None else None
 
