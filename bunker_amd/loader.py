@@ -143,24 +143,32 @@ def loadSafeTensors(path: str, chunk_bytes: int = CHUNK_BYTES) -> SafeTensorsFil
 
 def writeSafeTensors(path: str, tensors: dict, metadata: dict | None = None, align: int = 16) -> None:
     """``tensors``: name -> (dtype string, numpy array holding the raw values; bf16/f16 as uint16 bit patterns).
-    Data offsets are ``align``-byte aligned (16: device views can be read with 16-byte loads; files from other
-    writers pack tensors back to back, which ``align=1`` reproduces)."""
+
+    The format allows no gap between tensors (the published reader rejects a data section with holes), so alignment
+    can only come from the order: with ``align`` > 1 the tensors whose byte size is a multiple of ``align`` are
+    written first (each then starts on an ``align``-byte boundary: device views of them can be read with 16-byte
+    loads), the others behind them by falling power-of-two divisor of their size; ``align=1`` keeps the given order
+    (files from other writers: any element-aligned offset occurs)."""
+    def grain(nbytes: int) -> int:
+        g = 1
+        while g < align and nbytes % (2 * g) == 0:
+            g *= 2
+        return g
+
+    items = [(name, dtype, np.asarray(arr, order="C")) for name, (dtype, arr) in tensors.items()]      # keeps shape ()
+    if align > 1:
+        items.sort(key=lambda it: -grain(it[2].nbytes))           # stable: the given order inside a class
     header, off, blobs = {}, 0, []
-    for name, (dtype, arr) in tensors.items():
-        arr = np.ascontiguousarray(arr)
+    for name, dtype, arr in items:
         if arr.dtype.itemsize != _ST_ITEMSIZE[dtype]:
             raise ValueError(f"'{name}': array item size {arr.dtype.itemsize} does not match dtype {dtype}")
-        pad = (-off) % align
-        if pad:
-            blobs.append(b"\0" * pad)
-            off += pad
         header[name] = {"dtype": dtype, "shape": list(arr.shape), "data_offsets": [off, off + arr.nbytes]}
         blobs.append(arr.tobytes())
         off += arr.nbytes
     if metadata:
         header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
     hj = json.dumps(header, separators=(",", ":")).encode("utf-8")
-    hj += b" " * ((-(8 + len(hj))) % 16)          # keep the data section 16-byte aligned in the file as well
+    hj += b" " * ((-(8 + len(hj))) % 16)          # the data section starts 16-byte aligned in the file
     with open(path, "wb") as f:
         f.write(struct.pack("<Q", len(hj)))
         f.write(hj)

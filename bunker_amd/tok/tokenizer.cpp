@@ -1,5 +1,5 @@
 // Byte-level BPE tokenizer behind the C ABI the reference binds (shim/gigatoken_wrapper/src/lib.rs:19-93, used by
-// prototypes/decode.ts:78-86): gt_init(path to a Hugging Face tokenizer.json) / gt_encode / gt_free.  The reference's
+// prototypes/decode.ts:78-86): gt_init(path to a Hugging Face tokenizer.json) / gt_encode / gt_encode_mt / gt_free.  The reference's
 // wrapper is Rust over the gigatoken crate (a path dependency outside its tree, Cargo.toml:11); this is a C++ restatement
 // of the published algorithm those files implement:
 //   1. added tokens ("added_tokens": content -> id) are cut out of the text first, leftmost-longest;
@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -381,6 +382,46 @@ __attribute__((visibility("default"))) int gt_encode(void* tok, const uint8_t* t
   const size_t n = ids.size() < out_max ? ids.size() : out_max;
   memcpy(out_buf, ids.data(), n * sizeof(uint32_t));
   return (int)n;
+}
+
+// lib.rs:47-88: the text is cut into one chunk per hardware thread, each chunk ending behind the first space at or past
+// its share of the bytes, and the chunks are encoded side by side; a chunk is encoded on its own, so the ids are those
+// of gt_encode over each chunk (a piece that spans a cut is split there, as in the reference).  Returns the number of
+// ids of all chunks together, which may exceed out_max: a chunk whose ids do not fit behind the ones before it is left
+// out.  The reference hands chunks their place in out_buf in the order they finish; here chunk i follows chunk i - 1.
+__attribute__((visibility("default"))) int gt_encode_mt(void* tok, const uint8_t* text, size_t text_len, uint32_t* out_buf, size_t out_max) {
+  if (!tok || !text || !out_buf) return -1;
+  const Tokenizer* t = (const Tokenizer*)tok;
+  size_t n_threads = std::thread::hardware_concurrency();
+  if (n_threads == 0) n_threads = 32;                       // lib.rs:26
+  const size_t chunk_size = (text_len + n_threads - 1) / n_threads;
+  std::vector<std::pair<size_t, size_t>> chunks;            // (start, end)
+  for (size_t s = 0; s < text_len;) {
+    size_t e = s + chunk_size < text_len ? s + chunk_size : text_len;
+    if (e < text_len) {
+      while (e < text_len && text[e] != ' ') e++;
+      if (e < text_len) e++;
+    }
+    chunks.emplace_back(s, e);
+    s = e;
+  }
+  std::vector<std::vector<uint32_t>> ids(chunks.size());
+  std::vector<std::thread> workers;
+  const size_t nw = chunks.size() < n_threads ? chunks.size() : n_threads;
+  for (size_t w = 0; w < nw; w++)
+    workers.emplace_back([&, w] {
+      for (size_t c = w; c < chunks.size(); c += nw) {
+        ids[c].reserve(chunks[c].second - chunks[c].first);
+        t->encode(text + chunks[c].first, chunks[c].second - chunks[c].first, ids[c]);
+      }
+    });
+  for (auto& th : workers) th.join();
+  size_t cursor = 0;
+  for (const auto& v : ids) {
+    if (cursor + v.size() <= out_max) memcpy(out_buf + cursor, v.data(), v.size() * sizeof(uint32_t));
+    cursor += v.size();
+  }
+  return (int)cursor;
 }
 
 // lib.rs:90-93

@@ -100,3 +100,48 @@ def test_init_without_gpu_reports_no_device():
 def test_missing_library_raises():
     with pytest.raises(rt.BunkerError, match="no CPU fallback"):
         rt.load_library("/nonexistent/libbunker_hip.so")
+
+
+ABI_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi")
+
+
+def test_c_driver_compiles_against_the_header():
+    """tests/abi/abi_driver.c is plain C99 over include/bunker_hip.h (-Wall -Wextra -Werror -pedantic): the compiler
+    checks every call against the declarations; without a device the program reports bk_init's error and exits 2."""
+    import subprocess
+    _lib_or_skip()
+    subprocess.check_call(["make", "-C", ABI_DIR, "-B", "abi_driver"], stdout=subprocess.DEVNULL)
+    exe = os.path.join(ABI_DIR, "abi_driver")
+    blob = os.path.join(ABI_DIR, "_empty.bin")
+    try:
+        import numpy as np
+        np.concatenate([np.array([1, 256], np.int32).view(np.uint8), np.zeros(144 + 256 * 4, np.uint8)]).tofile(blob)
+        r = subprocess.run([exe, blob], capture_output=True, text=True, timeout=120)
+    finally:
+        if os.path.exists(blob):
+            os.remove(blob)
+    if r.returncode == 0:
+        assert r.stdout.strip().endswith("ok")            # a GPU is present
+    else:
+        assert r.returncode == 2 and r.stdout.startswith("ERROR: bk_init(0)"), (r.returncode, r.stdout, r.stderr)
+
+
+def test_bun_binding_file_matches_the_header():
+    """ts/hip.ts (the bun:ffi binding a maintainer drops next to src/ttir.ts) lists every function of the header with
+    the FFI type of every parameter; bun cannot run here, so the table is checked as text."""
+    import re
+    ffi = {"int": "i32", "int64_t": "i64", "uint64_t": "u64"}
+    text = open(os.path.join(os.path.dirname(rt.HEADER_PATH), "..", "ts", "hip.ts")).read()
+    table = dict((n, (re.findall(r'"(\w+)"', a), r)) for n, a, r in
+                 re.findall(r'^\s*(bk_\w+):\s*\{ args: \[([^\]]*)\], returns: "(\w+)" \},', text, flags=re.M))
+    protos = _header_prototypes()
+    assert set(table) == set(protos)
+    for name, (ret, params) in protos.items():
+        args, r = table[name]
+        assert r == ("i32" if ret == "int" else "ptr"), name
+        assert args == [ffi.get(p, "ptr") for p in params], (name, args, params)
+    # the names the call sites import from src/ttir.ts are all exported
+    for fn in ("cu", "cuAlloc", "cuHtoD", "cuDtoH", "cuFree", "cuSync", "cuHtoDAsync", "cuDtoHAsync", "cuCopySync",
+               "compileAndLoad", "cuLaunch", "profGpuReset", "profGpuReport"):
+        assert re.search(r"^export function %s\(" % fn, text, flags=re.M), fn
+    assert "export interface LoadedKernel" in text

@@ -71,3 +71,27 @@ def test_argmax_gpu():
         assert int(rt.from_device(dv, (1,), np.uint32)[0]) == c["val_f32_bits"]
         for p in (dl, dv, di):
             rt.cuFree(p)
+
+
+def test_c_driver_reproduces_the_golden_gemv(tmp_path):
+    """The compiled C caller (tests/abi/abi_driver.c: header included, library linked, no Python in between) runs
+    quantize -> GEMV on the golden fixture through the typed entry points and through bk_kernel_create / bk_launch."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi", "abi_driver")
+    assert os.path.exists(exe), "tests/abi/abi_driver is not built: make -C tests/abi"
+    g = gold("gemv_q4k_q8_1.json")
+    N, K = g["N"], g["K"]
+    blob = tmp_path / "in.bin"
+    with open(blob, "wb") as f:
+        f.write(np.array([N, K], np.int32).tobytes())
+        f.write(np.array(g["W_bytes"], np.uint8).tobytes())
+        f.write(bits_f32(g["x_f32_bits"]).tobytes())
+    r = subprocess.run([exe, str(blob)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.stdout[-400:], r.stderr[-400:])
+    lines = dict(l.split(" ", 1) for l in r.stdout.strip().splitlines() if " " in l)
+    assert bytes.fromhex(lines["xq"]) == bytes(g["xq_bytes"])
+    want = [f"{v:08x}" for v in g["y_f32_bits_exact_rounded_once"]]
+    assert lines["y"].split() == want and lines["y_launch"].split() == want
+    assert [int(v, 16) - (1 << 32) if int(v, 16) >> 31 else int(v, 16) for v in lines["subdot0"].split()] == g["subdots_int32"][0]
+    assert "refused" in lines and r.stdout.strip().endswith("ok")

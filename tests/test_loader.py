@@ -111,12 +111,59 @@ def test_safetensors_round_trip(tmp_path):
     raw = open(p, "rb").read()
     for name, (dt, arr) in tensors.items():
         b, e = header[name]["data_offsets"]
-        assert b % 16 == 0 and header[name]["dtype"] == dt and header[name]["shape"] == list(arr.shape)
+        assert header[name]["dtype"] == dt and header[name]["shape"] == list(arr.shape)
+        assert b % 16 == 0 or arr.nbytes % 16           # tensors of whole 16-byte pieces come first, aligned
         assert raw[start + b:start + e] == arr.tobytes()
+    spans = sorted(h["data_offsets"] for h in header.values())        # no gaps: the format allows none
+    assert spans[0][0] == 0 and all(a[1] == b[0] for a, b in zip(spans, spans[1:])) and spans[-1][1] == size - start
     with open(p, "r+b") as f:                       # a header that claims more bytes than the file has
         f.truncate(size - 8)
     with pytest.raises(ValueError):
         loader.readSafeTensorsHeader(p)
+
+
+def test_safetensors_against_the_safetensors_package(tmp_path):
+    """Both directions against the published implementation of the format (the `safetensors` package): a file this
+    writer makes is read back by the package, and a file the package writes (tensors packed back to back, sorted by
+    dtype and name, its own header padding) is parsed by this reader to the same bytes."""
+    st = pytest.importorskip("safetensors")
+    import safetensors.numpy as stnp
+    g = synth.rng(23)
+    f32 = g.standard_normal((5, 3)).astype(np.float32)
+    f16 = g.standard_normal(11).astype(np.float16)
+    i32 = g.integers(-9, 9, (2, 2, 2)).astype(np.int32)
+    one = np.array(3.5, np.float32)                          # a scalar: shape []
+    # ours -> theirs (bf16 is not a numpy dtype: the package reads it through its header only, checked as raw bytes)
+    bfa = bf(g.standard_normal((4, 6)).astype(np.float32))
+    p1 = str(tmp_path / "ours.safetensors")
+    loader.writeSafeTensors(p1, {"x.f32": ("F32", f32), "x.f16": ("F16", f16.view(np.uint16)), "x.i32": ("I32", i32),
+                                 "x.bf16": ("BF16", bfa), "x.one": ("F32", one)}, {"format": "pt", "n": 3})
+    back = stnp.load_file(p1) if not _has_bf16(p1) else None
+    with st.safe_open(p1, framework="numpy") as f:
+        assert set(f.keys()) == {"x.f32", "x.f16", "x.i32", "x.bf16", "x.one"} and f.metadata() == {"format": "pt", "n": "3"}
+        assert np.array_equal(f.get_tensor("x.f32"), f32) and np.array_equal(f.get_tensor("x.f16"), f16)
+        assert np.array_equal(f.get_tensor("x.i32"), i32) and f.get_tensor("x.one").shape == () and f.get_tensor("x.one") == 3.5
+        sl = f.get_slice("x.bf16")
+        assert sl.get_shape() == [4, 6] and sl.get_dtype() == "BF16"
+    assert back is None
+    # theirs -> ours
+    p2 = str(tmp_path / "theirs.safetensors")
+    stnp.save_file({"b.f32": f32, "a.f16": f16, "c.i32": i32, "d.one": one, "e.i64": np.arange(5, dtype=np.int64)}, p2,
+                   metadata={"who": "package"})
+    header, meta, start, size = loader.readSafeTensorsHeader(p2)
+    assert meta == {"who": "package"} and set(header) == {"b.f32", "a.f16", "c.i32", "d.one", "e.i64"}
+    raw = open(p2, "rb").read()
+    want = {"b.f32": ("F32", f32), "a.f16": ("F16", f16), "c.i32": ("I32", i32), "d.one": ("F32", one),
+            "e.i64": ("I64", np.arange(5, dtype=np.int64))}
+    for name, (dt, arr) in want.items():
+        b, e = header[name]["data_offsets"]
+        assert header[name]["dtype"] == dt and header[name]["shape"] == list(arr.shape)
+        assert raw[start + b:start + e] == arr.tobytes(), name
+    assert max(h["data_offsets"][1] for h in header.values()) == size - start       # the data section ends with the file
+
+
+def _has_bf16(path):
+    return any(v.get("dtype") == "BF16" for k, v in loader.readSafeTensorsHeader(path)[0].items())
 
 
 def test_gguf_round_trip(tmp_path):

@@ -84,3 +84,54 @@ def test_abi_errors_and_truncation(tmp_path):
     assert out.tolist() == hf.encode(text.decode()).ids[:3]
     assert lib.gt_encode(None, text, len(text), out.ctypes.data_as(C.c_void_p), 3) == -1
     lib.gt_free(h)
+
+
+def _mt_chunks(data: bytes, n_threads: int):
+    """The cuts of shim/gigatoken_wrapper/src/lib.rs:55-63: equal shares of the bytes, each run on to just behind the next space."""
+    size = (len(data) + n_threads - 1) // n_threads
+    out, s = [], 0
+    while s < len(data):
+        e = min(s + size, len(data))
+        if e < len(data):
+            while e < len(data) and data[e] != 0x20:
+                e += 1
+            if e < len(data):
+                e += 1
+        out.append(data[s:e])
+        s = e
+    return out
+
+
+def test_encode_mt_is_encode_over_space_cut_chunks(tmp_path):
+    import ctypes as C
+    path = str(tmp_path / "tokenizer.json")
+    hf = _train(path, QWEN)
+    t = tokenizer.Tokenizer(path)
+    n_threads = os.cpu_count() or 32
+    docs = [open(os.path.join(ROOT, "bench.py")).read(), "no-spaces-at-all" * 50, "", "a", "a b", " 日本語 한국어 😀 " * 300]
+    for s in docs:
+        data = s.encode("utf-8")
+        want = [i for c in _mt_chunks(data, n_threads) for i in hf.encode(c.decode("utf-8", "ignore")).ids] \
+            if all(_valid_utf8(c) for c in _mt_chunks(data, n_threads)) else None
+        got = t.encode(s, mt=True).tolist()
+        assert got == [i for c in _mt_chunks(data, n_threads) for i in t.encode(c).tolist()], s[:40]
+        if want is not None:
+            assert got == want, s[:40]
+    # a text without spaces is one chunk per share run to the end: the same ids as the single-thread call
+    assert t.encode("no-spaces-at-all" * 50, mt=True).tolist() == t.encode("no-spaces-at-all" * 50).tolist()
+    # the count returned is the total even when it exceeds out_max; chunks that do not fit are left out
+    lib = tokenizer.load_library()
+    text = ("word " * 400).encode()
+    full = t.encode(text, mt=True)
+    small = np.full(5, 0xFFFFFFFF, np.uint32)
+    assert lib.gt_encode_mt(t.h, text, len(text), small.ctypes.data_as(C.c_void_p), 5) == len(full)
+    assert lib.gt_encode_mt(None, text, len(text), small.ctypes.data_as(C.c_void_p), 5) == -1
+    t.close()
+
+
+def _valid_utf8(b: bytes) -> bool:
+    try:
+        b.decode("utf-8")
+        return True
+    except UnicodeDecodeError:
+        return False
