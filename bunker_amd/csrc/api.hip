@@ -241,6 +241,13 @@ static int run_rope(Kernel& k, const uint64_t* s) {
   return launch_rope(P<void>(s[0]), P<float>(s[1]), P<float>(s[2]), dev ? P<int32_t>(s[3]) : nullptr, dev ? 0 : (int)(int32_t)s[3],
                      nh, (int)k.get("HD", 0), (int)k.get("ROT_HALF", 0), (int)k.get("MAX_LEN", 0), (int)k.get("batch", 1));
 }
+// Attention ops: exact=1 (the default) runs the double-precision kernels, whose outputs are the bits of the host loop
+// (prototypes/fa2_vllm.ts:114-139 in doubles); exact=0 the bf16 matrix-instruction kernels (within 2e-2).
+static size_t fa2_qn_bytes(int rows, int NH, int HD) { return ((size_t)rows * NH * HD * 2 + 255) / 256 * 256; }
+static size_t fa2_ws_bytes(int rows, int NKV, int splits, int exact) {
+  if (exact) return attn_exact_workspace_bytes(rows, NKV, splits > 1 ? splits : 0);
+  return splits > 1 ? attn_workspace_bytes(rows, NKV, splits) : 0;
+}
 // ---- op: fa2_attn (src/model.ts:144-157)
 // slots: q, k, v, qgate, kv_k_in, kv_v_in, pos, out, kv_k_new, kv_v_new; like the reference's emitter only
 // kv_*_in are touched (the caller maps in and new to one buffer).  This step's k, v go into the cache at
@@ -258,7 +265,7 @@ static int run_fa2(Kernel& k, const uint64_t* s) {
   // the context of each sequence is its pos + 1
   return launch_attn_decode(P<void>(s[0]), P<void>(s[4]), P<void>(s[5]), nullptr, bt_stride, pos_dev, pos, 1, max_len,
                             P<uint16_t>(s[3]) + HD, (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[7]), nullptr, k.scratch, k.scratch_bytes,
-                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0));
+                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, 1, (int)k.get("exact", 1));
 }
 // ---- op: fa2_fused = qnorm, rope, knorm, ropek, fa2_attn of src/model.ts:126-157 as three launches
 // (norm + rotation + cache append; split attention; merge with the output gate).
@@ -270,14 +277,19 @@ static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   const int max_len = (int)k.get("MAX_LEN", 0), bt_stride = (max_len + 15) / 16, half = (int)k.get("ROT_HALF", 0);
   const int32_t* pos_dev = dev ? P<int32_t>(s[7]) : nullptr;
   const int pos = dev ? 0 : (int)(int32_t)s[7];
-  void* qn = k.scratch;                                              // bf16 [batch, NH, HD]
-  void* ws = (uint8_t*)k.scratch + (size_t)batch * NH * HD * 2;
+  // workspace: normalised, rotated q as bf16 [batch, NH, HD]; exact=1: the same as f64 [batch, NKV, HD, 8] (written by the
+  // prep kernel, unused columns stay zero from creation); then the partials of the splits
+  const int exact = (int)k.get("exact", 1);
+  const size_t qn_bytes = fa2_qn_bytes(batch, NH, HD), qf_bytes = exact ? attn_exact_qf_bytes(batch, NKV) : 0;
+  void* qn = k.scratch;
+  double* qf = exact ? (double*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
+  void* ws = (uint8_t*)k.scratch + qn_bytes + qf_bytes;
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
-                            pos_dev, pos, half, max_len, qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, batch, NH, NKV, HD, 16);
+                            pos_dev, pos, half, max_len, qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, batch, NH, NKV, HD, 16, qf);
   if (rc) return rc;
   return launch_attn_decode(qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, pos_dev, pos, 1, max_len, P<uint16_t>(s[0]) + HD,
-                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - (size_t)batch * NH * HD * 2,
-                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0), k.get("q8out", 0) ? P<void>(s[11]) : nullptr);
+                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - qn_bytes - qf_bytes,
+                            batch, NH, NKV, HD, 16, (int)k.get("splits", 0), k.get("q8out", 0) ? P<void>(s[11]) : nullptr, 1, exact, qf);
 }
 // ---- prefill ops: T consecutive tokens of ONE sequence per launch (rows of the activation buffers = tokens)
 // conv1d_prefill   slots: qkv [T, QKVD], conv_state_in [3, QKVD], weight, out [T, QKVD], conv_state_new    params: QKVD, T
@@ -301,14 +313,17 @@ static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
   const int32_t* pos = P<int32_t>(s[7]);
   const int32_t* table = P<int32_t>(s[8]);
   BK_REQUIRE(pos && table, "fa2_prefill: null position or block table pointer");
+  const int exact = (int)k.get("exact", 1);
+  const size_t qn_bytes = fa2_qn_bytes(T, NH, HD), qf_bytes = exact ? attn_exact_qf_bytes(T, NKV) : 0;
   void* qn = k.scratch;
-  void* ws = (uint8_t*)k.scratch + (size_t)T * NH * HD * 2;
+  double* qf = exact ? (double*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
+  void* ws = (uint8_t*)k.scratch + qn_bytes + qf_bytes;
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
-                            pos, 0, half, max_len, qn, P<void>(s[9]), P<void>(s[10]), table, 0, T, NH, NKV, HD, 16);
+                            pos, 0, half, max_len, qn, P<void>(s[9]), P<void>(s[10]), table, 0, T, NH, NKV, HD, 16, qf);
   if (rc) return rc;
   return launch_attn_decode(qn, P<void>(s[9]), P<void>(s[10]), table, 0, pos, 0, 1, max_len, P<uint16_t>(s[0]) + HD,
-                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - (size_t)T * NH * HD * 2,
-                            T, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, k.get("pair", 0) ? 2 : 1);
+                            (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - qn_bytes - qf_bytes,
+                            T, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, k.get("pair", 0) ? 2 : 1, exact, qf);
 }
 
 // ---- op: argmax (src/model.ts:198-201)   slots: logits, val, idx     params: VOCAB, batch=1
@@ -356,7 +371,9 @@ static int build_kernel(Kernel& k) {
     BK_REQUIRE(max_len % 16 == 0, "fa2_attn: MAX_LEN=%d must be a multiple of the 16-token page (a sequence owns MAX_LEN/16 pages)", max_len);
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
-    if (splits > 1 && (rc = alloc_scratch(k, attn_workspace_bytes(batch, NKV, splits)))) return rc;
+    const int exact = (int)k.get("exact", 1);
+    BK_REQUIRE(!exact || k.get("NH", 0) / NKV <= 8, "fa2_attn: exact=1 serves at most 8 query heads per KV head (exact=0 takes 16)");
+    if ((splits > 1 || exact) && (rc = alloc_scratch(k, fa2_ws_bytes(batch, NKV, splits, exact)))) return rc;
     k.run = run_fa2; k.nslots = 10;
     return BK_OK;
   }
@@ -367,8 +384,11 @@ static int build_kernel(Kernel& k) {
     BK_REQUIRE(max_len % 16 == 0, "fa2_fused: MAX_LEN=%d must be a multiple of the 16-token page (a sequence owns MAX_LEN/16 pages)", max_len);
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits(batch, NKV, max_len); k.p["splits"] = splits; }
-    const size_t qbytes = (size_t)batch * k.get("NH", 0) * k.get("HD", 0) * 2;
-    if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(batch, NKV, splits) : 0)))) return rc;
+    const int exact = (int)k.get("exact", 1);
+    BK_REQUIRE(!exact || k.get("NH", 0) / NKV <= 8, "fa2_fused: exact=1 serves at most 8 query heads per KV head (exact=0 takes 16)");
+    const size_t qbytes = fa2_qn_bytes(batch, (int)k.get("NH", 0), (int)k.get("HD", 0));
+    if ((rc = alloc_scratch(k, qbytes + fa2_ws_bytes(batch, NKV, splits, exact)))) return rc;
+    if (exact) BK_HIP(hipMemset(k.scratch, 0, k.scratch_bytes));        // columns of the f64 query copy past the group stay zero
     k.run = run_fa2_fused; k.nslots = 11 + (k.get("q8out", 0) ? 1 : 0);
     return BK_OK;
   }
@@ -391,12 +411,16 @@ static int build_kernel(Kernel& k) {
     BK_REQUIRE(T >= 1 && T <= 65535 && NKV >= 1 && max_len >= 1 && max_len % 16 == 0, "fa2_prefill: bad T/NKV/MAX_LEN (MAX_LEN a multiple of 16)");
     // two consecutive tokens per workgroup where their heads fit the 16 columns of the products (pair=0 switches it off)
     const int NHq = (int)k.get("NH", 0);
-    const int tpw = (NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
+    const int exact = (int)k.get("exact", 1);
+    BK_REQUIRE(!exact || NHq / NKV <= 8, "fa2_prefill: exact=1 serves at most 8 query heads per KV head (exact=0 takes 16)");
+    // (the double-precision kernel takes one token per workgroup)
+    const int tpw = (!exact && NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
     k.p["pair"] = tpw == 2;
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits((T + tpw - 1) / tpw, NKV, max_len); k.p["splits"] = splits; }
-    const size_t qbytes = (size_t)T * k.get("NH", 0) * k.get("HD", 0) * 2;
-    if ((rc = alloc_scratch(k, qbytes + (splits > 1 ? attn_workspace_bytes(T, NKV, splits) : 0)))) return rc;
+    const size_t qbytes = fa2_qn_bytes(T, (int)k.get("NH", 0), (int)k.get("HD", 0));
+    if ((rc = alloc_scratch(k, qbytes + fa2_ws_bytes(T, NKV, splits, exact)))) return rc;
+    if (exact) BK_HIP(hipMemset(k.scratch, 0, k.scratch_bytes));
     k.run = run_fa2_prefill; k.nslots = 12;
     return BK_OK;
   }
@@ -593,6 +617,26 @@ int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, i
   return launch_attn_decode(P<void>(q), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride, P<int32_t>(ctx_len), 0, 0,
                             max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse), P<void>(workspace),
                             (size_t)workspace_bytes, batch, NH, NKV, HD, page_size, splits);
+}
+int bk_attn_plan_exact(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes) {
+  BK_NEED_INIT();
+  BK_REQUIRE(splits && workspace_bytes, "bk_attn_plan_exact: null out");
+  BK_REQUIRE(batch > 0 && NKV > 0 && max_ctx > 0, "bk_attn_plan_exact: bad shape");
+  int s = *splits > 0 ? *splits : attn_choose_splits(batch, NKV, max_ctx);
+  const int pages = (max_ctx + 15) / 16;
+  if (s > pages) s = pages;
+  *splits = s;
+  *workspace_bytes = attn_exact_workspace_bytes(batch, NKV, s > 1 ? s : 0);
+  return BK_OK;
+}
+int bk_attn_decode_exact(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t ctx_len, int max_ctx,
+                         uint64_t gate, int64_t gate_bstride, int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
+                         uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size, int splits) {
+  BK_NEED_INIT();
+  BK_REQUIRE(ctx_len, "bk_attn_decode_exact: ctx_len is required");
+  return launch_attn_decode(P<void>(q), P<void>(kc), P<void>(vc), P<int32_t>(block_table), bt_stride, P<int32_t>(ctx_len), 0, 0,
+                            max_ctx, P<void>(gate), gate_bstride, gate_hstride, P<void>(out), P<float>(lse), P<void>(workspace),
+                            (size_t)workspace_bytes, batch, NH, NKV, HD, page_size, splits, nullptr, 1, 1, nullptr);
 }
 int bk_attn_decode_noalloc(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride, uint64_t ctx_len, int max_ctx,
                            uint64_t gate, int64_t gate_bstride, int64_t gate_hstride, uint64_t out, uint64_t lse, int batch, int NH,

@@ -33,86 +33,9 @@
 //    ceil(total pages / slots) pages, up to a rounding allowance; the first workgroup of a sequence leaves (first slot,
 //    splits) for the merge kernel.
 // With every length at the bound both give the page ranges of the plain form and the same bits.
-#include "ops.h"
+#include "attn_args.h"
 
 namespace bk {
-
-constexpr int ATT_HD = 256;
-constexpr int ATT_PAGE = 16;
-constexpr int ATT_WAVES = 4;
-constexpr int ATT_MAX_PPS = 1024;     // pages per split (the split's page table is staged in LDS)
-constexpr int ATT_MAX_SPLITS = 256;
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) short short4_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_nt;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_nt;
-
-struct AttnArgs {
-  const uint16_t* q;          // bf16 [B, NH, 256]
-  const uint16_t* kc;         // K pages
-  const uint16_t* vc;         // V pages (dim-major inside a page)
-  const int32_t* block_table; // int32 [B, bt_stride]; null = identity (page i of sequence b is b*bt_stride + i)
-  const int32_t* ctx_len;     // int32 [B]; null = ctx_scalar for every sequence; ctx_add is added to either
-  const uint16_t* gate;       // bf16 or null: gate of (b, head, i) at gate[b*gate_bstride + head*gate_hstride + i]
-  uint16_t* out;              // bf16 [B, NH, 256]
-  uint8_t* out_q8;            // optional: the same outputs as Q8_1 blocks [B, NH*256/32] (written by the merge kernel)
-  float* lse;                 // f32 [B, NH] or null
-  float* part_o;              // f32 [B, NKV, splits, 16, 256] unnormalised partial outputs
-  float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
-  int2* plan;                 // balanced form: (first slot, number of splits) of every sequence, behind the partials
-  int64_t gate_bstride, gate_hstride;
-  int bt_stride, ctx_scalar, ctx_add, NH, NKV, G, splits, pages_per_split;
-  int tpw, rows;              // query rows per workgroup (1, or 2 consecutive rows of one sequence: prompt tokens), rows in all
-  int max_pages;              // pages of the longest context the caller allows
-  int rel;                    // 1: lengths in device memory, every sequence cuts its own pages into `splits` equal ranges
-  int slots;                  // > 0: balanced form, this many workgroup slots per KV head shared by the rows (rows <= 64)
-  float scale;
-};
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
-}
-
-// ceil(a / b) for 0 <= a < 2^24, b >= 1, inv_b ~ 1 / b: the float quotient is off by less than one, the remainder settles it
-__device__ __forceinline__ int ceil_div_rcp(int a, int b, float inv_b) {
-  int q = (int)((float)a * inv_b);
-  int r = a - q * b;
-  if (r < 0) { q -= 1; r += b; }
-  if (r >= b) { q += 1; r -= b; }
-  return q + (r > 0 ? 1 : 0);
-}
-
-// Balanced plan, computed by every wave for itself: lane i < rows holds sequence i's pages `np`, its number of splits
-// `ns` and the first slot `first` of its splits.  The page budget of a slot is ceil(total / slots); when the round-up
-// of the sequences' split counts does not fit the slots, it is taken for rows - 1 slots fewer, which always fits
-// (sum ceil(np_i / t) <= total / t + rows - rows / t).  Sums and the prefix sum stay in the lanes (DPP), no LDS.
-__device__ __forceinline__ void attn_balanced_plan(const AttnArgs& A, int lane, int& np, int& ns, int& first) {
-  // a length outside 1 .. max_ctx (the caller's mistake) still plans inside the block table and the slots
-  np = lane < A.rows ? min(max((A.ctx_len[lane] + A.ctx_add + ATT_PAGE - 1) / ATT_PAGE, 1), A.max_pages) : 0;
-  const int t16 = row16_sum_i32(np);
-  const int total = (__builtin_amdgcn_readlane(t16, 0) + __builtin_amdgcn_readlane(t16, 16)) +
-                    (__builtin_amdgcn_readlane(t16, 32) + __builtin_amdgcn_readlane(t16, 48));
-  int incl = 0;
-  for (int attempt = 0; attempt < 2; attempt++) {
-    const int over = attempt ? A.slots - (A.rows - 1) : A.slots;
-    const int budget = ceil_div_rcp(total, over, __builtin_amdgcn_rcpf((float)over));
-    ns = ceil_div_rcp(np, budget, __builtin_amdgcn_rcpf((float)budget));
-    // inclusive prefix sum: inside each row of 16 lanes by row shifts (lanes without a source read 0), then the rows before
-    int v = ns;
-    v += dpp_i32<0x111>(v);      // row_shr:1
-    v += dpp_i32<0x112>(v);      // row_shr:2
-    v += dpp_i32<0x114>(v);      // row_shr:4
-    v += dpp_i32<0x118>(v);      // row_shr:8
-    const int r0 = __builtin_amdgcn_readlane(v, 15), r1 = __builtin_amdgcn_readlane(v, 31), r2 = __builtin_amdgcn_readlane(v, 47);
-    const int row = lane >> 4;
-    incl = v + (row == 0 ? 0 : row == 1 ? r0 : row == 2 ? r0 + r1 : r0 + r1 + r2);
-    const int used = r0 + r1 + r2 + __builtin_amdgcn_readlane(v, 63);
-    if (used <= A.slots) break;
-  }
-  first = incl - ns;
-}
 
 // PF = pages a wave requests ahead of the one it computes on (0 or 2).  Loads are issued
 // unconditionally (past its last page a wave requests a few fixed, cached lines instead), so the number of loads in
@@ -124,21 +47,9 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   __shared__ int lds_bt[ATT_MAX_PPS];           // physical page of every page of this split
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int split = blockIdx.x, b = blockIdx.z;       // b: workgroup's first query row is b * tpw
+  int split, b, p_begin, p_end;                 // b: workgroup's first query row is b * tpw
+  if (!attn_wg_range(A, lane, b, split, p_begin, p_end)) return;
   const int kvh = blockIdx.y;
-  int pps = A.pages_per_split;
-  if (A.slots > 0) {                            // balanced form: slot blockIdx.x belongs to the sequence whose range holds it
-    int np, ns, first;
-    attn_balanced_plan(A, lane, np, ns, first);
-    const unsigned long long own = __ballot((int)blockIdx.x >= first && (int)blockIdx.x < first + ns);
-    if (own == 0) return;                       // a slot past the last one in use (the whole workgroup leaves)
-    b = __ffsll(own) - 1;
-    split = blockIdx.x - __builtin_amdgcn_readlane(first, b);
-    const int nsb = __builtin_amdgcn_readlane(ns, b);
-    pps = ceil_div_rcp(__builtin_amdgcn_readlane(np, b), nsb, __builtin_amdgcn_rcpf((float)nsb));
-    // the merge kernel finds the sequence's partials through this pair
-    if (split == 0 && kvh == 0 && threadIdx.x == 0) A.plan[b] = make_int2(blockIdx.x, nsb);
-  }
   const int n = lane & 15, kg = lane >> 4;      // n: token (A operand) / head (B operand, C column); kg: lane group
   // column n of the products: head n % G of query row b * tpw + n / G; a row past the last one repeats the first (not stored)
   const int row0 = b * A.tpw;
@@ -147,12 +58,6 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   const bool col_valid = tk_n < ntk;
   const int row_n = row0 + (col_valid ? tk_n : 0);
   const int len = (A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add;       // of this lane's column
-  int len_max = (A.ctx_len ? A.ctx_len[row0] : A.ctx_scalar) + A.ctx_add;
-  if (ntk > 1) len_max = max(len_max, A.ctx_len[row0 + 1] + A.ctx_add);
-  const int npages = min((len_max + ATT_PAGE - 1) / ATT_PAGE, A.max_pages);
-  if (A.rel) pps = ceil_div_rcp(npages, A.splits, __builtin_amdgcn_rcpf((float)A.splits));   // equal parts of its own context
-  const int p_begin = split * pps;
-  const int p_end = min(npages, p_begin + pps);
 
   // Q as the B operand of the first product: lane (column n, group kg) holds dims 32*s + 8*kg .. +8
   uint4 qreg[8];
@@ -418,7 +323,7 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw) {
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw, int exact, const double* qf_ready) {
   BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
@@ -461,6 +366,18 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
     else if (pages < (1 << 24)) A.rel = 1;
   }
   A.scale = (float)(1.0 / sqrt((double)HD));
+  // A cache read that is larger than what the memory-side cache can still hold when the next token comes round (decode
+  // at large batch x context) bypasses the caches; prompt rows re-read the same pages and keep the plain loads.
+  const bool nt = g_tune_attn_nt >= 0 ? g_tune_attn_nt != 0
+                                      : (tpw == 1 && (int64_t)batch * NKV * max_ctx * ATT_HD * 4 >= ((int64_t)128 << 20));
+  const dim3 grid(A.slots > 0 ? A.slots : splits, NKV, A.slots > 0 ? 1 : groups), block(ATT_WAVES * 64);
+  if (exact) {
+    // double-precision form: same cut of the pages, its own kernels and workspace layout
+    int rc = launch_attn_exact(A, q, qf_ready, workspace, workspace_bytes, nt, grid, batch);
+    if (rc) return rc;
+    if (splits == 1 && out_q8) return launch_quantize_q8_1(out, DT_BF16, out_q8, NH * HD, batch);
+    return BK_OK;
+  }
   if (splits > 1) {
     BK_REQUIRE(workspace && workspace_bytes >= attn_workspace_bytes(batch, NKV, splits),
                "attn_decode: workspace of %zu bytes needed for %d splits", attn_workspace_bytes(batch, NKV, splits), splits);
@@ -469,11 +386,6 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
     A.plan = (int2*)(A.part_ml + (size_t)batch * NKV * splits * 16 * 2);
   }
   // waves with three pages or more keep two pages in flight ahead of the one they work on
-  // A cache read that is larger than what the memory-side cache can still hold when the next token comes round (decode
-  // at large batch x context) bypasses the caches; prompt rows re-read the same pages and keep the plain loads.
-  const bool nt = g_tune_attn_nt >= 0 ? g_tune_attn_nt != 0
-                                      : (tpw == 1 && (int64_t)batch * NKV * max_ctx * ATT_HD * 4 >= ((int64_t)128 << 20));
-  const dim3 grid(A.slots > 0 ? A.slots : splits, NKV, A.slots > 0 ? 1 : groups), block(ATT_WAVES * 64);
   if (A.pages_per_split >= 3 * ATT_WAVES) {
     if (nt) hipLaunchKernelGGL((attn_decode_kernel<2, true>), grid, block, 0, stream(), A);
     else hipLaunchKernelGGL((attn_decode_kernel<2, false>), grid, block, 0, stream(), A);
@@ -533,7 +445,7 @@ int launch_attn_decode_noalloc(int device, const void* q, const void* kc, const 
              "attn_decode_noalloc: batch %d x %d KV heads x %d splits = %lld partial results exceed the %d of the built-in scratch "
              "(use fewer splits, or bk_attn_decode with a workspace)", batch, NKV, splits, (long long)(groups * splits), NOALLOC_MAX_PARTIALS);
   return launch_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, 0, 0, max_ctx, gate, gate_bstride, gate_hstride, out, lse,
-                            g_scratch_ptr[device], NOALLOC_SCRATCH_BYTES, batch, NH, NKV, HD, page_size, splits);
+                            g_scratch_ptr[device], NOALLOC_SCRATCH_BYTES, batch, NH, NKV, HD, page_size, splits, nullptr, 1, 0, nullptr);
 }
 
 // ---------------------------------------------------------------- per-head norm + RoPE + cache append in one launch
@@ -549,6 +461,7 @@ struct PrepArgs {
   const float *cos_t, *sin_t;      // f32 [max_len, half]
   const int32_t* pos_dev; int pos_scalar;
   uint16_t *qout, *kc, *vc;
+  double* qf;                      // optional: the query heads also as f64 [B, NKV, 256, 8] for the double-precision attention
   const int32_t* block_table; int bt_stride;
   int NH, NKV, half, max_len;
 };
@@ -600,12 +513,16 @@ __global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs A) {
                    : f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, sn)));
     }
     dst[i] = o;
+    if (is_q && A.qf) {
+      const int G = A.NH / A.NKV;
+      A.qf[(((int64_t)b * A.NKV + role / G) * ATT_HD + i) * 8 + role % G] = (double)bf16_to_f32(o);
+    }
   }
 }
 
 int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
-                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size) {
+                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size, double* qf) {
   BK_REQUIRE(qg && k && v && qw && kw && cos_t && sin_t && qout && kc && vc, "attn_prep: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_prep: head_dim 256 and 16-token pages only");
   BK_REQUIRE(batch > 0 && batch <= 65535 && NH > 0 && NKV > 0 && half > 0 && 2 * half <= HD, "attn_prep: bad shape");
@@ -618,6 +535,8 @@ int launch_attn_prep(const void* qg, const void* k, const void* v, const void* q
   A.cos_t = cos_t; A.sin_t = sin_t; A.pos_dev = pos_dev; A.pos_scalar = pos_scalar;
   A.qout = (uint16_t*)qout; A.kc = (uint16_t*)kc; A.vc = (uint16_t*)vc; A.block_table = block_table; A.bt_stride = bt_stride;
   A.NH = NH; A.NKV = NKV; A.half = half; A.max_len = max_len;
+  BK_REQUIRE(!qf || (NH % NKV == 0 && NH / NKV <= 8), "attn_prep: the f64 query copy serves groups of at most 8 heads");
+  A.qf = qf;
   hipLaunchKernelGGL(attn_prep_kernel, dim3(NH + 2 * NKV, batch), dim3(64), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;

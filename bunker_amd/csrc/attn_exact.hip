@@ -1,0 +1,341 @@
+// Decode attention in double precision: the same split-K, paged, grouped-query attention as attn.hip, with every
+// product and sum carried in f64, so that the result is the correctly rounded value of the mathematical expression
+// (up to ~1e-15 relative before the single rounding to f32) and therefore the same bf16 bits as the host loop of
+// prototypes/fa2_vllm.ts:114-139 evaluated in JavaScript numbers (doubles) — whatever the split count, the tile
+// order or the batch.  bf16 x bf16 products are exact in f64; the order of the additions only moves the ~1e-16 tail.
+//
+// A workgroup (8 waves) walks its page range in tiles of 64 tokens (4 pages):
+//   1. the K rows of the tile go to LDS (coalesced 16-byte loads, one page per round of the 512 threads);
+//   2. scores: lane = token, wave = 32 of the 256 dims.  The lane converts its 32 K values to f64 once and multiplies
+//      each into the 8 query heads of the group; the query values are wave-uniform and come through the scalar
+//      unit (s_load from the f64 copy of q) as the SGPR operand of v_fmac_f64 — no cross-lane reduction, the
+//      conversions are shared by the 8 heads.  The 8 partial sums per (head, token) meet through LDS in wave order;
+//   3. weights: wave = head.  p = exp(s - ref) in f64; `ref` is a reference exponent per head, set from the first
+//      tile's maximum and moved only when a score exceeds it by more than 600 (f64 has the range: no running-max
+//      rescale per tile), the sum of p is kept per lane;
+//   4. values: wave = 8 tokens of the tile, lane = 4 of the 256 dims (V pages are dim-major, so a lane's 8 tokens are
+//      one 16-byte load and the wave's loads are contiguous); p is read from LDS at a wave-uniform address.
+// The waves' accumulators are added in a fixed tree through LDS; partials of the splits are f64 and a second
+// kernel merges them.  Roughly 90 vector instructions per (token, KV head), three quarters of them f64 FMAs.
+#include "attn_args.h"
+
+namespace bk {
+
+constexpr int EX_WAVES = 8;
+constexpr int EX_THREADS = EX_WAVES * 64;
+constexpr int EX_TILE = 64;                       // tokens per tile = 4 pages
+constexpr int EX_TILE_PAGES = EX_TILE / ATT_PAGE;
+constexpr int EX_COLS = 8;                        // query heads per KV head served by one workgroup
+constexpr int EX_KROW = ATT_HD * 2 + 16;          // bytes of a K row in LDS: 16 bytes of padding spread the rows over the banks
+constexpr double EX_REF_SLACK = 600.0;            // exp() of up to this much above the reference exponent stays far from overflow
+
+typedef const double __attribute__((address_space(4)))* cdptr_t;      // loads through this pointer may use the scalar unit
+
+__device__ __forceinline__ double bf16lo_to_f64(uint32_t w) { return (double)__uint_as_float(w << 16); }
+__device__ __forceinline__ double bf16hi_to_f64(uint32_t w) { return (double)__uint_as_float(w & 0xffff0000u); }
+
+template <bool NT>
+__global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
+  // K tile (33792 bytes) and the exchange buffer of the partial scores (8 waves x 8 heads x 64 tokens x 8 = 32768 bytes);
+  // the same memory carries the accumulator tree at the end (4 waves x 8 x 256 doubles = 65536 bytes)
+  __shared__ __align__(16) unsigned char lds_raw[EX_TILE * EX_KROW + EX_WAVES * EX_COLS * EX_TILE * 8];
+  __shared__ __align__(16) double lds_p[EX_COLS][EX_TILE];
+  __shared__ double lds_alpha[EX_COLS], lds_m[EX_COLS], lds_l[EX_COLS];
+  __shared__ int lds_bt[ATT_MAX_PPS];
+  unsigned char* ktile = lds_raw;
+  double (*xch)[EX_COLS][EX_TILE] = (double (*)[EX_COLS][EX_TILE])(lds_raw + EX_TILE * EX_KROW);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int split, b, p_begin, p_end;
+  if (!attn_wg_range(A, lane, b, split, p_begin, p_end)) return;
+  const int row = __builtin_amdgcn_readfirstlane(b);          // one query row per workgroup (tpw = 1)
+  const int kvh = blockIdx.y;
+  const int len = (A.ctx_len ? A.ctx_len[row] : A.ctx_scalar) + A.ctx_add;
+  const int lim = min(len, p_end * ATT_PAGE);                  // tokens of this split end here
+  const int npg = max(p_end - p_begin, 0);
+  const int ntiles = (npg + EX_TILE_PAGES - 1) / EX_TILE_PAGES;
+
+  for (int i = threadIdx.x; i < npg; i += EX_THREADS)
+    lds_bt[i] = A.block_table ? A.block_table[(int64_t)row * A.bt_stride + p_begin + i] : row * A.bt_stride + p_begin + i;
+  __syncthreads();
+
+  // a page past the range (the last tile may be short) reads the last page again; its tokens are masked below
+  auto page_base = [&](int i) -> int64_t { return ((int64_t)lds_bt[min(i, npg - 1)] * A.NKV + kvh) * (ATT_PAGE * ATT_HD); };
+  auto ld16 = [&](const uint16_t* p) -> uint4 {
+    const u32x4_nt* p4 = (const u32x4_nt*)p;
+    const u32x4_nt t4 = NT ? __builtin_nontemporal_load(p4) : *p4;
+    return make_uint4(t4[0], t4[1], t4[2], t4[3]);
+  };
+  auto load_k = [&](int tile, uint4 (&kr)[EX_TILE_PAGES]) {        // round r of the 512 threads covers page r of the tile (8 KiB)
+#pragma unroll
+    for (int r = 0; r < EX_TILE_PAGES; r++) kr[r] = ld16(A.kc + page_base(tile * EX_TILE_PAGES + r) + threadIdx.x * 8);
+  };
+  auto load_v = [&](int tile, uint4 (&vr)[4]) {                    // wave: tokens 8 * wave .. + 8 of the tile; lane: dims lane + 64 j
+    const int64_t base = page_base(tile * EX_TILE_PAGES + (wave >> 1)) + (wave & 1) * 8;
+#pragma unroll
+    for (int j = 0; j < 4; j++) vr[j] = ld16(A.vc + base + (lane + 64 * j) * ATT_PAGE);
+  };
+
+  uintptr_t q_addr = (uintptr_t)(A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + wave * 32) * EX_COLS);
+
+  double acc[EX_COLS][4];
+#pragma unroll
+  for (int c = 0; c < EX_COLS; c++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[c][j] = 0.0;
+  double l_lane = 0.0;            // wave = head: this lane's share of the sum of weights
+  double mref = -INFINITY;        // wave = head: the reference exponent
+
+  uint4 kpre[EX_TILE_PAGES], vcur[4];
+  if (ntiles > 0) load_k(0, kpre);
+  for (int tile = 0; tile < ntiles; tile++) {
+#pragma unroll
+    for (int r = 0; r < EX_TILE_PAGES; r++)
+      *(uint4*)(ktile + (r * ATT_PAGE + (threadIdx.x >> 5)) * EX_KROW + (threadIdx.x & 31) * 16) = kpre[r];
+    __syncthreads();
+    load_v(tile, vcur);
+    if (tile + 1 < ntiles) load_k(tile + 1, kpre);
+
+    // ---- scores: lane = token, this wave's 32 dims
+    {
+      // the query values are read again in every tile (they stay in the scalar cache): kept across tiles they would
+      // need 512 scalar registers, so the address is made opaque to keep the loads inside the loop
+      asm volatile("" : "+s"(q_addr));
+      cdptr_t q = (cdptr_t)q_addr;
+      double sacc[EX_COLS];
+#pragma unroll
+      for (int c = 0; c < EX_COLS; c++) sacc[c] = 0.0;
+      const uint4* krow = (const uint4*)(ktile + lane * EX_KROW + wave * 64);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint4 kk = krow[i];
+        const uint32_t w[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) {
+          const double k0 = bf16lo_to_f64(w[wi]), k1 = bf16hi_to_f64(w[wi]);
+          const int d = i * 8 + wi * 2;
+#pragma unroll
+          for (int c = 0; c < EX_COLS; c++) sacc[c] = fma(k0, q[d * EX_COLS + c], sacc[c]);
+#pragma unroll
+          for (int c = 0; c < EX_COLS; c++) sacc[c] = fma(k1, q[(d + 1) * EX_COLS + c], sacc[c]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < EX_COLS; c++) xch[wave][c][lane] = sacc[c];
+    }
+    __syncthreads();
+
+    // ---- weights: wave = head
+    {
+      double s = 0.0;
+#pragma unroll
+      for (int w2 = 0; w2 < EX_WAVES; w2++) s += xch[w2][wave][lane];
+      s *= (double)A.scale;
+      const int tok = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + lane;
+      const bool valid = tok < lim;
+      const float smax = wave_max(valid ? (float)s : -INFINITY);
+      double alpha = 1.0;
+      if (smax > -INFINITY && (mref == -INFINITY || (double)smax > mref + EX_REF_SLACK)) {      // wave-uniform, rare after the first tile
+        if (mref != -INFINITY) { alpha = exp(mref - (double)smax); l_lane *= alpha; }
+        mref = (double)smax;
+      }
+      const double p = valid ? exp(s - mref) : 0.0;
+      l_lane += p;
+      lds_p[wave][lane] = p;
+      if (lane == 0) lds_alpha[wave] = alpha;
+    }
+    __syncthreads();
+
+    // ---- values: wave = 8 tokens, lane = 4 dims
+    {
+      bool any = false;
+      double al[EX_COLS];
+#pragma unroll
+      for (int c = 0; c < EX_COLS; c++) { al[c] = lds_alpha[c]; any = any || al[c] != 1.0; }
+      if (any) {
+#pragma unroll
+        for (int c = 0; c < EX_COLS; c++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[c][j] *= al[c];
+      }
+      const int tok0 = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + wave * 8;
+      const uint32_t vw[4][4] = {{vcur[0].x, vcur[0].y, vcur[0].z, vcur[0].w}, {vcur[1].x, vcur[1].y, vcur[1].z, vcur[1].w},
+                                 {vcur[2].x, vcur[2].y, vcur[2].z, vcur[2].w}, {vcur[3].x, vcur[3].y, vcur[3].z, vcur[3].w}};
+#pragma unroll
+      for (int tp = 0; tp < 4; tp++) {
+        // a token past the context has weight 0, but what its cache slot holds need not be a number: it enters as 0
+        const bool in0 = tok0 + 2 * tp < lim, in1 = tok0 + 2 * tp + 1 < lim;
+        double v0[4], v1[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          v0[j] = in0 ? bf16lo_to_f64(vw[j][tp]) : 0.0;
+          v1[j] = in1 ? bf16hi_to_f64(vw[j][tp]) : 0.0;
+        }
+#pragma unroll
+        for (int c = 0; c < EX_COLS; c++) {
+          const double2 pp = *(const double2*)&lds_p[c][wave * 8 + 2 * tp];
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[c][j] = fma(pp.x, v0[j], acc[c][j]);
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[c][j] = fma(pp.y, v1[j], acc[c][j]);
+        }
+      }
+    }
+  }
+
+  // ---- the heads' sums and reference exponents, then the accumulators of the 8 waves as ((0+4)+(2+6)) + ((1+5)+(3+7))
+  {
+    const double lt = wave_sum_f64(l_lane);
+    if (lane == 0) { lds_l[wave] = lt; lds_m[wave] = mref; }
+  }
+  __syncthreads();
+  double* red = (double*)lds_raw;
+  auto put = [&](int slot) {
+#pragma unroll
+    for (int c = 0; c < EX_COLS; c++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) red[((slot * EX_COLS + c) * 4 + j) * 64 + lane] = acc[c][j];
+  };
+  auto get = [&](int slot) {
+#pragma unroll
+    for (int c = 0; c < EX_COLS; c++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[c][j] += red[((slot * EX_COLS + c) * 4 + j) * 64 + lane];
+  };
+  if (wave >= 4) put(wave - 4);
+  __syncthreads();
+  if (wave < 4) get(wave);
+  __syncthreads();
+  if (wave == 2 || wave == 3) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) get(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  get(0);
+
+  if (A.splits == 1) {
+#pragma unroll
+    for (int c = 0; c < EX_COLS; c++) {
+      if (c >= A.G) break;
+      const int head = kvh * A.G + c;
+      const double L = lds_l[c], M = lds_m[c];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int d = lane + 64 * j;
+        // a sequence without context (length <= 0 found in device memory) has no weights: zeros and lse = -inf
+        float o = L > 0.0 ? (float)(acc[c][j] / L) : 0.0f;
+        if (A.gate) {
+          const float gv = bf16_to_f32(A.gate[(int64_t)row * A.gate_bstride + (int64_t)head * A.gate_hstride + d]);
+          o = __fmul_rn(o, sigmoid_f64(gv));
+        }
+        A.out[((int64_t)row * A.NH + head) * ATT_HD + d] = f32_to_bf16(o);
+      }
+      if (lane == 0 && A.lse) A.lse[(int64_t)row * A.NH + head] = L > 0.0 ? (float)(M + log(L)) : -INFINITY;
+    }
+  } else {
+    const int64_t pidx = A.slots > 0 ? (int64_t)kvh * A.slots + blockIdx.x : ((int64_t)row * A.NKV + kvh) * A.splits + split;
+    double* po = A.part_o64 + pidx * EX_COLS * ATT_HD;
+#pragma unroll
+    for (int c = 0; c < EX_COLS; c++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) po[c * ATT_HD + lane + 64 * j] = acc[c][j];
+    if (lane < EX_COLS) {
+      A.part_ml64[(pidx * EX_COLS + lane) * 2] = lds_m[lane];
+      A.part_ml64[(pidx * EX_COLS + lane) * 2 + 1] = lds_l[lane];
+    }
+  }
+}
+
+// Merge of the f64 split partials: one workgroup per (head, query row), thread = dim.  The weights exp(ref_s - max ref)
+// of all splits are computed side by side first (thread = split), the partial outputs are then added in split order.
+__global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
+  __shared__ double wsh[ATT_MAX_SPLITS];
+  __shared__ float redm[4];
+  __shared__ double redl[4];
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int kvh = head / A.G, c = head % A.G;
+  int64_t p0 = ((int64_t)b * A.NKV + kvh) * A.splits;
+  int nsplit = A.splits;
+  if (A.slots > 0) {
+    const int2 pl = A.plan[b];
+    nsplit = pl.y;
+    p0 = (int64_t)kvh * A.slots + pl.x;
+  }
+  const bool has = d < nsplit;
+  const double ms = has ? A.part_ml64[((p0 + d) * EX_COLS + c) * 2] : -INFINITY;
+  const double ls = has ? A.part_ml64[((p0 + d) * EX_COLS + c) * 2 + 1] : 0.0;
+  // the reference exponents are f32 values (or -inf), so their maximum is found in f32 without loss
+  float Mf = wave_max((float)ms);
+  if ((d & 63) == 0) redm[d >> 6] = Mf;
+  __syncthreads();
+  const double M = (double)fmaxf(fmaxf(redm[0], redm[1]), fmaxf(redm[2], redm[3]));
+  const double w = (ms == -INFINITY) ? 0.0 : exp(ms - M);
+  wsh[d] = w;
+  double L = wave_sum_f64(ls * w);
+  if ((d & 63) == 0) redl[d >> 6] = L;
+  __syncthreads();
+  L = (redl[0] + redl[1]) + (redl[2] + redl[3]);
+  const float gsig = A.gate ? sigmoid_f64(bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d])) : 1.0f;
+  const double* po = A.part_o64 + (p0 * EX_COLS + c) * ATT_HD + d;
+  double o0 = 0.0, o1 = 0.0;
+  int s = 0;
+  for (; s + 2 <= nsplit; s += 2) {
+    o0 = fma(po[(int64_t)(s + 0) * EX_COLS * ATT_HD], wsh[s + 0], o0);
+    o1 = fma(po[(int64_t)(s + 1) * EX_COLS * ATT_HD], wsh[s + 1], o1);
+  }
+  if (s < nsplit) o0 = fma(po[(int64_t)s * EX_COLS * ATT_HD], wsh[s], o0);
+  float o = L > 0.0 ? (float)((o0 + o1) / L) : 0.0f;          // no context at all: zeros, lse = -inf
+  if (A.gate) o = __fmul_rn(o, gsig);
+  const uint16_t ob = f32_to_bf16(o);
+  A.out[((int64_t)b * A.NH + head) * ATT_HD + d] = ob;
+  if (A.out_q8) lane32_q8_1_store(bf16_to_f32(ob), A.out_q8 + (((int64_t)b * A.NH + head) * (ATT_HD / 32) + (d >> 5)) * 36, d & 31);
+  if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = L > 0.0 ? (float)(M + log(L)) : -INFINITY;
+}
+
+// q bf16 [rows, NH, 256] -> f64 [rows, NKV, 256, 8]: column c < G of (row, kv head) is head kvh * G + c, the rest zeros
+__global__ __launch_bounds__(256) void attn_q_to_f64_kernel(const uint16_t* __restrict__ q, double* __restrict__ qf, int NH, int NKV, int G) {
+  const int kvh = blockIdx.x, row = blockIdx.y, d = threadIdx.x;
+  double* o = qf + (((int64_t)row * NKV + kvh) * ATT_HD + d) * EX_COLS;
+#pragma unroll
+  for (int c = 0; c < EX_COLS; c++)
+    o[c] = c < G ? (double)bf16_to_f32(q[((int64_t)row * NH + kvh * G + c) * ATT_HD + d]) : 0.0;
+}
+
+size_t attn_exact_qf_bytes(int rows, int NKV) { return (size_t)rows * NKV * ATT_HD * EX_COLS * sizeof(double); }
+size_t attn_exact_workspace_bytes(int rows, int NKV, int max_splits) {
+  return (size_t)rows * NKV * max_splits * EX_COLS * (ATT_HD + 2) * sizeof(double) + 64 * sizeof(int2) + attn_exact_qf_bytes(rows, NKV);
+}
+
+// Called by launch_attn_decode with the split plan already in A (same planning as the matrix-instruction form).
+// workspace: partial outputs, partial (ref, sum), plan, then the f64 copy of q unless the caller has one (qf_ready).
+int launch_attn_exact(AttnArgs A, const void* q, const double* qf_ready, void* workspace, size_t workspace_bytes, bool nt, dim3 grid,
+                      int batch) {
+  BK_REQUIRE(A.tpw == 1, "attn_decode (exact): one query row per workgroup");
+  BK_REQUIRE(A.G <= EX_COLS, "attn_decode (exact): at most %d query heads per KV head (got %d)", EX_COLS, A.G);
+  const size_t npart = A.splits > 1 ? (size_t)batch * A.NKV * A.splits : 0;
+  const size_t need = npart * EX_COLS * (ATT_HD + 2) * sizeof(double) + 64 * sizeof(int2) + (qf_ready ? 0 : attn_exact_qf_bytes(batch, A.NKV));
+  BK_REQUIRE(workspace && workspace_bytes >= need, "attn_decode (exact): workspace of %zu bytes needed for %d splits (got %zu)", need, A.splits,
+             workspace_bytes);
+  A.part_o64 = (double*)workspace;
+  A.part_ml64 = A.part_o64 + npart * EX_COLS * ATT_HD;
+  A.plan = (int2*)(A.part_ml64 + npart * EX_COLS * 2);
+  if (qf_ready) {
+    A.qf = qf_ready;
+  } else {
+    double* qf = (double*)(A.plan + 64);
+    hipLaunchKernelGGL(attn_q_to_f64_kernel, dim3(A.NKV, batch), dim3(256), 0, stream(), (const uint16_t*)q, qf, A.NH, A.NKV, A.G);
+    A.qf = qf;
+  }
+  BK_REQUIRE(((uintptr_t)A.qf & 63) == 0, "attn_decode (exact): the f64 query copy must be 64-byte aligned");
+  const dim3 block(EX_THREADS);
+  if (nt) hipLaunchKernelGGL((attn_exact_kernel<true>), grid, block, 0, stream(), A);
+  else hipLaunchKernelGGL((attn_exact_kernel<false>), grid, block, 0, stream(), A);
+  if (A.splits > 1) hipLaunchKernelGGL(attn_exact_merge_kernel, dim3(A.NH, batch), dim3(256), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+}  // namespace bk

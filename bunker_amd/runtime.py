@@ -61,6 +61,8 @@ _SIGS = {
     "bk_gdn_core": [u64, u64, u64, u64, u64, u64, u64, u64, i32, i32],
     "bk_attn_plan": [i32, i32, i32, C.POINTER(i32), C.POINTER(u64)],
     "bk_attn_decode": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, u64, u64, i32, i32, i32, i32, i32, i32],
+    "bk_attn_plan_exact": [i32, i32, i32, C.POINTER(i32), C.POINTER(u64)],
+    "bk_attn_decode_exact": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, u64, u64, i32, i32, i32, i32, i32, i32],
     "bk_attn_decode_noalloc": [u64, u64, u64, u64, i32, u64, i32, u64, i64, i64, u64, u64, i32, i32, i32, i32, i32, i32],
     "bk_kv_append": [u64, u64, u64, u64, u64, i32, u64, i32, i32, i32, i32, i32],
 }
@@ -450,6 +452,23 @@ def attn_decode(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_
     _check(cu().bk_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, max_ctx, gate, gate_bstride, gate_hstride,
                                out, lse, workspace, workspace_bytes, batch, NH, NKV, HD, page_size, splits),
            "bk_attn_decode")
+
+
+def attn_plan_exact(batch: int, NKV: int, max_ctx: int, splits: int = 0):
+    """(splits, workspace bytes) of the double-precision form; the workspace is needed for a single split too."""
+    s, nbytes = i32(splits), u64(0)
+    _check(cu().bk_attn_plan_exact(batch, NKV, max_ctx, C.byref(s), C.byref(nbytes)), "bk_attn_plan_exact")
+    return s.value, nbytes.value
+
+
+def attn_decode_exact(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_len: int, max_ctx: int, out: int,
+                      lse: int, batch: int, NH: int = 16, NKV: int = 2, HD: int = 256, page_size: int = 16, splits: int = 0,
+                      workspace: int = 0, workspace_bytes: int = 0, gate: int = 0, gate_bstride: int = 0,
+                      gate_hstride: int = 0) -> None:
+    """``attn_decode`` with every product and sum in f64: the bits of a host evaluation in doubles."""
+    _check(cu().bk_attn_decode_exact(q, kc, vc, block_table, bt_stride, ctx_len, max_ctx, gate, gate_bstride, gate_hstride,
+                                     out, lse, workspace, workspace_bytes, batch, NH, NKV, HD, page_size, splits),
+           "bk_attn_decode_exact")
 
 
 def attn_decode_noalloc(q: int, kc: int, vc: int, block_table: int, bt_stride: int, ctx_len: int, max_ctx: int, out: int,

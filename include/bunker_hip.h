@@ -194,6 +194,19 @@ BK_API int bk_attn_decode(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_t
                           int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
                           uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size,
                           int splits);
+/* The same attention in double precision.  No GPU kernel exists in the reference for it; the arithmetic is that of its host
+ * loop refAttn (prototypes/fa2_vllm.ts:114-139), which runs in JavaScript numbers, i.e. doubles: every bf16 x bf16 product
+ * and every sum is carried in f64, exp() is evaluated in f64, and the quotient is rounded once to f32 (then gate, then
+ * bf16).  The result does not depend on the number of splits or the batch beyond ~1e-15 relative before that rounding,
+ * so the bf16 outputs equal a host evaluation in doubles bit for bit, and the decode step stays reproducible token for
+ * token.  Arguments as bk_attn_decode; NH / NKV <= 8; the workspace (size from bk_attn_plan_exact, needed also for one
+ * split) holds an f64 copy of q and the f64 partials.  About as fast as bk_attn_decode where the cache read dominates. */
+BK_API int bk_attn_plan_exact(int batch, int NKV, int max_ctx, int* splits, uint64_t* workspace_bytes);
+BK_API int bk_attn_decode_exact(uint64_t q, uint64_t kc, uint64_t vc, uint64_t block_table, int bt_stride,
+                                uint64_t ctx_len, int max_ctx, uint64_t gate, int64_t gate_bstride,
+                                int64_t gate_hstride, uint64_t out, uint64_t lse, uint64_t workspace,
+                                uint64_t workspace_bytes, int batch, int NH, int NKV, int HD, int page_size,
+                                int splits);
 /* bk_attn_decode for callers that cannot allocate device memory or bring a workspace: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and same
  * results (bit for bit, for the same number of splits) as bk_attn_decode, without workspace / workspace_bytes: the

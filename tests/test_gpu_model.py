@@ -1,16 +1,13 @@
 """Full decode step on the GPU against the CPU restatement.
 
-Every op of the step except attention shares its arithmetic rules with the checker and is equal
-to it bit for bit; attention is held to 2e-2 max-abs.  Two checks follow from that:
+Every op of the step shares its arithmetic rules with the checker and is equal to it bit for bit,
+attention included (its double-precision form is the default of the fa2_* ops).  Two checks:
 
-* strict: step by step, the checker recomputes the step from the same state and tokens, verifies
-  each attention output of the GPU within tolerance and continues from the GPU's value; logits
-  (all of them), the winning logit and the argmax token id must then be EQUAL, and so must the
-  recurrent state;
-* free-running: both sides decode on their own; token ids are compared, with the top-1/top-2
-  margin of the checker and the observed logit noise reported (a one-ulp bf16 difference in an
-  attention output can cross a Q8_1 rounding boundary downstream, so equality is demanded only
-  where the margin clears the noise).
+* strict: step by step, the checker recomputes the step from the same state and tokens; every
+  attention output of the GPU, all logits, the winning logit, the argmax token id and the
+  recurrent state must be EQUAL;
+* free-running: both sides decode on their own for the whole run; every token id and every
+  winning logit must be equal, whatever the top-1/top-2 margin (reported) is.
 
 TINY has the model's structure at small dims; SYNTH is the benchmark's synthetic Qwen3.5-style
 model (BASELINE configs[4]) with KV prefilled to 4096."""
@@ -57,7 +54,7 @@ def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=Fa
             (step, gt[step], idx)
         toks, pos = idx, pos + 1
     print("strict: tokens", loop.tokens()[0].T.tolist(), "max attention |gpu-ref| %.3g" % max(ref.attn_err), flush=True)
-    assert max(ref.attn_err) <= 2e-2
+    assert max(ref.attn_err) == 0.0          # the double-precision attention returns the checker's bits
     # recurrent state after the last token
     for l in range(D.NL):
         p = f"model.layers.{l}"
@@ -76,24 +73,16 @@ def _strict_decode(D, W, S, starts, pos0, steps, use_graph, check=None, fused=Fa
 
 
 def _free_running(D, W, S, starts, pos0, steps, got_tokens, got_vals):
-    """Both sides decode on their own.  The only arithmetic the two do not share is the attention output (bf16, 2e-2):
-    a one-ulp difference there reaches the logits as noise, so a token may differ only where the checker's top-1/top-2
-    margin does not clear the noise seen so far; from a sequence's first differing token on the two texts differ."""
+    """Both sides decode on their own: every op returns the checker's bits, so tokens and winning logits are equal for the
+    whole run however small the top-1/top-2 margin gets (it is printed: random weights give near-ties)."""
     from oracle.model_ref import RefModel, free_run_report
     ref = RefModel(D, W, S, batch=len(starts))
     rt_, rv = ref.decode(starts, pos0, steps)
     margins = np.array(ref.margins)
-    noise = np.abs(got_vals - rv)
-    same = got_tokens == rt_
     rep = free_run_report(got_tokens, got_vals, rt_, rv, margins)
     print("free-running:", rep, flush=True)
-    print("  per step (sequence 0): margin / noise", [(round(float(m), 4), round(float(n), 4)) for m, n in zip(margins[:, 0], noise[:, 0])], flush=True)
-    for b in range(len(starts)):
-        for s in range(steps):
-            if not same[s, b]:
-                assert margins[s, b] <= 8 * max(noise[: s + 1, b].max(), 1e-6), (s, b, margins[s, b], noise[: s + 1, b].max())
-                break
-    assert same[0].all() or margins[0].min() < 1e-3
+    assert np.array_equal(got_tokens, rt_), rep
+    assert np.array_equal(got_vals.view(np.uint32), rv.view(np.uint32)), rep
     return rep
 
 

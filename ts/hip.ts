@@ -68,6 +68,8 @@ const SYMBOLS = {
   bk_gdn_core:              { args: ["u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "i32", "i32"], returns: "i32" },
   bk_attn_plan:             { args: ["i32", "i32", "i32", "ptr", "ptr"], returns: "i32" },
   bk_attn_decode:           { args: ["u64", "u64", "u64", "u64", "i32", "u64", "i32", "u64", "i64", "i64", "u64", "u64", "u64", "u64", "i32", "i32", "i32", "i32", "i32", "i32"], returns: "i32" },
+  bk_attn_plan_exact:       { args: ["i32", "i32", "i32", "ptr", "ptr"], returns: "i32" },
+  bk_attn_decode_exact:     { args: ["u64", "u64", "u64", "u64", "i32", "u64", "i32", "u64", "i64", "i64", "u64", "u64", "u64", "u64", "i32", "i32", "i32", "i32", "i32", "i32"], returns: "i32" },
   bk_attn_decode_noalloc:   { args: ["u64", "u64", "u64", "u64", "i32", "u64", "i32", "u64", "i64", "i64", "u64", "u64", "i32", "i32", "i32", "i32", "i32", "i32"], returns: "i32" },
   bk_kv_append:             { args: ["u64", "u64", "u64", "u64", "u64", "i32", "u64", "i32", "i32", "i32", "i32", "i32"], returns: "i32" },
 } as const;
