@@ -282,7 +282,7 @@ static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   const int exact = (int)k.get("exact", 1);
   const size_t qn_bytes = fa2_qn_bytes(batch, NH, HD), qf_bytes = exact ? attn_exact_qf_bytes(batch, NKV) : 0;
   void* qn = k.scratch;
-  double* qf = exact ? (double*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
+  uint32_t* qf = exact ? (uint32_t*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
   void* ws = (uint8_t*)k.scratch + qn_bytes + qf_bytes;
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
                             pos_dev, pos, half, max_len, qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, batch, NH, NKV, HD, 16, qf);
@@ -316,7 +316,7 @@ static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
   const int exact = (int)k.get("exact", 1);
   const size_t qn_bytes = fa2_qn_bytes(T, NH, HD), qf_bytes = exact ? attn_exact_qf_bytes(T, NKV) : 0;
   void* qn = k.scratch;
-  double* qf = exact ? (double*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
+  uint32_t* qf = exact ? (uint32_t*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
   void* ws = (uint8_t*)k.scratch + qn_bytes + qf_bytes;
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
                             pos, 0, half, max_len, qn, P<void>(s[9]), P<void>(s[10]), table, 0, T, NH, NKV, HD, 16, qf);

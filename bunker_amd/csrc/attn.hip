@@ -323,7 +323,7 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw, int exact, const double* qf_ready) {
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw, int exact, const uint32_t* qf_ready) {
   BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
@@ -461,7 +461,7 @@ struct PrepArgs {
   const float *cos_t, *sin_t;      // f32 [max_len, half]
   const int32_t* pos_dev; int pos_scalar;
   uint16_t *qout, *kc, *vc;
-  double* qf;                      // optional: the query heads also as f64 [B, NKV, 256, 8] for the double-precision attention
+  uint32_t* qf;                    // optional: the query heads also widened to f64, high words [B, NKV, 256, 8], for the double-precision attention
   const int32_t* block_table; int bt_stride;
   int NH, NKV, half, max_len;
 };
@@ -515,14 +515,14 @@ __global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs A) {
     dst[i] = o;
     if (is_q && A.qf) {
       const int G = A.NH / A.NKV;
-      A.qf[(((int64_t)b * A.NKV + role / G) * ATT_HD + i) * 8 + role % G] = (double)bf16_to_f32(o);
+      A.qf[(((int64_t)b * A.NKV + role / G) * ATT_HD + i) * 8 + role % G] = (uint32_t)(__builtin_bit_cast(uint64_t, (double)bf16_to_f32(o)) >> 32);
     }
   }
 }
 
 int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
-                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size, double* qf) {
+                     void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size, uint32_t* qf) {
   BK_REQUIRE(qg && k && v && qw && kw && cos_t && sin_t && qout && kc && vc, "attn_prep: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_prep: head_dim 256 and 16-token pages only");
   BK_REQUIRE(batch > 0 && batch <= 65535 && NH > 0 && NKV > 0 && half > 0 && 2 * half <= HD, "attn_prep: bad shape");

@@ -31,7 +31,7 @@ struct AttnArgs {
   float* part_ml;             // f32 [B, NKV, splits, 16, 2] (max, sum)
   int2* plan;                 // balanced form: (first slot, number of splits) of every sequence, behind the partials
   // double-precision form (attn_exact.hip): q widened to f64 [rows, NKV, 256, 8 columns], partials in f64
-  const double* qf;           // column c of (row, kv head) is query head kvh * G + c (c < G <= 8; the other columns hold zeros)
+  const uint32_t* qf;          // column c of (row, kv head) is query head kvh * G + c (c < G <= 8; the other columns hold zeros)
   double* part_o64;           // f64 [partials, 8, 256] unnormalised partial outputs
   double* part_ml64;          // f64 [partials, 8, 2] (reference exponent, sum)
   int64_t gate_bstride, gate_hstride;
@@ -117,6 +117,6 @@ __device__ __forceinline__ bool attn_wg_range(const AttnArgs& A, int lane, int& 
 }
 
 // attn_exact.hip, called by launch_attn_decode with the cut of the pages already in A
-int launch_attn_exact(AttnArgs A, const void* q, const double* qf_ready, void* workspace, size_t workspace_bytes, bool nt, dim3 grid, int batch);
+int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void* workspace, size_t workspace_bytes, bool nt, dim3 grid, int batch);
 
 }  // namespace bk

@@ -7,16 +7,21 @@
 // A workgroup (8 waves) walks its page range in tiles of 64 tokens (4 pages):
 //   1. the K rows of the tile go to LDS (coalesced 16-byte loads, one page per round of the 512 threads);
 //   2. scores: lane = token, wave = 32 of the 256 dims.  The lane converts its 32 K values to f64 once and multiplies
-//      each into the 8 query heads of the group; the query values are wave-uniform and come through the scalar
-//      unit (s_load from the f64 copy of q) as the SGPR operand of v_fmac_f64 — no cross-lane reduction, the
-//      conversions are shared by the 8 heads.  The 8 partial sums per (head, token) meet through LDS in wave order;
+//      each into the 8 query heads of the group.  A query value is the same for all lanes: it is the DPP operand of
+//      v_fmac_f64 (row_newbcast:n = lane n of every row of 16 lanes, for all lanes of the row), read from registers
+//      that hold 16 query values each, the same 16 in all four rows, loaded once per workgroup — no cross-lane
+//      reduction, no operand traffic, the conversions are shared by the 8 heads.  The 8 partial sums per (head, token)
+//      meet through LDS in wave order;
 //   3. weights: wave = head.  p = exp(s - ref) in f64; `ref` is a reference exponent per head, set from the first
 //      tile's maximum and moved only when a score exceeds it by more than 600 (f64 has the range: no running-max
 //      rescale per tile), the sum of p is kept per lane;
 //   4. values: wave = 8 tokens of the tile, lane = 4 of the 256 dims (V pages are dim-major, so a lane's 8 tokens are
-//      one 16-byte load and the wave's loads are contiguous); p is read from LDS at a wave-uniform address.
+//      one 16-byte load and the wave's loads are contiguous); the weights of the wave's 8 tokens x 8 heads sit in four
+//      register pairs (16 per pair, again the same in every row) and enter the FMAs through the same DPP broadcast.
 // The waves' accumulators are added in a fixed tree through LDS; partials of the splits are f64 and a second
 // kernel merges them.  Roughly 90 vector instructions per (token, KV head), three quarters of them f64 FMAs.
+#include <type_traits>
+
 #include "attn_args.h"
 
 namespace bk {
@@ -29,18 +34,57 @@ constexpr int EX_COLS = 8;                        // query heads per KV head ser
 constexpr int EX_KROW = ATT_HD * 2 + 16;          // bytes of a K row in LDS: 16 bytes of padding spread the rows over the banks
 constexpr double EX_REF_SLACK = 600.0;            // exp() of up to this much above the reference exponent stays far from overflow
 
-typedef const double __attribute__((address_space(4)))* cdptr_t;      // loads through this pointer may use the scalar unit
+constexpr int EX_PROW = EX_COLS + 1;              // doubles per token row of the weights in LDS (padded against bank conflicts)
+
+// A bf16 value widened to f64 has an all-zero low word, so the query copy holds the high words only.
+__device__ __forceinline__ double f64_from_high(uint32_t hi) { return __builtin_bit_cast(double, (uint64_t)hi << 32); }
+__device__ __forceinline__ uint32_t bf16_to_f64_high(uint16_t b) {
+  return (uint32_t)(__builtin_bit_cast(uint64_t, (double)bf16_to_f32(b)) >> 32);
+}
 
 __device__ __forceinline__ double bf16lo_to_f64(uint32_t w) { return (double)__uint_as_float(w << 16); }
 __device__ __forceinline__ double bf16hi_to_f64(uint32_t w) { return (double)__uint_as_float(w & 0xffff0000u); }
+
+// acc[c] += bsrc(lane 8 * E + c of the lane's row of 16) * v for the 8 columns c: eight v_fmac_f64 whose first factor is
+// read through the DPP row broadcast (the only DPP form of the f64 unit).  The two idle cycles in front keep the
+// distance a DPP read needs from a vector instruction that may have written `bsrc` just before.
+template <int E>
+__device__ __forceinline__ void fmac8_bcast(double (&a)[EX_COLS], double bsrc, double v) {
+  static_assert(E == 0 || E == 1, "half of the row");
+  if (E == 0)
+    asm("s_nop 1\n\t"
+        "v_fmac_f64_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %1, %8, %9 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %2, %8, %9 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %3, %8, %9 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %4, %8, %9 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %5, %8, %9 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %6, %8, %9 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %7, %8, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+        : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
+        : "v"(bsrc), "v"(v));
+  else
+    asm("s_nop 1\n\t"
+        "v_fmac_f64_dpp %0, %8, %9 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %1, %8, %9 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %2, %8, %9 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %3, %8, %9 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %4, %8, %9 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %5, %8, %9 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %6, %8, %9 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %7, %8, %9 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
+        : "v"(bsrc), "v"(v));
+}
 
 template <bool NT>
 __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   // K tile (33792 bytes) and the exchange buffer of the partial scores (8 waves x 8 heads x 64 tokens x 8 = 32768 bytes);
   // the same memory carries the accumulator tree at the end (4 waves x 8 x 256 doubles = 65536 bytes)
   __shared__ __align__(16) unsigned char lds_raw[EX_TILE * EX_KROW + EX_WAVES * EX_COLS * EX_TILE * 8];
-  __shared__ __align__(16) double lds_p[EX_COLS][EX_TILE];
+  __shared__ __align__(16) double lds_p[EX_TILE][EX_PROW];      // weights of the tile, [token][head]
   __shared__ double lds_alpha[EX_COLS], lds_m[EX_COLS], lds_l[EX_COLS];
+  __shared__ int lds_rescale[2];                // set by a head that moved its reference exponent in an even / odd tile
   __shared__ int lds_bt[ATT_MAX_PPS];
   unsigned char* ktile = lds_raw;
   double (*xch)[EX_COLS][EX_TILE] = (double (*)[EX_COLS][EX_TILE])(lds_raw + EX_TILE * EX_KROW);
@@ -77,7 +121,13 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
     for (int j = 0; j < 4; j++) vr[j] = ld16(A.vc + base + (lane + 64 * j) * ATT_PAGE);
   };
 
-  uintptr_t q_addr = (uintptr_t)(A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + wave * 32) * EX_COLS);
+  // the wave's 32 dims x 8 heads of q: register pair g holds dims 2g, 2g + 1 (lane n of a row: dim 2g + n / 8, head n % 8)
+  double qreg[16];
+  {
+    const uint32_t* qw = A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + wave * 32) * EX_COLS + (lane & 15);
+#pragma unroll
+    for (int g = 0; g < 16; g++) qreg[g] = f64_from_high(qw[g * 16]);
+  }
 
   double acc[EX_COLS][4];
 #pragma unroll
@@ -87,22 +137,21 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   double l_lane = 0.0;            // wave = head: this lane's share of the sum of weights
   double mref = -INFINITY;        // wave = head: the reference exponent
 
-  uint4 kpre[EX_TILE_PAGES], vcur[4];
-  if (ntiles > 0) load_k(0, kpre);
+  // K and V of the next tile are requested a whole tile ahead (a tile's work is shorter than a trip to memory under load)
+  uint4 kpre[EX_TILE_PAGES], vcur[4], vpre[4];
+  if (ntiles > 0) { load_k(0, kpre); load_v(0, vpre); }
   for (int tile = 0; tile < ntiles; tile++) {
 #pragma unroll
     for (int r = 0; r < EX_TILE_PAGES; r++)
       *(uint4*)(ktile + (r * ATT_PAGE + (threadIdx.x >> 5)) * EX_KROW + (threadIdx.x & 31) * 16) = kpre[r];
+#pragma unroll
+    for (int j = 0; j < 4; j++) vcur[j] = vpre[j];
+    if (threadIdx.x == 0) lds_rescale[tile & 1] = 0;      // read two barriers back at the latest; set again behind the next barrier
     __syncthreads();
-    load_v(tile, vcur);
-    if (tile + 1 < ntiles) load_k(tile + 1, kpre);
+    if (tile + 1 < ntiles) { load_k(tile + 1, kpre); load_v(tile + 1, vpre); }
 
     // ---- scores: lane = token, this wave's 32 dims
     {
-      // the query values are read again in every tile (they stay in the scalar cache): kept across tiles they would
-      // need 512 scalar registers, so the address is made opaque to keep the loads inside the loop
-      asm volatile("" : "+s"(q_addr));
-      cdptr_t q = (cdptr_t)q_addr;
       double sacc[EX_COLS];
 #pragma unroll
       for (int c = 0; c < EX_COLS; c++) sacc[c] = 0.0;
@@ -113,12 +162,8 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
         const uint32_t w[4] = {kk.x, kk.y, kk.z, kk.w};
 #pragma unroll
         for (int wi = 0; wi < 4; wi++) {
-          const double k0 = bf16lo_to_f64(w[wi]), k1 = bf16hi_to_f64(w[wi]);
-          const int d = i * 8 + wi * 2;
-#pragma unroll
-          for (int c = 0; c < EX_COLS; c++) sacc[c] = fma(k0, q[d * EX_COLS + c], sacc[c]);
-#pragma unroll
-          for (int c = 0; c < EX_COLS; c++) sacc[c] = fma(k1, q[(d + 1) * EX_COLS + c], sacc[c]);
+          fmac8_bcast<0>(sacc, qreg[i * 4 + wi], bf16lo_to_f64(w[wi]));
+          fmac8_bcast<1>(sacc, qreg[i * 4 + wi], bf16hi_to_f64(w[wi]));
         }
       }
 #pragma unroll
@@ -142,45 +187,53 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
       }
       const double p = valid ? exp(s - mref) : 0.0;
       l_lane += p;
-      lds_p[wave][lane] = p;
-      if (lane == 0) lds_alpha[wave] = alpha;
+      lds_p[lane][wave] = p;
+      if (lane == 0) {
+        lds_alpha[wave] = alpha;
+        if (alpha != 1.0) lds_rescale[tile & 1] = 1;
+      }
     }
     __syncthreads();
 
     // ---- values: wave = 8 tokens, lane = 4 dims
     {
-      bool any = false;
-      double al[EX_COLS];
+      // a head whose reference exponent moved in this tile (first tile aside: rare) rescales what was summed under the old one
+      if (__builtin_amdgcn_readfirstlane(lds_rescale[tile & 1])) {
 #pragma unroll
-      for (int c = 0; c < EX_COLS; c++) { al[c] = lds_alpha[c]; any = any || al[c] != 1.0; }
-      if (any) {
+        for (int c = 0; c < EX_COLS; c++) {
+          const double al = lds_alpha[c];
 #pragma unroll
-        for (int c = 0; c < EX_COLS; c++)
-#pragma unroll
-          for (int j = 0; j < 4; j++) acc[c][j] *= al[c];
+          for (int j = 0; j < 4; j++) acc[c][j] *= al;
+        }
       }
+      // the weights of this wave's 8 tokens: pair h holds tokens 2h, 2h + 1 (lane n of a row: token 2h + n / 8, head n % 8)
+      double preg[4];
+#pragma unroll
+      for (int h = 0; h < 4; h++) preg[h] = lds_p[wave * 8 + 2 * h + ((lane & 15) >> 3)][lane & 7];
       const int tok0 = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + wave * 8;
       const uint32_t vw[4][4] = {{vcur[0].x, vcur[0].y, vcur[0].z, vcur[0].w}, {vcur[1].x, vcur[1].y, vcur[1].z, vcur[1].w},
                                  {vcur[2].x, vcur[2].y, vcur[2].z, vcur[2].w}, {vcur[3].x, vcur[3].y, vcur[3].z, vcur[3].w}};
+      // a token past the context has weight 0, but what its cache slot holds need not be a number: it enters as 0
+      // (only the tile that holds the end of the context pays for the test)
+      auto values = [&](auto tail_c) {
+        constexpr bool TAIL = decltype(tail_c)::value;
 #pragma unroll
-      for (int tp = 0; tp < 4; tp++) {
-        // a token past the context has weight 0, but what its cache slot holds need not be a number: it enters as 0
-        const bool in0 = tok0 + 2 * tp < lim, in1 = tok0 + 2 * tp + 1 < lim;
-        double v0[4], v1[4];
+        for (int h = 0; h < 4; h++) {
+          const bool in0 = !TAIL || tok0 + 2 * h < lim, in1 = !TAIL || tok0 + 2 * h + 1 < lim;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          v0[j] = in0 ? bf16lo_to_f64(vw[j][tp]) : 0.0;
-          v1[j] = in1 ? bf16hi_to_f64(vw[j][tp]) : 0.0;
+          for (int j = 0; j < 4; j++) {
+            double a[EX_COLS];
+#pragma unroll
+            for (int c = 0; c < EX_COLS; c++) a[c] = acc[c][j];
+            fmac8_bcast<0>(a, preg[h], in0 ? bf16lo_to_f64(vw[j][h]) : 0.0);
+            fmac8_bcast<1>(a, preg[h], in1 ? bf16hi_to_f64(vw[j][h]) : 0.0);
+#pragma unroll
+            for (int c = 0; c < EX_COLS; c++) acc[c][j] = a[c];
+          }
         }
-#pragma unroll
-        for (int c = 0; c < EX_COLS; c++) {
-          const double2 pp = *(const double2*)&lds_p[c][wave * 8 + 2 * tp];
-#pragma unroll
-          for (int j = 0; j < 4; j++) acc[c][j] = fma(pp.x, v0[j], acc[c][j]);
-#pragma unroll
-          for (int j = 0; j < 4; j++) acc[c][j] = fma(pp.y, v1[j], acc[c][j]);
-        }
-      }
+      };
+      if (tok0 + 8 > lim) values(std::true_type{});
+      else values(std::false_type{});
     }
   }
 
@@ -295,23 +348,24 @@ __global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
   if (d == 0 && A.lse) A.lse[(int64_t)b * A.NH + head] = L > 0.0 ? (float)(M + log(L)) : -INFINITY;
 }
 
-// q bf16 [rows, NH, 256] -> f64 [rows, NKV, 256, 8]: column c < G of (row, kv head) is head kvh * G + c, the rest zeros
-__global__ __launch_bounds__(256) void attn_q_to_f64_kernel(const uint16_t* __restrict__ q, double* __restrict__ qf, int NH, int NKV, int G) {
+// q bf16 [rows, NH, 256] -> high words of the f64 values [rows, NKV, 256, 8]: column c < G of (row, kv head) is head
+// kvh * G + c, the rest zeros
+__global__ __launch_bounds__(256) void attn_q_to_f64_kernel(const uint16_t* __restrict__ q, uint32_t* __restrict__ qf, int NH, int NKV, int G) {
   const int kvh = blockIdx.x, row = blockIdx.y, d = threadIdx.x;
-  double* o = qf + (((int64_t)row * NKV + kvh) * ATT_HD + d) * EX_COLS;
+  uint32_t* o = qf + (((int64_t)row * NKV + kvh) * ATT_HD + d) * EX_COLS;
 #pragma unroll
   for (int c = 0; c < EX_COLS; c++)
-    o[c] = c < G ? (double)bf16_to_f32(q[((int64_t)row * NH + kvh * G + c) * ATT_HD + d]) : 0.0;
+    o[c] = c < G ? bf16_to_f64_high(q[((int64_t)row * NH + kvh * G + c) * ATT_HD + d]) : 0u;
 }
 
-size_t attn_exact_qf_bytes(int rows, int NKV) { return (size_t)rows * NKV * ATT_HD * EX_COLS * sizeof(double); }
+size_t attn_exact_qf_bytes(int rows, int NKV) { return (size_t)rows * NKV * ATT_HD * EX_COLS * sizeof(uint32_t); }
 size_t attn_exact_workspace_bytes(int rows, int NKV, int max_splits) {
   return (size_t)rows * NKV * max_splits * EX_COLS * (ATT_HD + 2) * sizeof(double) + 64 * sizeof(int2) + attn_exact_qf_bytes(rows, NKV);
 }
 
 // Called by launch_attn_decode with the split plan already in A (same planning as the matrix-instruction form).
 // workspace: partial outputs, partial (ref, sum), plan, then the f64 copy of q unless the caller has one (qf_ready).
-int launch_attn_exact(AttnArgs A, const void* q, const double* qf_ready, void* workspace, size_t workspace_bytes, bool nt, dim3 grid,
+int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void* workspace, size_t workspace_bytes, bool nt, dim3 grid,
                       int batch) {
   BK_REQUIRE(A.tpw == 1, "attn_decode (exact): one query row per workgroup");
   BK_REQUIRE(A.G <= EX_COLS, "attn_decode (exact): at most %d query heads per KV head (got %d)", EX_COLS, A.G);
@@ -325,7 +379,7 @@ int launch_attn_exact(AttnArgs A, const void* q, const double* qf_ready, void* w
   if (qf_ready) {
     A.qf = qf_ready;
   } else {
-    double* qf = (double*)(A.plan + 64);
+    uint32_t* qf = (uint32_t*)(A.plan + 64);
     hipLaunchKernelGGL(attn_q_to_f64_kernel, dim3(A.NKV, batch), dim3(256), 0, stream(), (const uint16_t*)q, qf, A.NH, A.NKV, A.G);
     A.qf = qf;
   }

@@ -90,7 +90,7 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
                        int NH, int NKV, int HD, int page_size, int splits, void* out_q8 = nullptr, int tpw = 1, int exact = 0,
-                       const double* qf_ready = nullptr);
+                       const uint32_t* qf_ready = nullptr);
 // attn_exact.hip: the double-precision form (workspace: f64 partials, plan, f64 copy of q)
 size_t attn_exact_qf_bytes(int rows, int NKV);
 size_t attn_exact_workspace_bytes(int rows, int NKV, int max_splits);
@@ -102,7 +102,7 @@ int launch_attn_decode_noalloc(int device, const void* q, const void* kc, const 
 int launch_attn_prep(const void* qg, const void* k, const void* v, const void* qw, const void* kw, const float* cos_t,
                      const float* sin_t, const int32_t* pos_dev, int pos_scalar, int half, int max_len, void* qout, void* kc,
                      void* vc, const int32_t* block_table, int bt_stride, int batch, int NH, int NKV, int HD, int page_size,
-                     double* qf = nullptr);
+                     uint32_t* qf = nullptr);
 int launch_kv_append(const void* k, const void* v, void* kc, void* vc, const int32_t* block_table, int bt_stride,
                      const int32_t* pos_dev, int pos_scalar, int max_len, int batch, int NKV, int HD, int page_size);
 
