@@ -196,7 +196,31 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     parity_runs = {}
     PARITY = {1: ([0], 32), 32: ([0, 13, 31], 16)}       # sequences and steps the checker decodes again on the CPU
     weight_bytes = sum(v.nbytes for k, v in W.items() if v.dtype == np.uint8)
-    for B, steps in ((1, steps_bs1), (32, steps_bs32)):
+    # the step as it ships (attention in double precision: the checker's bits) and, as a second figure, with the bf16
+    # matrix-instruction attention (within 2e-2 per attention output; tokens then follow the checker only while the
+    # top-1 / top-2 margin clears the noise)
+    for B, steps, exact in ((1, steps_bs1, True), (32, steps_bs32, True), (1, steps_bs1, False), (32, steps_bs32, False)):
+        runner.ATTN_EXACT = exact
+        if not exact:
+            S = synth_model.device_state(synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True))
+            g = model.buildModelGraph(D, B)
+            env = runner.DecodeEnv(g, W, S, inplace_state=True, device_weights=dev_w)
+            starts = [(9419 + 4099 * i) % D.VOCAB for i in range(B)]
+            warm = 8 if B == 1 else 4
+            loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph,
+                                     partition=runner.fusedPartition(g) if fused else None)
+            runner.ATTN_EXACT = True
+            loop.step(warm)
+            rt.cuSync()
+            e0, e1 = rt.Event().record(), rt.Event()
+            loop.step(steps)
+            e1.record()
+            rt.cuSync()
+            ms = e0.elapsed_ms(e1) / steps
+            out[f"bs{B}"]["with_bf16_mfma_attention"] = {"tok_per_s": round(B / (ms * 1e-3), 1), "ms_per_step": round(ms, 4)}
+            loop.close()
+            env.close()                    # its state; the weights belong to the first environment
+            continue
         S_host = synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True)
         chk, nchk = PARITY[B]
         S_chk = {k: np.array(np.asarray(v)[chk], copy=True) for k, v in S_host.items()}
@@ -232,6 +256,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
                          "wall_ms_per_step": round(wall * 1e3 / steps, 4), "steps": steps,
                          "launch": "hip graph replay" if use_graph else "eager", "launches_per_step": len(loop.launches), "partition": "fused" if fused else "node per kernel", "step_bytes": weight_bytes + state_bytes,
                          "hbm_floor_us": round(floor_us, 1), "frac_of_floor": round(floor_us / (ms * 1e3), 4),
+                         "attention": "double precision (fa2 ops exact=1)",
                          "first_tokens": toks[:4, 0].tolist()}
     # prompt processing on the same model (sequence 0 of the batch-1 environment, from an empty state)
     from bunker_amd import prefill
@@ -394,19 +419,25 @@ def bench_kernels(rt, synth, use_graph=True, iters=50):
         dq = rt.to_device(bf(g.standard_normal((B, NH, HD), dtype=np.float32)))
         dbt, dctx = rt.to_device(bt), rt.to_device(ctx)
         dout, dlse = rt.cuAlloc(B * NH * HD * 2), rt.cuAlloc(B * NH * 4)
-        splits, ws = rt.attn_plan(B, NKV, L)
-        dws = rt.cuAlloc(ws) if ws else 0
-
-        def run(i):
-            rt.attn_decode(dq, kcs[i % ROT], vcs[i % ROT], dbt, ppseq, dctx, L, dout, dlse, B, NH, NKV, HD, 16, splits, dws, ws)
-
-        for i in range(3):
-            run(i)
-        us = _time_launches(rt, lambda: [run(i) for i in range(iters)], use_graph) / iters
         nbytes = int(sum(2 * NKV * int(c) * HD * 2 for c in ctx) + B * NH * HD * 2 * 2 + B * NH * 4)
-        res[f"attn_decode_b{B}_L{L}"] = {"us": round(us, 3), "bytes": nbytes, "splits": splits,
-                                         "GBps": round(nbytes / us / 1e3, 1),
-                                         "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        # the matrix-instruction form (bf16 products, 2e-2) and the double-precision form (the checker's bits; the
+        # default of the decode step's attention op)
+        for key, plan, fn in (("attn_decode", rt.attn_plan, rt.attn_decode), ("attn_decode_exact", rt.attn_plan_exact, rt.attn_decode_exact)):
+            splits, ws = plan(B, NKV, L)
+            dws = rt.cuAlloc(ws) if ws else 0
+
+            def run(i):
+                fn(dq, kcs[i % ROT], vcs[i % ROT], dbt, ppseq, dctx, L, dout, dlse, B, NH, NKV, HD, 16, splits, dws, ws)
+
+            for i in range(3):
+                run(i)
+            us = _time_launches(rt, lambda: [run(i) for i in range(iters)], use_graph) / iters
+            res[f"{key}_b{B}_L{L}"] = {"us": round(us, 3), "bytes": nbytes, "splits": splits,
+                                       "GBps": round(nbytes / us / 1e3, 1),
+                                       "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+            if dws:
+                rt.cuFree(dws)
+        dws = 0
         for p in kcs + vcs + [dq, dbt, dctx, dout, dlse] + ([dws] if dws else []):
             rt.cuFree(p)
     return res
@@ -530,9 +561,13 @@ def main():
     for si, (name, N, K) in enumerate(SHAPES):
         ms = region_ms[name] / args.steps
         b = gemv_bytes(N, K)
+        body_us = max(ms * 1e3 - launch_floor_us, 1e-3)      # what the kernel adds to the shortest possible launch
         per_shape[name] = {"N": N, "K": K, "us_per_launch": round(ms * 1e3, 3), "bytes": b,
                            "GBps": round(b / (ms * 1e-3) / 1e9, 1),
-                           "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                           "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                           "us_minus_launch_floor": round(body_us, 3),
+                           "GBps_minus_launch_floor": round(b / body_us / 1e3, 1),
+                           "frac_hbm_peak_minus_launch_floor": round(b / body_us / 1e3 / HBM_PEAK_GBS, 4)}
     step_bytes = sum(gemv_bytes(N, K) for _, N, K in SHAPES)
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9

@@ -202,8 +202,15 @@ def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str
             parts.append("ids_dev=1")
         if n.op in ("rope", "ropek", "fa2_attn"):
             parts.append("pos_dev=1")
+    if n.op == "fa2_attn" and not ATTN_EXACT:
+        parts.append("exact=0")
     return " ".join(parts)
 
+
+# Attention ops run their double-precision form by default (the checker's bits, so a decode reproduces the host
+# evaluation token for token); False selects the bf16 matrix-instruction form (within 2e-2, 1.5 to 1.8 times faster on
+# the attention launches themselves) for every plan built afterwards.
+ATTN_EXACT = True
 
 Q8OUT_MIN_BATCH = 8      # from this batch on producers also emit their output as Q8_1 (gemv_fused then runs its batched path)
 
@@ -262,7 +269,8 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         qn, rp, kn, rk, fa = grp
         P = fa.params
         spec = (f"fa2_fused HD={int(P['HD'])} NH={int(P['NH'])} NKV={int(P['NKV'])} MAX_LEN={int(P['MAX_LEN'])} "
-                f"ROT_HALF={int(rp.params['ROT_HALF'])}") + bpart + (" pos_dev=1" if device_scalars else "")
+                f"ROT_HALF={int(rp.params['ROT_HALF'])}") + bpart + (" pos_dev=1" if device_scalars else "") + \
+            ("" if ATTN_EXACT else " exact=0")
         args = [qn.inputs[0].tensorName, kn.inputs[0].tensorName, fa.inputs[2].tensorName, qn.inputs[1].tensorName,
                 kn.inputs[1].tensorName, rp.inputs[1].tensorName, rp.inputs[2].tensorName, rp.inputs[3].tensorName,
                 fa.inputs[4].tensorName, fa.inputs[5].tensorName, fa.outputs[0].tensorName]
