@@ -4,8 +4,9 @@
 // prototypes/fa2_vllm.ts:114-139 evaluated in JavaScript numbers (doubles) — whatever the split count, the tile
 // order or the batch.  bf16 x bf16 products are exact in f64; the order of the additions only moves the ~1e-16 tail.
 //
-// A workgroup (8 waves) walks its page range in tiles of 64 tokens (4 pages):
-//   1. the K rows of the tile go to LDS (coalesced 16-byte loads, one page per round of the 512 threads);
+// A workgroup walks its page range in tiles of 64 tokens (4 pages) with 16 waves in two roles, 8 score waves and 8
+// value waves, one tile apart:
+//   1. (score waves) the K rows of the tile go to LDS (coalesced 16-byte loads, one page per round of the 512 threads);
 //   2. scores: lane = token, wave = 32 of the 256 dims.  The lane converts its 32 K values to f64 once and multiplies
 //      each into the 8 query heads of the group.  A query value is the same for all lanes: it is the DPP operand of
 //      v_fmac_f64 (row_newbcast:n = lane n of every row of 16 lanes, for all lanes of the row), read from registers
@@ -15,10 +16,15 @@
 //   3. weights: wave = head.  p = exp(s - ref) in f64; `ref` is a reference exponent per head, set from the first
 //      tile's maximum and moved only when a score exceeds it by more than 600 (f64 has the range: no running-max
 //      rescale per tile), the sum of p is kept per lane;
-//   4. values: wave = 8 tokens of the tile, lane = 4 of the 256 dims (V pages are dim-major, so a lane's 8 tokens are
-//      one 16-byte load and the wave's loads are contiguous); the weights of the wave's 8 tokens x 8 heads sit in four
-//      register pairs (16 per pair, again the same in every row) and enter the FMAs through the same DPP broadcast.
-// The waves' accumulators are added in a fixed tree through LDS; partials of the splits are f64 and a second
+//   4. (value waves, one step later) values: wave = 8 tokens of the tile, lane = 4 of the 256 dims (V pages are
+//      dim-major, so a lane's 8 tokens of a dim are one 16-byte load and the wave's loads are contiguous); the weights
+//      of the wave's 8 tokens x 8 heads sit in four register pairs (16 per pair, again the same in every row) and
+//      enter the FMAs through the same DPP broadcast.
+// Three barriers per step separate 1 | 2 | 3; the value waves do a quarter, a half and a quarter of their tile in the
+// three intervals, so the vector unit always has work of both roles to choose from (4 waves per SIMD) and the waits
+// of one role (barriers, LDS, memory) are covered by the other.  Every load is issued a step ahead of its use and
+// unconditionally, so the waits count loads instead of draining the queue.
+// The value waves' accumulators are added in a fixed tree through LDS; partials of the splits are f64 and a second
 // kernel merges them.  Roughly 90 vector instructions per (token, KV head), three quarters of them f64 FMAs.
 #include <type_traits>
 
@@ -26,8 +32,8 @@
 
 namespace bk {
 
-constexpr int EX_WAVES = 8;
-constexpr int EX_THREADS = EX_WAVES * 64;
+constexpr int EX_SW = 8;                          // score waves of a workgroup; as many value waves
+constexpr int EX_THREADS = 2 * EX_SW * 64;
 constexpr int EX_TILE = 64;                       // tokens per tile = 4 pages
 constexpr int EX_TILE_PAGES = EX_TILE / ATT_PAGE;
 constexpr int EX_COLS = 8;                        // query heads per KV head served by one workgroup
@@ -81,9 +87,9 @@ template <bool NT>
 __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   // K tile (33792 bytes) and the exchange buffer of the partial scores (8 waves x 8 heads x 64 tokens x 8 = 32768 bytes);
   // the same memory carries the accumulator tree at the end (4 waves x 8 x 256 doubles = 65536 bytes)
-  __shared__ __align__(16) unsigned char lds_raw[EX_TILE * EX_KROW + EX_WAVES * EX_COLS * EX_TILE * 8];
-  __shared__ __align__(16) double lds_p[EX_TILE][EX_PROW];      // weights of the tile, [token][head]
-  __shared__ double lds_alpha[EX_COLS], lds_m[EX_COLS], lds_l[EX_COLS];
+  __shared__ __align__(16) unsigned char lds_raw[EX_TILE * EX_KROW + EX_SW * EX_COLS * EX_TILE * 8];
+  __shared__ __align__(16) double lds_p[2][EX_TILE][EX_PROW];   // weights of a tile, [token][head]; even / odd tiles
+  __shared__ double lds_alpha[2][EX_COLS], lds_m[EX_COLS], lds_l[EX_COLS];
   __shared__ int lds_rescale[2];                // set by a head that moved its reference exponent in an even / odd tile
   __shared__ int lds_bt[ATT_MAX_PPS];
   unsigned char* ktile = lds_raw;
@@ -91,6 +97,9 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool value_role = wave >= EX_SW;                       // waves 0..7 score, waves 8..15 accumulate values
+  const int w8 = wave & (EX_SW - 1);
+  const int tid8 = threadIdx.x & (EX_SW * 64 - 1);             // thread index within the role
   int split, b, p_begin, p_end;
   if (!attn_wg_range(A, lane, b, split, p_begin, p_end)) return;
   const int row = __builtin_amdgcn_readfirstlane(b);          // one query row per workgroup (tpw = 1)
@@ -102,6 +111,7 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 
   for (int i = threadIdx.x; i < npg; i += EX_THREADS)
     lds_bt[i] = A.block_table ? A.block_table[(int64_t)row * A.bt_stride + p_begin + i] : row * A.bt_stride + p_begin + i;
+  if (threadIdx.x < 2) lds_rescale[threadIdx.x] = 0;
   __syncthreads();
 
   // a page past the range (the last tile may be short) reads the last page again; its tokens are masked below
@@ -111,22 +121,82 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
     const u32x4_nt t4 = NT ? __builtin_nontemporal_load(p4) : *p4;
     return make_uint4(t4[0], t4[1], t4[2], t4[3]);
   };
-  auto load_k = [&](int tile, uint4 (&kr)[EX_TILE_PAGES]) {        // round r of the 512 threads covers page r of the tile (8 KiB)
-#pragma unroll
-    for (int r = 0; r < EX_TILE_PAGES; r++) kr[r] = ld16(A.kc + page_base(tile * EX_TILE_PAGES + r) + threadIdx.x * 8);
-  };
-  auto load_v = [&](int tile, uint4 (&vr)[4]) {                    // wave: tokens 8 * wave .. + 8 of the tile; lane: dims lane + 64 j
-    const int64_t base = page_base(tile * EX_TILE_PAGES + (wave >> 1)) + (wave & 1) * 8;
-#pragma unroll
-    for (int j = 0; j < 4; j++) vr[j] = ld16(A.vc + base + (lane + 64 * j) * ATT_PAGE);
-  };
 
-  // the wave's 32 dims x 8 heads of q: register pair g holds dims 2g, 2g + 1 (lane n of a row: dim 2g + n / 8, head n % 8)
-  double qreg[16];
-  {
-    const uint32_t* qw = A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + wave * 32) * EX_COLS + (lane & 15);
+  // The two roles meet at three barriers per step.  In step s the score waves take tile s through [K rows -> LDS |
+  // scores | weights]; the value waves add tile s - 1 (whose weights the third barrier of step s - 1 published) in three
+  // pieces, one per interval, so that neither role waits long for the other and the vector unit always has work of
+  // both kinds to choose from (4 waves per SIMD, 2 of each).
+  if (!value_role) {
+    // the wave's 32 dims x 8 heads of q: register pair g holds dims 2g, 2g + 1 (lane n of a row: dim 2g + n / 8, head n % 8)
+    double qreg[16];
+    {
+      const uint32_t* qw = A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + w8 * 32) * EX_COLS + (lane & 15);
 #pragma unroll
-    for (int g = 0; g < 16; g++) qreg[g] = f64_from_high(qw[g * 16]);
+      for (int g = 0; g < 16; g++) qreg[g] = f64_from_high(qw[g * 16]);
+    }
+    auto load_k = [&](int tile, uint4 (&kr)[EX_TILE_PAGES]) {      // round r of the 512 threads covers page r of the tile (8 KiB)
+#pragma unroll
+      for (int r = 0; r < EX_TILE_PAGES; r++) kr[r] = ld16(A.kc + page_base(tile * EX_TILE_PAGES + r) + tid8 * 8);
+    };
+    double l_lane = 0.0;            // wave = head: this lane's share of the sum of weights
+    double mref = -INFINITY;        // wave = head: the reference exponent
+    uint4 kpre[EX_TILE_PAGES];      // K of the next tile, requested a whole step ahead
+    if (ntiles > 0) load_k(0, kpre);
+    for (int tile = 0; tile <= ntiles && ntiles > 0; tile++) {      // (an empty page range: neither role enters its loop)
+      const bool live = tile < ntiles;                             // the last step only drains the value waves
+      if (live) {
+#pragma unroll
+        for (int r = 0; r < EX_TILE_PAGES; r++)
+          *(uint4*)(ktile + (r * ATT_PAGE + (tid8 >> 5)) * EX_KROW + (tid8 & 31) * 16) = kpre[r];
+      }
+      __syncthreads();
+      if (live) {
+        load_k(min(tile + 1, ntiles - 1), kpre);         // unconditional (the last tile again), so that the waits stay countable
+        // ---- scores: lane = token, this wave's 32 dims
+        double sacc[EX_COLS];
+#pragma unroll
+        for (int c = 0; c < EX_COLS; c++) sacc[c] = 0.0;
+        const uint4* krow = (const uint4*)(ktile + lane * EX_KROW + w8 * 64);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint4 kk = krow[i];
+          const uint32_t w[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+          for (int wi = 0; wi < 4; wi++) {
+            fmac8_bcast<0>(sacc, qreg[i * 4 + wi], bf16lo_to_f64(w[wi]));
+            fmac8_bcast<1>(sacc, qreg[i * 4 + wi], bf16hi_to_f64(w[wi]));
+          }
+        }
+#pragma unroll
+        for (int c = 0; c < EX_COLS; c++) xch[w8][c][lane] = sacc[c];
+      }
+      __syncthreads();
+      if (live) {
+        // ---- weights: wave = head
+        double s = 0.0;
+#pragma unroll
+        for (int w2 = 0; w2 < EX_SW; w2++) s += xch[w2][w8][lane];
+        s *= (double)A.scale;
+        const int tok = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + lane;
+        const bool valid = tok < lim;
+        const float smax = wave_max(valid ? (float)s : -INFINITY);
+        double alpha = 1.0;
+        if (smax > -INFINITY && (mref == -INFINITY || (double)smax > mref + EX_REF_SLACK)) {      // wave-uniform, rare after the first tile
+          if (mref != -INFINITY) { alpha = exp(mref - (double)smax); l_lane *= alpha; }
+          mref = (double)smax;
+        }
+        const double p = valid ? exp(s - mref) : 0.0;
+        l_lane += p;
+        lds_p[tile & 1][lane][w8] = p;
+        if (lane == 0) {
+          lds_alpha[tile & 1][w8] = alpha;
+          if (alpha != 1.0) lds_rescale[tile & 1] = 1;
+        }
+      }
+      __syncthreads();
+    }
+    const double lt = wave_sum_f64(l_lane);
+    if (lane == 0) { lds_l[w8] = lt; lds_m[w8] = mref; }
   }
 
   double acc[EX_COLS][4];
@@ -134,114 +204,77 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   for (int c = 0; c < EX_COLS; c++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[c][j] = 0.0;
-  double l_lane = 0.0;            // wave = head: this lane's share of the sum of weights
-  double mref = -INFINITY;        // wave = head: the reference exponent
-
-  // K and V of the next tile are requested a whole tile ahead (a tile's work is shorter than a trip to memory under load)
-  uint4 kpre[EX_TILE_PAGES], vcur[4], vpre[4];
-  if (ntiles > 0) { load_k(0, kpre); load_v(0, vpre); }
-  for (int tile = 0; tile < ntiles; tile++) {
+  if (value_role) {
+    // wave: tokens 8 * w8 .. + 8 of a tile; lane: dims lane + 64 j.  vreg[j] holds the 8 tokens of dim lane + 64 j and is
+    // requested again, for the next tile, as soon as the piece that uses it is done: every load has a step to arrive
+    uint4 vreg[4];
+    auto load_v = [&](int tile, int j) {
+      const int64_t base = page_base(tile * EX_TILE_PAGES + (w8 >> 1)) + (w8 & 1) * 8;
+      vreg[j] = ld16(A.vc + base + (lane + 64 * j) * ATT_PAGE);
+    };
+    if (ntiles > 0) {
 #pragma unroll
-    for (int r = 0; r < EX_TILE_PAGES; r++)
-      *(uint4*)(ktile + (r * ATT_PAGE + (threadIdx.x >> 5)) * EX_KROW + (threadIdx.x & 31) * 16) = kpre[r];
-#pragma unroll
-    for (int j = 0; j < 4; j++) vcur[j] = vpre[j];
-    if (threadIdx.x == 0) lds_rescale[tile & 1] = 0;      // read two barriers back at the latest; set again behind the next barrier
-    __syncthreads();
-    if (tile + 1 < ntiles) { load_k(tile + 1, kpre); load_v(tile + 1, vpre); }
-
-    // ---- scores: lane = token, this wave's 32 dims
-    {
-      double sacc[EX_COLS];
-#pragma unroll
-      for (int c = 0; c < EX_COLS; c++) sacc[c] = 0.0;
-      const uint4* krow = (const uint4*)(ktile + lane * EX_KROW + wave * 64);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const uint4 kk = krow[i];
-        const uint32_t w[4] = {kk.x, kk.y, kk.z, kk.w};
-#pragma unroll
-        for (int wi = 0; wi < 4; wi++) {
-          fmac8_bcast<0>(sacc, qreg[i * 4 + wi], bf16lo_to_f64(w[wi]));
-          fmac8_bcast<1>(sacc, qreg[i * 4 + wi], bf16hi_to_f64(w[wi]));
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < EX_COLS; c++) xch[wave][c][lane] = sacc[c];
+      for (int j = 0; j < 4; j++) load_v(0, j);
     }
-    __syncthreads();
-
-    // ---- weights: wave = head
-    {
-      double s = 0.0;
-#pragma unroll
-      for (int w2 = 0; w2 < EX_WAVES; w2++) s += xch[w2][wave][lane];
-      s *= (double)A.scale;
-      const int tok = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + lane;
-      const bool valid = tok < lim;
-      const float smax = wave_max(valid ? (float)s : -INFINITY);
-      double alpha = 1.0;
-      if (smax > -INFINITY && (mref == -INFINITY || (double)smax > mref + EX_REF_SLACK)) {      // wave-uniform, rare after the first tile
-        if (mref != -INFINITY) { alpha = exp(mref - (double)smax); l_lane *= alpha; }
-        mref = (double)smax;
-      }
-      const double p = valid ? exp(s - mref) : 0.0;
-      l_lane += p;
-      lds_p[lane][wave] = p;
-      if (lane == 0) {
-        lds_alpha[wave] = alpha;
-        if (alpha != 1.0) lds_rescale[tile & 1] = 1;
-      }
-    }
-    __syncthreads();
-
-    // ---- values: wave = 8 tokens, lane = 4 dims
-    {
-      // a head whose reference exponent moved in this tile (first tile aside: rare) rescales what was summed under the old one
-      if (__builtin_amdgcn_readfirstlane(lds_rescale[tile & 1])) {
-#pragma unroll
-        for (int c = 0; c < EX_COLS; c++) {
-          const double al = lds_alpha[c];
-#pragma unroll
-          for (int j = 0; j < 4; j++) acc[c][j] *= al;
-        }
-      }
-      // the weights of this wave's 8 tokens: pair h holds tokens 2h, 2h + 1 (lane n of a row: token 2h + n / 8, head n % 8)
-      double preg[4];
-#pragma unroll
-      for (int h = 0; h < 4; h++) preg[h] = lds_p[wave * 8 + 2 * h + ((lane & 15) >> 3)][lane & 7];
-      const int tok0 = (p_begin + tile * EX_TILE_PAGES) * ATT_PAGE + wave * 8;
-      const uint32_t vw[4][4] = {{vcur[0].x, vcur[0].y, vcur[0].z, vcur[0].w}, {vcur[1].x, vcur[1].y, vcur[1].z, vcur[1].w},
-                                 {vcur[2].x, vcur[2].y, vcur[2].z, vcur[2].w}, {vcur[3].x, vcur[3].y, vcur[3].z, vcur[3].w}};
-      // a token past the context has weight 0, but what its cache slot holds need not be a number: it enters as 0
-      // (only the tile that holds the end of the context pays for the test)
-      auto values = [&](auto tail_c) {
+    double preg[4];
+    for (int step = 0; step <= ntiles && ntiles > 0; step++) {
+      const int t = step - 1;                                      // the tile whose values are added in this step
+      const bool live = t >= 0;
+      const int tok0 = (p_begin + t * EX_TILE_PAGES) * ATT_PAGE + w8 * 8;
+      const bool tail = tok0 + 8 > lim;
+      // one dim-group j of the tile: 8 tokens x 8 heads; a token past the context has weight 0, but what its cache slot
+      // holds need not be a number: it enters as 0 (only the tile that holds the end of the context pays for the test)
+      auto piece = [&](int j, auto tail_c) {
         constexpr bool TAIL = decltype(tail_c)::value;
+        const uint32_t vw[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+        double a[EX_COLS];
+#pragma unroll
+        for (int c = 0; c < EX_COLS; c++) a[c] = acc[c][j];
 #pragma unroll
         for (int h = 0; h < 4; h++) {
           const bool in0 = !TAIL || tok0 + 2 * h < lim, in1 = !TAIL || tok0 + 2 * h + 1 < lim;
+          fmac8_bcast<0>(a, preg[h], in0 ? bf16lo_to_f64(vw[h]) : 0.0);
+          fmac8_bcast<1>(a, preg[h], in1 ? bf16hi_to_f64(vw[h]) : 0.0);
+        }
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            double a[EX_COLS];
+        for (int c = 0; c < EX_COLS; c++) acc[c][j] = a[c];
+      };
+      // the piece's arithmetic, then the request for the same dims of the next tile (issued in every step, for the last
+      // tile again behind the end: a load behind a branch would leave the number of loads in flight unknown at the waits)
+      auto pieces = [&](int j) {
+        if (live) {
+          if (tail) piece(j, std::true_type{});
+          else piece(j, std::false_type{});
+        }
+        load_v(min(t + 1, ntiles - 1), j);
+      };
+      if (live) {
+        // a head whose reference exponent moved in this tile (first tile aside: rare) rescales what was summed under the old one
+        if (__builtin_amdgcn_readfirstlane(lds_rescale[t & 1])) {
 #pragma unroll
-            for (int c = 0; c < EX_COLS; c++) a[c] = acc[c][j];
-            fmac8_bcast<0>(a, preg[h], in0 ? bf16lo_to_f64(vw[j][h]) : 0.0);
-            fmac8_bcast<1>(a, preg[h], in1 ? bf16hi_to_f64(vw[j][h]) : 0.0);
+          for (int c = 0; c < EX_COLS; c++) {
+            const double al = lds_alpha[t & 1][c];
 #pragma unroll
-            for (int c = 0; c < EX_COLS; c++) acc[c][j] = a[c];
+            for (int j = 0; j < 4; j++) acc[c][j] *= al;
           }
         }
-      };
-      if (tok0 + 8 > lim) values(std::true_type{});
-      else values(std::false_type{});
+        // the weights of this wave's 8 tokens: pair h holds tokens 2h, 2h + 1 (lane n of a row: token 2h + n / 8, head n % 8)
+#pragma unroll
+        for (int h = 0; h < 4; h++) preg[h] = lds_p[t & 1][w8 * 8 + 2 * h + ((lane & 15) >> 3)][lane & 7];
+      }
+      pieces(0);
+      __syncthreads();
+      // the flag of tile t has been read by every value wave; tile t + 2 sets it again two steps from now
+      if (live && w8 == 0 && lane == 0) lds_rescale[t & 1] = 0;
+      pieces(1);
+      pieces(2);
+      __syncthreads();
+      pieces(3);
+      __syncthreads();
     }
   }
 
-  // ---- the heads' sums and reference exponents, then the accumulators of the 8 waves as ((0+4)+(2+6)) + ((1+5)+(3+7))
-  {
-    const double lt = wave_sum_f64(l_lane);
-    if (lane == 0) { lds_l[wave] = lt; lds_m[wave] = mref; }
-  }
+  // ---- the accumulators of the 8 value waves as ((0+4)+(2+6)) + ((1+5)+(3+7)); every wave of the workgroup walks the barriers
   __syncthreads();
   double* red = (double*)lds_raw;
   auto put = [&](int slot) {
@@ -256,17 +289,17 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 #pragma unroll
       for (int j = 0; j < 4; j++) acc[c][j] += red[((slot * EX_COLS + c) * 4 + j) * 64 + lane];
   };
-  if (wave >= 4) put(wave - 4);
+  if (value_role && w8 >= 4) put(w8 - 4);
   __syncthreads();
-  if (wave < 4) get(wave);
+  if (value_role && w8 < 4) get(w8);
   __syncthreads();
-  if (wave == 2 || wave == 3) put(wave - 2);
+  if (value_role && (w8 == 2 || w8 == 3)) put(w8 - 2);
   __syncthreads();
-  if (wave < 2) get(wave);
+  if (value_role && w8 < 2) get(w8);
   __syncthreads();
-  if (wave == 1) put(0);
+  if (value_role && w8 == 1) put(0);
   __syncthreads();
-  if (wave != 0) return;
+  if (!value_role || w8 != 0) return;
   get(0);
 
   if (A.splits == 1) {
