@@ -52,8 +52,11 @@ __device__ __forceinline__ double bf16lo_to_f64(uint32_t w) { return (double)__u
 __device__ __forceinline__ double bf16hi_to_f64(uint32_t w) { return (double)__uint_as_float(w & 0xffff0000u); }
 
 // acc[c] += bsrc(lane 8 * E + c of the lane's row of 16) * v for the 8 columns c: eight v_fmac_f64 whose first factor is
-// read through the DPP row broadcast (the only DPP form of the f64 unit).  The two idle cycles in front keep the
-// distance a DPP read needs from a vector instruction that may have written `bsrc` just before.
+// read through the DPP row broadcast (the only DPP form of the f64 unit).  The compiler does not see a DPP instruction
+// inside the asm block and inserts none of the idle cycles one needs: the two in front keep the distance from a vector
+// instruction that may have written `bsrc` just before; the five a DPP read needs behind a vector instruction that
+// writes the execution mask (v_cmpx) are not paid for, because the compiled kernel contains no such instruction —
+// tests/test_isa_checks.py compiles this file and fails if one appears.
 template <int E>
 __device__ __forceinline__ void fmac8_bcast(double (&a)[EX_COLS], double bsrc, double v) {
   static_assert(E == 0 || E == 1, "half of the row");

@@ -1,0 +1,62 @@
+"""Properties of the compiled gfx950 code that the source relies on but the compiler does not guarantee (CPU only: hipcc
+cross-compiles without a GPU).
+
+attn_exact.hip issues v_fmac_f64 with a DPP operand from inline assembly.  The compiler's hazard recognizer does not look
+into asm blocks, so the idle cycles a DPP read needs are written by hand (two, in front of every group, against a vector
+write of the DPP source) or avoided by construction (five behind a vector instruction that writes EXEC: the kernel must
+not contain one)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "bunker_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+@pytest.fixture(scope="module")
+def exact_asm(tmp_path_factory):
+    if not (os.path.exists(HIPCC) or shutil.which(HIPCC)):
+        pytest.skip("hipcc not found")
+    out = str(tmp_path_factory.mktemp("isa") / "attn_exact.s")
+    flags = re.search(r"^HIPFLAGS \?= (.*?)(?<!\\)$", open(os.path.join(CSRC, "Makefile")).read(), flags=re.M | re.S).group(1)
+    flags = flags.replace("\\\n", " ").replace("$(ARCH)", "gfx950").split()
+    subprocess.check_call([HIPCC, *flags, "-S", "--cuda-device-only", "-o", out, os.path.join(CSRC, "attn_exact.hip")],
+                          stderr=subprocess.DEVNULL)
+    return open(out).read()
+
+
+def _kernels(asm):
+    """name -> body of every kernel of the file"""
+    out = {}
+    for m in re.finditer(r"^(_ZN2bk\w+):[^\n]*\n(.*?)^\.Lfunc_end", asm, flags=re.M | re.S):
+        out[m.group(1)] = m.group(2)
+    return out
+
+
+def test_dpp_groups_in_the_exact_attention_are_hazard_free(exact_asm):
+    ks = {k: v for k, v in _kernels(exact_asm).items() if "attn_exact_kernel" in k}
+    assert len(ks) == 2                                         # the plain and the nontemporal instantiation
+    for name, body in ks.items():
+        n_dpp = len(re.findall(r"\bv_fmac_f64_dpp\b", body))
+        assert n_dpp >= 512 and n_dpp % 8 == 0, (name, n_dpp)
+        # no vector instruction writes EXEC anywhere in the kernel
+        assert not re.search(r"\bv_cmpx", body), name
+        # every DPP instruction sits in an asm block that opens with the two idle cycles, eight to a block
+        blocks = re.findall(r";;#ASMSTART\n(.*?);;#ASMEND", body, flags=re.S)
+        dpp_blocks = [b for b in blocks if "v_fmac_f64_dpp" in b]
+        assert sum(len(re.findall(r"v_fmac_f64_dpp", b)) for b in dpp_blocks) == n_dpp
+        for b in dpp_blocks:
+            lines = [l.strip() for l in b.strip().splitlines()]
+            assert lines[0] == "s_nop 1" and len(lines) == 9 and all(l.startswith("v_fmac_f64_dpp") for l in lines[1:]), b
+            # the broadcast source is read, never written, inside the block
+            src = {re.match(r"v_fmac_f64_dpp (v\[\d+:\d+\]), (v\[\d+:\d+\]),", l).group(2) for l in lines[1:]}
+            dst = {re.match(r"v_fmac_f64_dpp (v\[\d+:\d+\]),", l).group(1) for l in lines[1:]}
+            assert len(src) == 1 and not (src & dst), b
+        # no register spills: the kernel is sized for 128 registers per lane and 4 waves per SIMD
+        meta = re.search(r"\.name:\s+%s\n(.*?)\.wavefront_size" % re.escape(name), exact_asm, flags=re.S).group(1)
+        assert int(re.search(r"\.vgpr_count:\s+(\d+)", meta).group(1)) <= 128
+        assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0
