@@ -292,18 +292,17 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 #pragma unroll
       for (int j = 0; j < 4; j++) acc[c][j] += red[((slot * EX_COLS + c) * 4 + j) * 64 + lane];
   };
+  // a wave puts into the slot it alone read in the round before, so one barrier per round is enough
   if (value_role && w8 >= 4) put(w8 - 4);
   __syncthreads();
   if (value_role && w8 < 4) get(w8);
+  if (value_role && (w8 == 2 || w8 == 3)) put(w8);
   __syncthreads();
-  if (value_role && (w8 == 2 || w8 == 3)) put(w8 - 2);
-  __syncthreads();
-  if (value_role && w8 < 2) get(w8);
-  __syncthreads();
-  if (value_role && w8 == 1) put(0);
+  if (value_role && w8 < 2) get(w8 + 2);
+  if (value_role && w8 == 1) put(1);
   __syncthreads();
   if (!value_role || w8 != 0) return;
-  get(0);
+  get(1);
 
   if (A.splits == 1) {
 #pragma unroll
@@ -340,6 +339,7 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 
 // Merge of the f64 split partials: one workgroup per (head, query row), thread = dim.  The weights exp(ref_s - max ref)
 // of all splits are computed side by side first (thread = split), the partial outputs are then added in split order.
+template <int PRE>
 __global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
   __shared__ double wsh[ATT_MAX_SPLITS];
   __shared__ float redm[4];
@@ -356,6 +356,14 @@ __global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
   const bool has = d < nsplit;
   const double ms = has ? A.part_ml64[((p0 + d) * EX_COLS + c) * 2] : -INFINITY;
   const double ls = has ? A.part_ml64[((p0 + d) * EX_COLS + c) * 2 + 1] : 0.0;
+  const uint16_t gbits = A.gate ? A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d] : (uint16_t)0;
+  // The partial outputs of the first PRE splits (4, 16 or 64, by the split count of the launch) are requested right behind the exponents, all at once and
+  // unconditionally (a split past the last one reads the last one again and gets weight 0): they travel while the
+  // weights are worked out, and the kernel waits for memory once instead of once per pair of splits.
+  const double* po = A.part_o64 + (p0 * EX_COLS + c) * ATT_HD + d;
+  double pv[PRE];
+#pragma unroll
+  for (int s = 0; s < PRE; s++) pv[s] = po[(int64_t)min(s, nsplit - 1) * EX_COLS * ATT_HD];
   // the reference exponents are f32 values (or -inf), so their maximum is found in f32 without loss
   float Mf = wave_max((float)ms);
   if ((d & 63) == 0) redm[d >> 6] = Mf;
@@ -367,10 +375,14 @@ __global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
   if ((d & 63) == 0) redl[d >> 6] = L;
   __syncthreads();
   L = (redl[0] + redl[1]) + (redl[2] + redl[3]);
-  const float gsig = A.gate ? sigmoid_f64(bf16_to_f32(A.gate[(int64_t)b * A.gate_bstride + (int64_t)head * A.gate_hstride + d])) : 1.0f;
-  const double* po = A.part_o64 + (p0 * EX_COLS + c) * ATT_HD + d;
+  const float gsig = A.gate ? sigmoid_f64(bf16_to_f32(gbits)) : 1.0f;
   double o0 = 0.0, o1 = 0.0;
-  int s = 0;
+#pragma unroll
+  for (int s = 0; s < PRE; s += 2) {
+    o0 = fma(pv[s], wsh[s], o0);              // wsh[s] = 0 for s >= nsplit
+    o1 = fma(pv[s + 1], wsh[s + 1], o1);
+  }
+  int s = PRE;
   for (; s + 2 <= nsplit; s += 2) {
     o0 = fma(po[(int64_t)(s + 0) * EX_COLS * ATT_HD], wsh[s + 0], o0);
     o1 = fma(po[(int64_t)(s + 1) * EX_COLS * ATT_HD], wsh[s + 1], o1);
@@ -423,7 +435,12 @@ int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void*
   const dim3 block(EX_THREADS);
   if (nt) hipLaunchKernelGGL((attn_exact_kernel<true>), grid, block, 0, stream(), A);
   else hipLaunchKernelGGL((attn_exact_kernel<false>), grid, block, 0, stream(), A);
-  if (A.splits > 1) hipLaunchKernelGGL(attn_exact_merge_kernel, dim3(A.NH, batch), dim3(256), 0, stream(), A);
+  if (A.splits > 1) {
+    const dim3 mgrid(A.NH, batch);
+    if (A.splits <= 4) hipLaunchKernelGGL(attn_exact_merge_kernel<4>, mgrid, dim3(256), 0, stream(), A);
+    else if (A.splits <= 16) hipLaunchKernelGGL(attn_exact_merge_kernel<16>, mgrid, dim3(256), 0, stream(), A);
+    else hipLaunchKernelGGL(attn_exact_merge_kernel<64>, mgrid, dim3(256), 0, stream(), A);
+  }
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
