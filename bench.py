@@ -270,7 +270,17 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     wall = time.perf_counter() - t0
     pf.close()
     out["prefill"] = {"prompt_tokens": n_prompt, "chunk": chunk, "chunks_in_flight": 2, "tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
-                      "first_generated_token": tok}
+                      "first_generated_token": tok, "attention": "double precision (the state T decode steps leave, bit for bit)"}
+    runner.ATTN_EXACT = False
+    pf = prefill.Prefill(D, envs[0], chunk=chunk)
+    runner.ATTN_EXACT = True
+    pf.run(prompt, 0, 0)
+    rt.cuSync()
+    t0 = time.perf_counter()
+    pf.run(prompt, 0, 0)
+    wall = time.perf_counter() - t0
+    pf.close()
+    out["prefill"]["with_bf16_mfma_attention"] = {"tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2)}
     for env in envs:
         env.close()
     # the reference model's own dimensions (src/model.ts:14-18), random Q4_K weights, KV at 4096: batch 1 only

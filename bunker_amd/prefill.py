@@ -25,6 +25,7 @@ import numpy as np
 
 from . import runtime as rt
 from .model import Dims, L
+from . import runner as _runner
 from .runner import DecodeEnv, Q8OUT_MIN_BATCH
 
 
@@ -51,6 +52,7 @@ class Prefill:
         if chunk < 1 or chunk > 4096:
             raise ValueError("Prefill: chunk must be 1..4096 tokens")
         self.D, self.env, self.chunk, self.on_attention = D, env, int(chunk), on_attention
+        self.attn_exact = bool(_runner.ATTN_EXACT)       # double-precision attention, or the matrix-instruction form (runner.ATTN_EXACT)
         self._owned: list[int] = []
         in_flight = 2 if overlap is True else max(int(overlap), 1)
         self._streams = [rt.Stream() for _ in range(in_flight)] if in_flight > 1 else []
@@ -100,7 +102,8 @@ class Prefill:
             "gdn": c(f"gdn_prefill LVH={D.LVH} T={T}"),
             "gdn_out": c(f"gemv_fused K={D.ZD} pro=1 G=1 N0={D.H} epi0=2" + bp),
             "fa_in": c(f"gemv_fused K={D.H} pro=2 G=3 N0={D.QGATE} epi0=1 N1={D.KV_DIM} epi1=1 N2={D.KV_DIM} epi2=1" + bp),
-            "fa": c(f"fa2_prefill HD={D.HD} NH={D.NH} NKV={D.NKV} MAX_LEN={D.MAX_LEN} ROT_HALF={D.ROT_HALF} T={T}"),
+            "fa": c(f"fa2_prefill HD={D.HD} NH={D.NH} NKV={D.NKV} MAX_LEN={D.MAX_LEN} ROT_HALF={D.ROT_HALF} T={T}"
+                    + ("" if self.attn_exact else " exact=0")),
             "fa_out": c(f"gemv_fused K={D.NH * D.HD} pro=1 G=1 N0={D.H} epi0=2" + bp),
         }
         # batched form: the matmul leaves the SwiGLU result as Q8_1 blocks too and the down projection reads those

@@ -1,7 +1,7 @@
 """Prompt processing on the GPU against token-by-token runs of the CPU checker.
 
 conv1d_prefill and gdn_prefill must give the bits of T single-token steps; fa2_prefill must leave the same cache
-bytes and attention outputs within 2e-2; the whole prefill must leave the state and the last token's logits of a
+bytes and attention outputs with equal bits (exact=0: within 2e-2); the whole prefill must leave the state and the last token's logits of a
 token-by-token run (the checker continues from the GPU's attention outputs, as in the decode tests), and decoding
 must continue from that state as if every prompt token had been decoded."""
 import numpy as np
@@ -72,7 +72,7 @@ def test_gdn_prefill_is_T_decode_steps(orc, Hg, T):
 
 @pytest.mark.parametrize("T,pos0,splits", [(6, 0, 0), (37, 12, 0), (37, 60, 3), (2, 15, 2)])
 def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits):
-    """Two consecutive tokens per workgroup (their heads side by side in the 16 columns of the products, each column
+    """The matrix-instruction form (exact=0): two consecutive tokens per workgroup (their heads side by side in the 16 columns of the products, each column
     masked to its own length) against one token per workgroup: the same output and cache bytes."""
     print(f"fa2_prefill pairs T={T} pos0={pos0} splits={splits}", flush=True)
     g = synth.rng(870 + T + pos0)
@@ -92,7 +92,7 @@ def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits
         dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
         dout = rt.cuAlloc(T * NH * HD * 2)
         rt.cuMemset(dout, 0xff, T * NH * HD * 2)
-        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} pair={pair}" + (f" splits={splits}" if splits else ""),
+        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} pair={pair} exact=0" + (f" splits={splits}" if splits else ""),
                 ptrs + [dkc, dvc, dout])
         res.append((rt.from_device(dout, (T, NH, HD), np.uint16), rt.from_device(dkc, kc.shape, np.uint16),
                     rt.from_device(dvc, (pages, NKV, HD, 16), np.uint16)))
@@ -105,9 +105,11 @@ def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits
         rt.cuFree(p)
 
 
+@pytest.mark.parametrize("exact", [1, 0])
 @pytest.mark.parametrize("T,pos0", [(1, 0), (5, 0), (37, 12)])
-def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0):
-    print(f"fa2_prefill T={T} pos0={pos0}", flush=True)
+def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0, exact):
+    """exact=1 (the default): every output row has the checker's bits; exact=0: within 2e-2."""
+    print(f"fa2_prefill T={T} pos0={pos0} exact={exact}", flush=True)
     g = synth.rng(840 + T)
     NH, NKV, HD, HALF, MAXL = 16, 2, 256, 32, 128
     pages = MAXL // 16
@@ -123,7 +125,7 @@ def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0):
     dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
     dout = rt.cuAlloc(T * NH * HD * 2)
     ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
-    _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T}", ptrs + [dkc, dvc, dout])
+    _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T}" + ("" if exact else " exact=0"), ptrs + [dkc, dvc, dout])
     out = rt.from_device(dout, (T, NH, HD), np.uint16)
     worst = 0.0
     for t in range(T):
@@ -133,7 +135,7 @@ def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0):
         ro, _ = orc.attn_decode_paged(qn, kc, vc, table[None], np.array([pos[t] + 1], np.int32), 1, NH, NKV, HD, 16,
                                       gate=qgate[t].ravel()[HD:], gate_bstride=0, gate_hstride=2 * HD)
         worst = max(worst, float(np.abs(f32(out[t]).astype(np.float64) - f32(ro[0])).max()))
-    assert worst <= 2e-2, worst
+    assert worst <= (0.0 if exact else 2e-2), worst
     kc_d = rt.from_device(dkc, kc.shape, np.uint16)
     vc_d = rt.from_device(dvc, (2 * pages, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
     assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
@@ -167,7 +169,7 @@ def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
     for t in range(n_prompt):
         inj = {l: captured[l][t][None] for l in captured}
         idx, rv, rlogits = ref.step([prompt[t]], [t], attn_override=inj)
-    assert max(ref.attn_err) <= 2e-2, max(ref.attn_err)
+    assert max(ref.attn_err) == 0.0, max(ref.attn_err)         # double-precision attention: the checker's bits
     assert np.array_equal(glogits.view(np.uint32), rlogits[0].view(np.uint32)), \
         f"{int((glogits != rlogits[0]).sum())} logits differ, worst {np.abs(glogits - rlogits[0]).max():.3e}"
     assert tok == int(idx[0]) and np.float32(val).view(np.uint32) == rv[0].view(np.uint32)
@@ -201,7 +203,7 @@ def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
         gt, gv = loop.tokens()
         assert gt[step][seq] == idx[0] and gv[step][seq].view(np.uint32) == rv[0].view(np.uint32), (step, gt[step], idx)
         toks, pos = idx, pos + 1
-    assert max(ref.attn_err) <= 2e-2
+    assert max(ref.attn_err) == 0.0
     env.close()
 
 
