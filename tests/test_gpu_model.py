@@ -169,3 +169,26 @@ def test_reference_dims_decode(orc, batch):
     starts = [(113 * i + 9) % D.VOCAB for i in range(batch)]
     toks, vals = _strict_decode(D, W, S, starts, 30, 3, use_graph=True, fused=True, check=[0, batch - 1] if batch > 1 else None)
     assert toks.shape == (3, batch)
+
+
+@pytest.mark.parametrize("seed", [100, 104, 106, 109])
+def test_free_running_decode_equals_the_checker_over_seeds(orc, seed):
+    """No injection, no step-by-step resynchronisation: 4 sequences decode 23 tokens on the GPU (fused partition, replayed
+    graph) and on the CPU from the same weights and state; tokens and winning logits must be equal although the top-1 /
+    top-2 margins of random weights fall below 1e-3 (seeds 106, 109)."""
+    from oracle.model_ref import RefModel
+    D, B, steps = TINY, 4, 23
+    pos0 = 5 + seed % 30
+    W = synth_model.synth_weights(D, seed=seed)
+    S = synth_model.synth_state(D, batch=B, seed=seed + 1)
+    g = model.buildModelGraph(D, B)
+    env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+    starts = [(17 + 911 * i + seed) % D.VOCAB for i in range(B)]
+    loop = runner.DeviceLoop(g, env, B, starts, pos0, max_steps=steps, use_graph=True, partition=runner.fusedPartition(g))
+    loop.step(steps)
+    toks, vals = loop.tokens()
+    ref = RefModel(D, W, S, batch=B)
+    rtok, rv = ref.decode(starts, pos0, steps)
+    print(f"seed {seed}: min margin {np.min(ref.margins):.5f}", flush=True)
+    assert np.array_equal(toks, rtok) and np.array_equal(vals.view(np.uint32), rv.view(np.uint32))
+    loop.close(); env.close()
