@@ -331,6 +331,15 @@ static int run_argmax(Kernel& k, const uint64_t* s) {
   return launch_argmax(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1));
 }
 
+// ---- op: argmax_feed = argmax + advance + the next step's embed (device-resident loop: two launches instead of four)
+// slots: logits, val, idx, token ids, positions, history, counters (int32 [batch], one per sequence), embed.weight, x (next step's input)
+// params: VOCAB, H, batch, max_steps, max_pos
+static int run_argmax_feed(Kernel& k, const uint64_t* s) {
+  return launch_argmax_feed(P<float>(s[0]), P<float>(s[1]), P<int32_t>(s[2]), k.scratch, (int)k.get("VOCAB", 0), (int)k.get("batch", 1),
+                            P<int32_t>(s[3]), P<int32_t>(s[4]), P<int32_t>(s[5]), P<int32_t>(s[6]), (int)k.get("max_steps", 0),
+                            (int)k.get("max_pos", 0), P<void>(s[7]), P<void>(s[8]), (int)k.get("H", 0));
+}
+
 // ---- op: advance   slots: argmax idx, argmax val, token ids, positions, history, counter    params: batch, max_steps, max_pos
 // (max_pos = the cache capacity MAX_LEN: positions are not advanced past it, and the cache writers skip a position that reached it)
 static int run_advance(Kernel& k, const uint64_t* s) {
@@ -430,6 +439,15 @@ static int build_kernel(Kernel& k) {
     BK_REQUIRE(batch >= 1 && V >= 1, "argmax: bad VOCAB/batch");
     if ((rc = alloc_scratch(k, argmax_workspace_bytes(V, batch)))) return rc;
     k.run = run_argmax; k.nslots = 3;
+    return BK_OK;
+  }
+  if (k.op == "argmax_feed") {
+    for (const char* p : {"VOCAB", "H", "max_steps", "max_pos"})
+      if ((rc = need(k, p))) return rc;
+    const int batch = (int)k.get("batch", 1), V = (int)k.get("VOCAB", 0);
+    BK_REQUIRE(batch >= 1 && V >= 1, "argmax_feed: bad VOCAB/batch");
+    if ((rc = alloc_scratch(k, argmax_workspace_bytes(V, batch)))) return rc;
+    k.run = run_argmax_feed; k.nslots = 9;
     return BK_OK;
   }
   if (k.op == "gemv_fused") return build_gemv_fused(k);

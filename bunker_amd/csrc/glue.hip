@@ -469,6 +469,61 @@ __global__ __launch_bounds__(256) void advance_kernel(const int32_t* __restrict_
   if (threadIdx.x == 0) counter[0] = c + 1;
 }
 
+// argmax's second stage, the token feedback above and the embedding of the next step's token in one launch (one
+// workgroup per sequence): what would be three launches of a few microseconds each between two tokens.  `counter` holds
+// one step count per sequence here (every workgroup advances its own).
+__global__ __launch_bounds__(256) void argmax_feed_kernel(const float* __restrict__ pv, const int32_t* __restrict__ pi,
+                                                          float* __restrict__ val, int32_t* __restrict__ idx, int ntiles,
+                                                          int32_t* __restrict__ ids, int32_t* __restrict__ pos,
+                                                          int32_t* __restrict__ hist, int32_t* __restrict__ counter, int batch,
+                                                          int max_steps, int max_pos, const uint16_t* __restrict__ E,
+                                                          uint16_t* __restrict__ x, int H, int vocab) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  __shared__ int s_id;
+  const int b = blockIdx.x;
+  float v = ARGMAX_INIT; int i = 0x7fffffff;
+  for (int t = threadIdx.x; t < ntiles; t += 256) argmax_merge(v, i, pv[(int64_t)b * ntiles + t], pi[(int64_t)b * ntiles + t]);
+  argmax_wave(v, i);
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = v; si[threadIdx.x >> 6] = i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; k++) argmax_merge(v, i, sv[k], si[k]);
+    i = (i == 0x7fffffff) ? 0 : i;          // nothing above -FLT_MAX: index 0, like the sequential scan
+    val[b] = v; idx[b] = i;
+    const int c = counter[b];
+    if (c < max_steps) {
+      hist[((int64_t)c * batch + b) * 2] = i;
+      hist[((int64_t)c * batch + b) * 2 + 1] = __float_as_int(v);
+    }
+    counter[b] = c + 1;
+    ids[b] = i;
+    const int p = pos[b];
+    if (p < max_pos) pos[b] = p + 1;      // positions stop at the cache capacity, as in advance_kernel
+    s_id = i < 0 ? 0 : (i >= vocab ? vocab - 1 : i);
+  }
+  __syncthreads();
+  const int id = s_id;
+  for (int e = threadIdx.x * 8; e < H; e += 256 * 8) *(uint4*)(x + (int64_t)b * H + e) = *(const uint4*)(E + (int64_t)id * H + e);
+}
+
+int launch_argmax_feed(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch, int32_t* ids, int32_t* pos,
+                       int32_t* hist, int32_t* counter, int max_steps, int max_pos, const void* E, void* x, int H) {
+  BK_REQUIRE(logits && val && idx && workspace && ids && pos && hist && counter && E && x, "argmax_feed: null pointer");
+  BK_REQUIRE(n > 0 && batch > 0 && batch <= 65535 && max_steps > 0 && max_pos > 0, "argmax_feed: bad n=%d batch=%d max_steps=%d max_pos=%d", n,
+             batch, max_steps, max_pos);
+  BK_REQUIRE(H > 0 && H % 8 == 0 && ((uintptr_t)E & 15) == 0 && ((uintptr_t)x & 15) == 0, "argmax_feed: H=%d must be a multiple of 8, rows 16-byte aligned", H);
+  const int ntiles = (n + ARGMAX_TILE - 1) / ARGMAX_TILE;
+  float* pv = (float*)workspace;
+  int32_t* pi = (int32_t*)(pv + (size_t)batch * ntiles);
+  const bool vec4 = n % 4 == 0 && ((uintptr_t)logits & 15) == 0;
+  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(ntiles, batch), dim3(256), 0, stream(), logits, pv, pi, n, ntiles, vec4);
+  hipLaunchKernelGGL(argmax_feed_kernel, dim3(batch), dim3(256), 0, stream(), pv, pi, val, idx, ntiles, ids, pos, hist, counter, batch,
+                     max_steps, max_pos, (const uint16_t*)E, (uint16_t*)x, H, n);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
 int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
                    int max_steps, int max_pos) {
   BK_REQUIRE(idx && val && ids && pos && hist && counter, "advance: null pointer");

@@ -70,6 +70,8 @@ int launch_rope(void* x, const float* cos_t, const float* sin_t, const int32_t* 
 size_t argmax_workspace_bytes(int n, int batch);
 int launch_argmax(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch);
 
+int launch_argmax_feed(const float* logits, float* val, int32_t* idx, void* workspace, int n, int batch, int32_t* ids, int32_t* pos,
+                       int32_t* hist, int32_t* counter, int max_steps, int max_pos, const void* E, void* x, int H);
 int launch_advance(const int32_t* idx, const float* val, int32_t* ids, int32_t* pos, int32_t* hist, int32_t* counter, int batch,
                    int max_steps, int max_pos);
 

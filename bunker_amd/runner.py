@@ -500,7 +500,7 @@ class DeviceLoop:
     """
 
     def __init__(self, graph: Graph, env: DecodeEnv, batch: int, start_tokens, start_pos, max_steps: int,
-                 partition: Partition | None = None, use_graph: bool = True):
+                 partition: Partition | None = None, use_graph: bool = True, feed: bool = True):
         if not env.inplace:
             raise ValueError("DeviceLoop needs DecodeEnv(inplace_state=True)")
         ids = np.asarray(start_tokens, np.int32).reshape(batch)
@@ -521,22 +521,39 @@ class DeviceLoop:
         self.d_ids = rt.to_device(ids)
         self.d_pos = rt.to_device(pos)
         self.d_hist = rt.cuAlloc(max_steps * batch * 8)
-        self.d_count = rt.to_device(np.zeros(1, np.int32))
+        self.d_count = rt.to_device(np.zeros(batch, np.int32))
         argmax = next(n for n in graph.nodes if n.op == "argmax")
         self.idx_ptr = env.resolve(argmax.outputs[1].tensorName)
         self.val_ptr = env.resolve(argmax.outputs[0].tensorName)
-        self.k_adv = rt.compileAndLoad(f"advance batch={batch} max_steps={max_steps} max_pos={max_len if max_len is not None else 2**31 - 1}")
+        max_pos = max_len if max_len is not None else 2**31 - 1
         self.launches = []
         for plan, k in self.compiled.schedule:
             args = [self.d_ids if a == "token_id" else self.d_pos if a == "pos" else env.resolve(a) for a in plan.args]
             self.launches.append((k, plan, args))
-        self.launches.append((self.k_adv, None, [self.idx_ptr, self.val_ptr, self.d_ids, self.d_pos, self.d_hist, self.d_count]))
+        # Between two tokens: argmax's second stage, the token feedback and the next token's embedding are one launch
+        # (argmax_feed) when the step begins with the embed node and ends with the argmax node on their own; the embed
+        # launch then runs once, in front of the first step.  Otherwise argmax, then `advance`.
+        self.first_only = []
+        first, last = self.launches[0][1], self.launches[-1][1]
+        if feed and len(first.group) == 1 and first.group[0].op == "embed" and len(last.group) == 1 and last.group[0].op == "argmax":
+            emb = first.group[0]
+            H, V = int(emb.params["H"]), int(emb.params["VOCAB"])
+            k_feed = rt.compileAndLoad(f"argmax_feed VOCAB={V} H={H} batch={batch} max_steps={max_steps} max_pos={max_pos}")
+            self.first_only = [self.launches[0]]
+            rt.unloadKernel(self.launches[-1][0])
+            self.launches = self.launches[1:-1]
+            self.launches.append((k_feed, None, [env.resolve(argmax.inputs[0].tensorName), self.val_ptr, self.idx_ptr, self.d_ids, self.d_pos,
+                                                 self.d_hist, self.d_count, env.resolve(emb.inputs[0].tensorName),
+                                                 env.resolve(emb.outputs[0].tensorName)]))
+        else:
+            self.k_adv = rt.compileAndLoad(f"advance batch={batch} max_steps={max_steps} max_pos={max_pos}")
+            self.launches.append((self.k_adv, None, [self.idx_ptr, self.val_ptr, self.d_ids, self.d_pos, self.d_hist, self.d_count]))
         self.graph_exec = None
         self.use_graph = use_graph
         self.steps_done = 0
 
-    def _enqueue(self):
-        for k, plan, args in self.launches:
+    def _enqueue(self, first: bool = False):
+        for k, plan, args in (self.first_only if first else []) + self.launches:
             rc = rt.cuLaunch(k, [1, 1, 1], [128, 1, 1], args)
             if rc != 0:
                 raise rt.BunkerError(f"{plan.name if plan else 'advance'}: {rt.last_error()} (rc={rc})")
@@ -551,7 +568,7 @@ class DeviceLoop:
                 self.graph_exec.launch()
             else:
                 # the first token runs eagerly (it also loads every kernel); the recording happens after it
-                self._enqueue()
+                self._enqueue(first=self.steps_done == 0)
                 if self.use_graph:
                     rt.cuSync()
                     with rt.Graph() as gr:
@@ -567,11 +584,12 @@ class DeviceLoop:
             self.graph_exec.destroy()
             self.graph_exec = None
         seen = set()
-        for k, _, _ in self.launches:
+        for k, _, _ in self.first_only + self.launches:
             if k.fn not in seen:
                 seen.add(k.fn)
                 rt.unloadKernel(k)
         self.launches = []
+        self.first_only = []
         for p in (self.d_ids, self.d_pos, self.d_hist, self.d_count):
             if p:
                 rt.cuFree(p)

@@ -192,3 +192,21 @@ def test_free_running_decode_equals_the_checker_over_seeds(orc, seed):
     print(f"seed {seed}: min margin {np.min(ref.margins):.5f}", flush=True)
     assert np.array_equal(toks, rtok) and np.array_equal(vals.view(np.uint32), rv.view(np.uint32))
     loop.close(); env.close()
+
+
+def test_token_feedback_forms_agree(orc):
+    """argmax_feed (argmax's second stage + token feedback + the next embedding in one launch) against argmax, advance and the
+    step's own embed launch: same tokens, same logits."""
+    D, B, steps = TINY, 3, 9
+    W = synth_model.synth_weights(D, seed=41)
+    S = synth_model.synth_state(D, batch=B, seed=42)
+    g = model.buildModelGraph(D, B)
+    res = []
+    for feed in (True, False):
+        env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+        loop = runner.DeviceLoop(g, env, B, [3, 700, 41], 20, max_steps=steps, use_graph=True, partition=runner.fusedPartition(g), feed=feed)
+        assert (len(loop.first_only) == 1) == feed
+        loop.step(steps)
+        res.append(loop.tokens())
+        loop.close(); env.close()
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1].view(np.uint32), res[1][1].view(np.uint32))
