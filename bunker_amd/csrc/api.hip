@@ -267,10 +267,12 @@ static int run_fa2(Kernel& k, const uint64_t* s) {
                             P<uint16_t>(s[3]) + HD, (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[7]), nullptr, k.scratch, k.scratch_bytes,
                             batch, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, 1, (int)k.get("exact", 1));
 }
-// ---- op: fa2_fused = qnorm, rope, knorm, ropek, fa2_attn of src/model.ts:126-157 as three launches
-// (norm + rotation + cache append; split attention; merge with the output gate).
+// ---- op: fa2_fused = qnorm, rope, knorm, ropek, fa2_attn of src/model.ts:126-157 as two launches (split attention
+// with the norms, the rotation and the cache append inside; merge with the output gate), or as three with the
+// preparation as a launch of its own (prep_fused=0, and always with exact=0).
 // slots: qgate (q_proj output, [q | gate] per head), k, v, q_norm.weight, k_norm.weight, rope_cos, rope_sin, pos,
-//        kv_k, kv_v, out [, out as Q8_1 blocks when q8out=1]        params: HD, NH, NKV, MAX_LEN, ROT_HALF, batch=1, pos_dev=0, q8out=0
+//        kv_k, kv_v, out [, out as Q8_1 blocks when q8out=1]        params: HD, NH, NKV, MAX_LEN, ROT_HALF, batch=1, pos_dev=0, q8out=0,
+//        exact=1, prep_fused=1
 static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   const bool dev = k.get("pos_dev", 0) != 0;
   const int HD = (int)k.get("HD", 0), NH = (int)k.get("NH", 0), NKV = (int)k.get("NKV", 0), batch = (int)k.get("batch", 1);
@@ -284,6 +286,14 @@ static int run_fa2_fused(Kernel& k, const uint64_t* s) {
   void* qn = k.scratch;
   uint32_t* qf = exact ? (uint32_t*)((uint8_t*)k.scratch + qn_bytes) : nullptr;
   void* ws = (uint8_t*)k.scratch + qn_bytes + qf_bytes;
+  if (exact && k.get("prep_fused", 1) != 0) {
+    // one launch less: the attention kernel prepares q itself and the workgroup that holds the new position appends k, v
+    BK_REQUIRE(dev || (pos >= 0 && pos < max_len), "attn_prep: pos=%d outside the cache (max_len=%d)", pos, max_len);
+    const AttnPrepFuse pf{P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]), half, max_len};
+    return launch_attn_decode(nullptr, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, pos_dev, pos, 1, max_len, P<uint16_t>(s[0]) + HD,
+                              (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[10]), nullptr, ws, k.scratch_bytes - qn_bytes - qf_bytes,
+                              batch, NH, NKV, HD, 16, (int)k.get("splits", 0), k.get("q8out", 0) ? P<void>(s[11]) : nullptr, 1, 1, nullptr, &pf);
+  }
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
                             pos_dev, pos, half, max_len, qn, P<void>(s[8]), P<void>(s[9]), nullptr, bt_stride, batch, NH, NKV, HD, 16, qf);
   if (rc) return rc;

@@ -323,8 +323,9 @@ int attn_choose_splits(int batch, int NKV, int max_ctx) {
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
-                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw, int exact, const uint32_t* qf_ready) {
-  BK_REQUIRE(q && kc && vc && out, "attn_decode: null pointer");
+                       int NH, int NKV, int HD, int page_size, int splits, void* out_q8, int tpw, int exact, const uint32_t* qf_ready,
+                       const AttnPrepFuse* prep) {
+  BK_REQUIRE((q || prep) && kc && vc && out, "attn_decode: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_decode: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(NKV > 0 && NH > 0 && NH % NKV == 0 && NH / NKV <= 16, "attn_decode: NH=%d NKV=%d (group must be <= 16)", NH, NKV);
   BK_REQUIRE(batch > 0 && batch <= 65535 && NKV <= 65535, "attn_decode: bad batch=%d", batch);
@@ -373,6 +374,15 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   const dim3 grid(A.slots > 0 ? A.slots : splits, NKV, A.slots > 0 ? 1 : groups), block(ATT_WAVES * 64);
   if (exact) {
     // double-precision form: same cut of the pages, its own kernels and workspace layout
+    if (prep) {
+      BK_REQUIRE(tpw == 1 && !(block_table && bt_stride == 0), "attn_decode: the folded preparation serves one new token per sequence");
+      BK_REQUIRE(prep->qg && prep->k && prep->v && prep->qw && prep->kw && prep->cos_t && prep->sin_t, "attn_decode: null preparation input");
+      BK_REQUIRE(prep->half > 0 && 2 * prep->half <= HD && prep->max_len >= 1 && (prep->max_len + ATT_PAGE - 1) / ATT_PAGE <= bt_stride,
+                 "attn_decode: bad rotary width %d or capacity %d", prep->half, prep->max_len);
+      A.pq = (const uint16_t*)prep->qg; A.pk = (const uint16_t*)prep->k; A.pv = (const uint16_t*)prep->v;
+      A.pqw = (const uint16_t*)prep->qw; A.pkw = (const uint16_t*)prep->kw; A.pcos = prep->cos_t; A.psin = prep->sin_t;
+      A.phalf = prep->half; A.pmax_len = prep->max_len; A.kcw = (uint16_t*)kc; A.vcw = (uint16_t*)vc;
+    }
     int rc = launch_attn_exact(A, q, qf_ready, workspace, workspace_bytes, nt, grid, batch);
     if (rc) return rc;
     if (splits == 1 && out_q8) return launch_quantize_q8_1(out, DT_BF16, out_q8, NH * HD, batch);
@@ -445,7 +455,7 @@ int launch_attn_decode_noalloc(int device, const void* q, const void* kc, const 
              "attn_decode_noalloc: batch %d x %d KV heads x %d splits = %lld partial results exceed the %d of the built-in scratch "
              "(use fewer splits, or bk_attn_decode with a workspace)", batch, NKV, splits, (long long)(groups * splits), NOALLOC_MAX_PARTIALS);
   return launch_attn_decode(q, kc, vc, block_table, bt_stride, ctx_len, 0, 0, max_ctx, gate, gate_bstride, gate_hstride, out, lse,
-                            g_scratch_ptr[device], NOALLOC_SCRATCH_BYTES, batch, NH, NKV, HD, page_size, splits, nullptr, 1, 0, nullptr);
+                            g_scratch_ptr[device], NOALLOC_SCRATCH_BYTES, batch, NH, NKV, HD, page_size, splits, nullptr, 1, 0, nullptr, nullptr);
 }
 
 // ---------------------------------------------------------------- per-head norm + RoPE + cache append in one launch

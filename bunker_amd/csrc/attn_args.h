@@ -41,7 +41,16 @@ struct AttnArgs {
   int rel;                    // 1: lengths in device memory, every sequence cuts its own pages into `splits` equal ranges
   int slots;                  // > 0: balanced form, this many workgroup slots per KV head shared by the rows (rows <= 64)
   float scale;
+  // Double-precision form with the step's preparation folded in (decode only: one new token per sequence): the query
+  // heads are normalised and rotated by every workgroup for itself, and the workgroup whose pages hold the new position
+  // normalises and rotates the key, appends key and value to the cache and uses them from registers / LDS.
+  const uint16_t *pq, *pk, *pv;      // q|gate bf16 [B, NH, 2*256]; k, v bf16 [B, NKV, 256]; pq == null: no preparation
+  const uint16_t *pqw, *pkw;         // norm weights bf16 [256]
+  const float *pcos, *psin;          // f32 [max_len, half]
+  uint16_t *kcw, *vcw;               // the caches, writable
+  int phalf, pmax_len;
 };
+
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);

@@ -86,7 +86,44 @@ __device__ __forceinline__ void fmac8_bcast(double (&a)[EX_COLS], double bsrc, d
         : "v"(bsrc), "v"(v));
 }
 
-template <bool NT>
+// One head's RMS norm and rotation, the arithmetic of attn_prep_kernel (attn.hip) to the bit: lane holds elements
+// lane + 64 j.  `sh` is 256 bf16 of LDS that belong to the calling wave alone.
+__device__ __forceinline__ void head_norm_rope(const uint16_t* xh, const uint16_t* w, const float* cos_t, const float* sin_t, int pos, int half,
+                                               uint16_t* sh, uint16_t (&o)[ATT_HD / 64], int lane) {
+  float xv[ATT_HD / 64];
+  double ss = 0.0;
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) { xv[j] = bf16_to_f32(xh[lane + 64 * j]); ss += (double)(xv[j] * xv[j]); }
+  ss = wave_sum_f64(ss);
+  const float rstd = rsqrt_f64(ss / (double)ATT_HD + 1e-6);
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) {
+    const int i = lane + 64 * j;
+    sh[i] = f32_to_bf16(__fmul_rn(__fmul_rn(xv[j], rstd), __fadd_rn(1.0f, bf16_to_f32(w[i]))));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int j = 0; j < ATT_HD / 64; j++) {
+    const int i = lane + 64 * j;
+    o[j] = sh[i];
+    if (i < 2 * half) {
+      const int i1 = i < half ? i : i - half;
+      const float x1 = bf16_to_f32(sh[i1]), x2 = bf16_to_f32(sh[i1 + half]);
+      const float c = cos_t[(int64_t)pos * half + i1], sn = sin_t[(int64_t)pos * half + i1];
+      o[j] = i < half ? f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, sn)))
+                      : f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, sn)));
+    }
+  }
+}
+
+// PREP: the step's preparation happens here instead of in a launch of its own (one new token per sequence, at
+// position len - 1).  Every workgroup normalises and rotates its 8 query heads itself (score wave = head).  The
+// workgroup whose pages hold the new position does the same for the key, stores key and value in the cache for the
+// steps to come, and takes both from LDS / registers where its tiles reach that token, so nothing waits for memory
+// that this launch itself writes.  A position outside the cache appends nothing, like attn_prep_kernel.
+template <bool NT, bool PREP>
 __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   // K tile (33792 bytes) and the exchange buffer of the partial scores (8 waves x 8 heads x 64 tokens x 8 = 32768 bytes);
   // the same memory carries the accumulator tree at the end (4 waves x 8 x 256 doubles = 65536 bytes)
@@ -95,6 +132,8 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   __shared__ double lds_alpha[2][EX_COLS], lds_m[EX_COLS], lds_l[EX_COLS];
   __shared__ int lds_rescale[2];                // set by a head that moved its reference exponent in an even / odd tile
   __shared__ int lds_bt[ATT_MAX_PPS];
+  __shared__ __align__(16) uint16_t lds_knew[PREP ? ATT_HD : 8];   // the new token's key, normalised and rotated
+  __shared__ uint16_t lds_vnew[PREP ? ATT_HD : 8];                 // and its value
   unsigned char* ktile = lds_raw;
   double (*xch)[EX_COLS][EX_TILE] = (double (*)[EX_COLS][EX_TILE])(lds_raw + EX_TILE * EX_KROW);
 
@@ -125,6 +164,49 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
     return make_uint4(t4[0], t4[1], t4[2], t4[3]);
   };
 
+  // ---- preparation: q of this group into LDS (high words, [dim][head], in the exchange buffer, which the first tile
+  // overwrites only behind the next barrier), the new key into lds_knew, key and value into the cache
+  int new_tile = -1, new_row = 0;                 // tile and row within the tile of the new token, if this workgroup holds it
+  if (PREP) {
+    uint32_t* lds_q = (uint32_t*)xch;
+    uint16_t* sh = (uint16_t*)(lds_q + ATT_HD * EX_COLS) + wave * ATT_HD;
+    const int pos_raw = len - 1;
+    const int pos = min(max(pos_raw, 0), A.pmax_len - 1);
+    const int ppage = pos / ATT_PAGE - p_begin, slot = pos % ATT_PAGE;
+    const bool holds = pos == pos_raw && ppage >= 0 && ppage < npg;
+    if (holds) {
+      new_tile = __builtin_amdgcn_readfirstlane(ppage / EX_TILE_PAGES);
+      new_row = __builtin_amdgcn_readfirstlane((ppage % EX_TILE_PAGES) * ATT_PAGE + slot);
+    }
+    if (!value_role) {
+      uint16_t o[ATT_HD / 64];
+      if (w8 < A.G)
+        head_norm_rope(A.pq + ((int64_t)row * A.NH + kvh * A.G + w8) * 2 * ATT_HD, A.pqw, A.pcos, A.psin, pos, A.phalf, sh, o, lane);
+#pragma unroll
+      for (int j = 0; j < ATT_HD / 64; j++) lds_q[(lane + 64 * j) * EX_COLS + w8] = w8 < A.G ? bf16_to_f64_high(o[j]) : 0u;
+    } else if (holds) {
+      const int64_t base = ((int64_t)lds_bt[ppage] * A.NKV + kvh) * (ATT_PAGE * ATT_HD);
+      if (w8 == 0) {
+        uint16_t o[ATT_HD / 64];
+        head_norm_rope(A.pk + ((int64_t)row * A.NKV + kvh) * ATT_HD, A.pkw, A.pcos, A.psin, pos, A.phalf, sh, o, lane);
+#pragma unroll
+        for (int j = 0; j < ATT_HD / 64; j++) {
+          lds_knew[lane + 64 * j] = o[j];
+          A.kcw[base + slot * ATT_HD + lane + 64 * j] = o[j];
+        }
+      } else if (w8 == 1) {
+        const uint16_t* vp = A.pv + ((int64_t)row * A.NKV + kvh) * ATT_HD;
+#pragma unroll
+        for (int j = 0; j < ATT_HD / 64; j++) {
+          const uint16_t x = vp[lane + 64 * j];
+          lds_vnew[lane + 64 * j] = x;
+          A.vcw[base + (lane + 64 * j) * ATT_PAGE + slot] = x;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
   // The two roles meet at three barriers per step.  In step s the score waves take tile s through [K rows -> LDS |
   // scores | weights]; the value waves add tile s - 1 (whose weights the third barrier of step s - 1 published) in three
   // pieces, one per interval, so that neither role waits long for the other and the vector unit always has work of
@@ -132,7 +214,11 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   if (!value_role) {
     // the wave's 32 dims x 8 heads of q: register pair g holds dims 2g, 2g + 1 (lane n of a row: dim 2g + n / 8, head n % 8)
     double qreg[16];
-    {
+    if (PREP) {
+      const uint32_t* qw = (const uint32_t*)xch + w8 * 32 * EX_COLS + (lane & 15);
+#pragma unroll
+      for (int g = 0; g < 16; g++) qreg[g] = f64_from_high(qw[g * 16]);
+    } else {
       const uint32_t* qw = A.qf + (((int64_t)row * A.NKV + kvh) * ATT_HD + w8 * 32) * EX_COLS + (lane & 15);
 #pragma unroll
       for (int g = 0; g < 16; g++) qreg[g] = f64_from_high(qw[g * 16]);
@@ -149,8 +235,13 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
       const bool live = tile < ntiles;                             // the last step only drains the value waves
       if (live) {
 #pragma unroll
-        for (int r = 0; r < EX_TILE_PAGES; r++)
-          *(uint4*)(ktile + (r * ATT_PAGE + (tid8 >> 5)) * EX_KROW + (tid8 & 31) * 16) = kpre[r];
+        for (int r = 0; r < EX_TILE_PAGES; r++) {
+          const int krow_i = r * ATT_PAGE + (tid8 >> 5);
+          uint4 kv = kpre[r];
+          // the new token's row comes from LDS: what memory returned for it may be older than this launch's store
+          if (PREP && tile == new_tile && krow_i == new_row) kv = *(const uint4*)(lds_knew + (tid8 & 31) * 8);
+          *(uint4*)(ktile + krow_i * EX_KROW + (tid8 & 31) * 16) = kv;
+        }
       }
       __syncthreads();
       if (live) {
@@ -251,6 +342,19 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
         }
         load_v(min(t + 1, ntiles - 1), j);
       };
+      if (PREP && live && t == new_tile && w8 == (new_row >> 3)) {
+        // the new token's value, from LDS (see the key above): element new_row % 8 of each of the four loads
+        const int e = new_row & 7;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const uint32_t vn = lds_vnew[lane + 64 * j];
+          uint32_t vw[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+#pragma unroll
+          for (int h = 0; h < 4; h++)
+            if ((e >> 1) == h) vw[h] = (e & 1) ? (vw[h] & 0x0000ffffu) | (vn << 16) : (vw[h] & 0xffff0000u) | vn;
+          vreg[j] = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+        }
+      }
       if (live) {
         // a head whose reference exponent moved in this tile (first tile aside: rare) rescales what was summed under the old one
         if (__builtin_amdgcn_readfirstlane(lds_rescale[t & 1])) {
@@ -418,13 +522,15 @@ int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void*
   BK_REQUIRE(A.tpw == 1, "attn_decode (exact): one query row per workgroup");
   BK_REQUIRE(A.G <= EX_COLS, "attn_decode (exact): at most %d query heads per KV head (got %d)", EX_COLS, A.G);
   const size_t npart = A.splits > 1 ? (size_t)batch * A.NKV * A.splits : 0;
-  const size_t need = npart * EX_COLS * (ATT_HD + 2) * sizeof(double) + 64 * sizeof(int2) + (qf_ready ? 0 : attn_exact_qf_bytes(batch, A.NKV));
+  const size_t need = npart * EX_COLS * (ATT_HD + 2) * sizeof(double) + 64 * sizeof(int2) + (qf_ready || A.pq ? 0 : attn_exact_qf_bytes(batch, A.NKV));
   BK_REQUIRE(workspace && workspace_bytes >= need, "attn_decode (exact): workspace of %zu bytes needed for %d splits (got %zu)", need, A.splits,
              workspace_bytes);
   A.part_o64 = (double*)workspace;
   A.part_ml64 = A.part_o64 + npart * EX_COLS * ATT_HD;
   A.plan = (int2*)(A.part_ml64 + npart * EX_COLS * 2);
-  if (qf_ready) {
+  if (A.pq) {
+    A.qf = nullptr;                            // the kernel makes its own query copy, in LDS
+  } else if (qf_ready) {
     A.qf = qf_ready;
   } else {
     uint32_t* qf = (uint32_t*)(A.plan + 64);
@@ -433,8 +539,13 @@ int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void*
   }
   BK_REQUIRE(((uintptr_t)A.qf & 63) == 0, "attn_decode (exact): the f64 query copy must be 64-byte aligned");
   const dim3 block(EX_THREADS);
-  if (nt) hipLaunchKernelGGL((attn_exact_kernel<true>), grid, block, 0, stream(), A);
-  else hipLaunchKernelGGL((attn_exact_kernel<false>), grid, block, 0, stream(), A);
+  if (A.pq) {
+    if (nt) hipLaunchKernelGGL((attn_exact_kernel<true, true>), grid, block, 0, stream(), A);
+    else hipLaunchKernelGGL((attn_exact_kernel<false, true>), grid, block, 0, stream(), A);
+  } else {
+    if (nt) hipLaunchKernelGGL((attn_exact_kernel<true, false>), grid, block, 0, stream(), A);
+    else hipLaunchKernelGGL((attn_exact_kernel<false, false>), grid, block, 0, stream(), A);
+  }
   if (A.splits > 1) {
     const dim3 mgrid(A.NH, batch);
     if (A.splits <= 4) hipLaunchKernelGGL(attn_exact_merge_kernel<4>, mgrid, dim3(256), 0, stream(), A);

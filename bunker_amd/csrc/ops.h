@@ -86,13 +86,20 @@ int launch_gdn_core(const void* q, const void* k, const void* v, const float* g,
                     void* out, float* S_out, int Hg, int batch);
 
 // attn.hip
+// what launch_attn_decode needs to fold the step's preparation (head norms, rotation, cache append) into the
+// double-precision attention kernel: the inputs of launch_attn_prep
+struct AttnPrepFuse {
+  const void *qg, *k, *v, *qw, *kw;
+  const float *cos_t, *sin_t;
+  int half, max_len;
+};
 size_t attn_workspace_bytes(int batch, int NKV, int max_splits);
 int attn_choose_splits(int batch, int NKV, int max_ctx);
 int launch_attn_decode(const void* q, const void* kc, const void* vc, const int32_t* block_table, int bt_stride,
                        const int32_t* ctx_len, int ctx_scalar, int ctx_add, int max_ctx, const void* gate, int64_t gate_bstride,
                        int64_t gate_hstride, void* out, float* lse, void* workspace, size_t workspace_bytes, int batch,
                        int NH, int NKV, int HD, int page_size, int splits, void* out_q8 = nullptr, int tpw = 1, int exact = 0,
-                       const uint32_t* qf_ready = nullptr);
+                       const uint32_t* qf_ready = nullptr, const AttnPrepFuse* prep = nullptr);
 // attn_exact.hip: the double-precision form (workspace: f64 partials, plan, f64 copy of q)
 size_t attn_exact_qf_bytes(int rows, int NKV);
 size_t attn_exact_workspace_bytes(int rows, int NKV, int max_splits);

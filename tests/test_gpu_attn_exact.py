@@ -163,3 +163,40 @@ def test_fa2_attn_op_exact_bits(orc, dev, batch):
             assert np.array_equal(out, ro), spec
         else:
             assert np.abs(f32(out).astype(np.float64) - f32(ro)).max() <= 2e-2, spec
+
+
+@pytest.mark.parametrize("NH,NKV,splits", [(16, 2, 0), (16, 2, 1), (16, 2, 5), (8, 2, 3), (2, 2, 0)])
+def test_folded_preparation_equals_the_separate_launch(dev, NH, NKV, splits):
+    """fa2_fused with the norms, the rotation and the cache append inside the attention kernel (the default) against
+    the same op with the preparation as a launch of its own (prep_fused=0): the same bits in the output, in its Q8_1
+    copy and in both caches.  The positions sit on both sides of page and tile borders, at 0, at the last slot of the
+    cache and behind it (no append), and differ from sequence to sequence."""
+    print(f"fa2_fused folded prep NH={NH} NKV={NKV} splits={splits}", flush=True)
+    g = synth.rng(4300 + NH + splits)
+    HD, HALF, MAXL = 256, 32, 512
+    pos = np.array([0, 15, 16, 17, 63, 64, 65, 300, 447, 448, 510, 511, 512, 600], np.int32)
+    B = len(pos)
+    ppseq = MAXL // 16
+    half_cols = 64
+    cos_t = g.uniform(-1, 1, (MAXL, half_cols // 2)).astype(np.float32); sin_t = g.uniform(-1, 1, (MAXL, half_cols // 2)).astype(np.float32)
+    kc = bf(g.standard_normal((B * ppseq, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((B * ppseq, NKV, HD, 16)).astype(np.float32))
+    qgate = bf(g.standard_normal((B, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((B, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((B, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    common = [dev.up(qgate), dev.up(k), dev.up(v), dev.up(qw), dev.up(kw), dev.up(cos_t), dev.up(sin_t), dev.up(pos)]
+    res = []
+    for folded in (1, 0):
+        dkc, dvc = dev.up(kc), dev.up(vc)
+        dout = dev.empty(B * NH * HD * 2); dq8 = dev.empty(B * NH * HD // 32 * 36)
+        sp = f" splits={splits}" if splits else ""
+        launch(f"fa2_fused HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} batch={B} pos_dev=1 q8out=1 prep_fused={folded}{sp}",
+               common + [dkc, dvc, dout, dq8])
+        res.append((rt.from_device(dout, (B, NH, HD), np.uint16), rt.from_device(dq8, (B, NH * HD // 32 * 36), np.uint8),
+                    rt.from_device(dkc, kc.shape, np.uint16), rt.from_device(dvc, vc.shape, np.uint16)))
+    (o1, q1, k1, v1), (o0, q0, k0, v0) = res
+    assert np.array_equal(k1, k0) and np.array_equal(v1, v0)
+    assert not np.array_equal(k0, kc) and np.array_equal(k0[-ppseq:], kc[-ppseq:])      # appended; the last sequence (behind the cache) not
+    bad = (o1 != o0).reshape(B, -1).any(axis=1)
+    assert not bad.any(), f"sequences {np.nonzero(bad)[0].tolist()} differ"
+    assert np.array_equal(q1, q0)
