@@ -331,6 +331,9 @@ static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
   int rc = launch_attn_prep(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), P<float>(s[5]), P<float>(s[6]),
                             pos, 0, half, max_len, qn, P<void>(s[9]), P<void>(s[10]), table, 0, T, NH, NKV, HD, 16, qf);
   if (rc) return rc;
+  if (k.get("tiled", 0))
+    return launch_attn_prefill_tiled(qn, P<void>(s[9]), P<void>(s[10]), table, pos, max_len, P<uint16_t>(s[0]) + HD, (int64_t)NH * 2 * HD, 2 * HD,
+                                     P<void>(s[11]), T, NH, NKV, HD, 16);
   return launch_attn_decode(qn, P<void>(s[9]), P<void>(s[10]), table, 0, pos, 0, 1, max_len, P<uint16_t>(s[0]) + HD,
                             (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - qn_bytes - qf_bytes,
                             T, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, k.get("pair", 0) ? 2 : 1, exact, qf);
@@ -433,7 +436,13 @@ static int build_kernel(Kernel& k) {
     const int exact = (int)k.get("exact", 1);
     BK_REQUIRE(!exact || NHq / NKV <= 8, "fa2_prefill: exact=1 serves at most 8 query heads per KV head (exact=0 takes 16)");
     // (the double-precision kernel takes one token per workgroup)
-    const int tpw = (!exact && NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
+    // exact=0: query tiles against K/V tiles (attn_prefill.hip) where that kernel serves the shape, unless tiled=0 asks for
+    // the decode kernel per token (pair) instead
+    const bool tiled = !exact && k.get("tiled", 1) != 0 && attn_prefill_tiled_serves(NHq, NKV, max_len);
+    BK_REQUIRE(tiled || k.get("tiled", 0) == 0, "fa2_prefill: tiled=1 needs exact=0 and 1, 2, 4, 8 or 16 query heads per KV head (NH=%d NKV=%d MAX_LEN=%d)",
+               NHq, NKV, max_len);
+    k.p["tiled"] = tiled;
+    const int tpw = (!exact && !tiled && NKV <= NHq && 2 * (NHq / NKV) <= 16 && T >= 2 && k.get("pair", 1) != 0) ? 2 : 1;
     k.p["pair"] = tpw == 2;
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits((T + tpw - 1) / tpw, NKV, max_len); k.p["splits"] = splits; }

@@ -58,6 +58,9 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   const bool col_valid = tk_n < ntk;
   const int row_n = row0 + (col_valid ? tk_n : 0);
   const int len = (A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add;       // of this lane's column
+  int len_wg = len;                             // the longest column: what the cache holds behind it need not be a number
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) len_wg = max(len_wg, __shfl_xor(len_wg, off));
 
   // Q as the B operand of the first product: lane (column n, group kg) holds dims 32*s + 8*kg .. +8
   uint4 qreg[8];
@@ -141,11 +144,15 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
     for (int r = 0; r < 4; r++) plo[r] = p[r] - bf16_to_f32(f32_to_bf16(p[r]));
     const uint2 pb = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
     const uint2 pl = make_uint2(pack_bf16x2(plo[0], plo[1]), pack_bf16x2(plo[2], plo[3]));
+    // the values of tokens behind every column's end enter as zeros (their weights are 0, but 0 * NaN is not)
+    const uint32_t vm0 = (tok0 < len_wg ? 0x0000ffffu : 0u) | (tok0 + 1 < len_wg ? 0xffff0000u : 0u);
+    const uint32_t vm1 = (tok0 + 2 < len_wg ? 0x0000ffffu : 0u) | (tok0 + 3 < len_wg ? 0xffff0000u : 0u);
 #pragma unroll
     for (int t = 0; t < 16; t++) {
-      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pb),
+      const uint2 vv = make_uint2(vreg[t].x & vm0, vreg[t].y & vm1);
+      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vv), __builtin_bit_cast(short4_t, pb),
                                                           oacc[t], 0, 0, 0);
-      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vreg[t]), __builtin_bit_cast(short4_t, pl),
+      oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, vv), __builtin_bit_cast(short4_t, pl),
                                                           oacc[t], 0, 0, 0);
     }
   };

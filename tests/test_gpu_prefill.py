@@ -92,7 +92,7 @@ def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits
         dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
         dout = rt.cuAlloc(T * NH * HD * 2)
         rt.cuMemset(dout, 0xff, T * NH * HD * 2)
-        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} pair={pair} exact=0" + (f" splits={splits}" if splits else ""),
+        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} pair={pair} exact=0 tiled=0" + (f" splits={splits}" if splits else ""),
                 ptrs + [dkc, dvc, dout])
         res.append((rt.from_device(dout, (T, NH, HD), np.uint16), rt.from_device(dkc, kc.shape, np.uint16),
                     rt.from_device(dvc, (pages, NKV, HD, 16), np.uint16)))
@@ -140,6 +140,56 @@ def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0, exact):
     vc_d = rt.from_device(dvc, (2 * pages, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
     assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
     for p in ptrs + [dkc, dvc, dout]:
+        rt.cuFree(p)
+
+
+@pytest.mark.parametrize("NH,NKV,T,pos0", [(16, 2, 200, 70), (16, 2, 64, 0), (8, 2, 97, 33), (4, 4, 130, 5), (16, 1, 50, 17), (4, 2, 129, 0)])
+def test_fa2_prefill_tiled_attention_against_the_checker(orc, NH, NKV, T, pos0):
+    """exact=0 runs the query-tile x K/V-tile kernel (bf16 matrix cores): every row within 2e-2 of the f64 checker, for
+    every group size it serves, ragged last query tile, a context that starts in the middle of a K/V tile, a permuted page
+    table, and NaN bit patterns in the cache behind the prompt (they must not reach any output).  The caches get the
+    same bytes as with exact=1 (the preparation is the same kernel)."""
+    print(f"fa2_prefill tiled NH={NH} NKV={NKV} T={T} pos0={pos0}", flush=True)
+    g = synth.rng(880 + NH + T)
+    HD, HALF, MAXL = 256, 32, 512
+    pages = MAXL // 16
+    cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+    kc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    table = g.permutation(pages).astype(np.int32)
+    end = pos0 + T
+    for tok in range(end, MAXL):                   # behind the prompt: not numbers
+        kc[table[tok // 16], :, tok % 16, :] = 0x7fc0
+        vc[table[tok // 16], :, tok % 16, :] = 0xffc1
+    qgate = bf(g.standard_normal((T, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((T, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((T, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    pos = (pos0 + np.arange(T)).astype(np.int32)
+    ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
+    outs = {}
+    for tiled in (1, 0):
+        dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
+        dout = rt.cuAlloc(T * NH * HD * 2)
+        rt.cuMemset(dout, 0xff, T * NH * HD * 2)
+        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} exact=0 tiled={tiled}", ptrs + [dkc, dvc, dout])
+        outs[tiled] = rt.from_device(dout, (T, NH, HD), np.uint16)
+        kc_d = rt.from_device(dkc, kc.shape, np.uint16)
+        vc_d = rt.from_device(dvc, (pages, NKV, HD, 16), np.uint16).transpose(0, 1, 3, 2)
+        for p in (dkc, dvc, dout):
+            rt.cuFree(p)
+    assert not np.any(outs[1] == 0xffff)            # every row written, none of them NaN
+    worst = 0.0
+    for t in range(T):
+        qn = orc.rope(orc.headnorm(qgate[t].ravel(), qw, NH, HD, 2 * HD), cos_t, sin_t, pos[t], NH, HD, HALF).reshape(1, NH, HD)
+        kn = orc.rope(orc.headnorm(k[t].ravel(), kw, NKV, HD, HD), cos_t, sin_t, pos[t], NKV, HD, HALF)
+        orc.kv_append(kn.reshape(NKV, HD), v[t], kc, vc, table, pos[t], NKV, HD, 16)
+        ro, _ = orc.attn_decode_paged(qn, kc, vc, table[None], np.array([pos[t] + 1], np.int32), 1, NH, NKV, HD, 16,
+                                      gate=qgate[t].ravel()[HD:], gate_bstride=0, gate_hstride=2 * HD)
+        worst = max(worst, float(np.abs(f32(outs[1][t]).astype(np.float64) - f32(ro[0])).max()))
+    assert worst <= 2e-2, worst
+    assert np.array_equal(kc_d, kc) and np.array_equal(vc_d, vc)
+    assert np.abs(f32(outs[1]).astype(np.float64) - f32(outs[0])).max() <= 2e-2
+    for p in ptrs:
         rt.cuFree(p)
 
 
