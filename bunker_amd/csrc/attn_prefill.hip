@@ -19,6 +19,11 @@
 namespace bk {
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+// two f32 -> two bf16 (round to nearest even) in one instruction, a in the low half
+__device__ __forceinline__ uint32_t pk_bf16(float a, float b) { return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){a, b}, bf16x2_t)); }
 
 constexpr int PF_THREADS = 256;
 constexpr int PF_ROWS = 128;                 // query rows (token, head) of a workgroup; 32 per wave
@@ -160,11 +165,10 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     // of the eight matrix instructions that use them: a read directly in front of its instruction costs the whole LDS
     // latency per instruction, with one wave per SIMD and nothing else to run.
     f32x16_t s[2];
-#pragma unroll
-    for (int u = 0; u < 2; u++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[u][r] = 0.0f;
     {
+      f32x16_t zero16;
+#pragma unroll
+      for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
       uint4 ka[2][8];
       auto kread = [&](int bt, uint4 (&dst)[8]) {
 #pragma unroll
@@ -181,26 +185,30 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
 #pragma unroll
         for (int i = 0; i < 8; i++)
           s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[bt & 1][i]),
-                                                             __builtin_bit_cast(bf16x8_t, qreg[4 * bt + (i >> 1)]), s[i & 1], 0, 0, 0);
+                                                             __builtin_bit_cast(bf16x8_t, qreg[4 * bt + (i >> 1)]),
+                                                             (bt == 0 && i < 2) ? zero16 : s[i & 1], 0, 0, 0);   // (an inline 0 operand)
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- running-maximum softmax of the row (base 2)
-    const bool masked = tok_base + PF_TILE > wave_minlen;           // wave-uniform
+    // ---- running-maximum softmax of the row (base 2).  The maximum is taken over the raw scores (the scale is positive);
+    // scale and subtraction are one fused multiply-add in front of the hardware exponential (v_exp_f32: 1 ulp, results
+    // below 2^-126 become 0 — far inside the 2e-2 of this kernel).
+    if (tok_base + PF_TILE > wave_minlen) {                         // (wave-uniform) the tile crosses the end of a row
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (tok_base + 32 * u + 16 * (r >> 3) + 8 * half + (r & 7) >= mylen) s[u][r] = -INFINITY;
+    }
     float mloc = -INFINITY;
 #pragma unroll
     for (int u = 0; u < 2; u++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float v = s[u][r] * A.scale_log2;
-        if (masked && tok_base + 32 * u + 16 * (r >> 3) + 8 * half + (r & 7) >= mylen) v = -INFINITY;
-        s[u][r] = v;
-        mloc = fmaxf(mloc, v);
-      }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[u][r]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * A.scale_log2;
     const float mnew = fmaxf(mrow, mloc);
     const float msub = mnew == -INFINITY ? 0.0f : mnew;             // a row without any token so far: every weight is 0
-    const float alpha = mnew == -INFINITY ? 1.0f : exp2f(mrow - mnew);   // (first tile with a token: exp2(-inf) = 0 times the zeros)
+    const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mrow - mnew);   // (first tile with a token: exp2(-inf) = 0 times the zeros)
     mrow = mnew;
     float psum = 0.0f;
     uint4 pb[4];
@@ -208,8 +216,8 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     for (int j = 0; j < 4; j++) {
       float p[8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) { p[e] = exp2f(s[j >> 1][8 * (j & 1) + e] - msub); psum += p[e]; }
-      pb[j] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
+      for (int e = 0; e < 8; e++) { p[e] = __builtin_amdgcn_exp2f(__fmaf_rn(s[j >> 1][8 * (j & 1) + e], A.scale_log2, -msub)); psum += p[e]; }
+      pb[j] = make_uint4(pk_bf16(p[0], p[1]), pk_bf16(p[2], p[3]), pk_bf16(p[4], p[5]), pk_bf16(p[6], p[7]));
     }
     lrow = lrow * alpha + psum;
     if (__ballot(alpha != 1.0f) != 0ull) {
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
         v[2] = __fmul_rn(v[2], sigmoid_f64(__uint_as_float(gw.y << 16)));
         v[3] = __fmul_rn(v[3], sigmoid_f64(__uint_as_float(gw.y & 0xffff0000u)));
       }
-      *(uint2*)(op + d) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      *(uint2*)(op + d) = make_uint2(pk_bf16(v[0], v[1]), pk_bf16(v[2], v[3]));
     }
 }
 
