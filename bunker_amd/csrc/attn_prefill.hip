@@ -134,9 +134,6 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   int wave_minlen = mylen;
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) wave_minlen = min(wave_minlen, __shfl_xor(wave_minlen, off));
-  int wave_maxlen = mylen;
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) wave_maxlen = max(wave_maxlen, __shfl_xor(wave_maxlen, off));
 
   // Row `col` of the first product's A operand is K token tau(col) of the 32 (bits 2 and 3 of col exchanged): the
   // result registers 8 jj .. 8 jj + 7 of a lane then belong to the 8 consecutive tokens 16 jj + 8 half .. + 8, which is
@@ -158,7 +155,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     const unsigned char* lds_v = lds_k + PF_KBYTES;
     // the next tile goes to the other buffer, which every wave left at the last barrier
     if (tile + 1 < ntiles) copy_tile(tile + 1);
-    if (tok_base < wave_maxlen) {       // (wave-uniform) else every row of this wave ends before the tile
+    {
 
     // ---- scores, transposed: s[u][r] = S^T[token 32 u + 16 (r / 8) + 8 half + r % 8, this lane's row].  The A operands
     // come from LDS in batches of eight 16-byte reads (four dim slices x the two token halves), requested a batch ahead
@@ -169,23 +166,23 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
       f32x16_t zero16;
 #pragma unroll
       for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
-      uint4 ka[2][8];
-      auto kread = [&](int bt, uint4 (&dst)[8]) {
+      uint4 ka[2][4];
+      auto kread = [&](int bt, uint4 (&dst)[4]) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const int sl = 4 * bt + (i >> 1);
+        for (int i = 0; i < 4; i++) {
+          const int sl = 2 * bt + (i >> 1);
           dst[i] = *(const uint4*)(lds_k + koff[sl & 7] + (sl >> 3) * 256 + (i & 1) * 32 * (ATT_HD * 2));
         }
       };
       kread(0, ka[0]);
 #pragma unroll
-      for (int bt = 0; bt < 4; bt++) {
-        if (bt + 1 < 4) kread(bt + 1, ka[(bt + 1) & 1]);
+      for (int bt = 0; bt < 8; bt++) {
+        if (bt + 1 < 8) kread(bt + 1, ka[(bt + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 8; i++)
+        for (int i = 0; i < 4; i++)
           s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[bt & 1][i]),
-                                                             __builtin_bit_cast(bf16x8_t, qreg[4 * bt + (i >> 1)]),
+                                                             __builtin_bit_cast(bf16x8_t, qreg[2 * bt + (i >> 1)]),
                                                              (bt == 0 && i < 2) ? zero16 : s[i & 1], 0, 0, 0);   // (an inline 0 operand)
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -206,7 +203,10 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
 #pragma unroll
       for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[u][r]);
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * A.scale_log2;
-    const float mnew = fmaxf(mrow, mloc);
+    // The reference exponent of a row follows its maximum only when that has grown by more than 2^24 (or is the first):
+    // weights up to 2^24 are as exact in bf16 and f32 as weights up to 1, and the 128 accumulators of a lane need their
+    // rescaling pass in a few early tiles only instead of in every tile where some row of the wave sees a new maximum.
+    const float mnew = (mloc > mrow + 24.0f) ? mloc : mrow;
     const float msub = mnew == -INFINITY ? 0.0f : mnew;             // a row without any token so far: every weight is 0
     const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mrow - mnew);   // (first tile with a token: exp2(-inf) = 0 times the zeros)
     mrow = mnew;
@@ -229,19 +229,21 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     // ---- values: O^T[dim 32 dt + .., row] += V^T . P^T over the four 16-token slices, the A operands again a batch
     // (one slice, eight dim tiles) ahead
     {
-      uint4 va[2][8];
-      auto vread = [&](int j, uint4 (&dst)[8]) {
+      uint4 va[2][4];
+      auto vread = [&](int b, uint4 (&dst)[4]) {       // batch b: slice b / 2, dim tiles 4 (b % 2) .. + 4
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) dst[dt] = *(const uint4*)(lds_v + voff[j] + dt * 32 * (PF_TILE * 2));
+        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(lds_v + voff[b >> 1] + (4 * (b & 1) + i) * 32 * (PF_TILE * 2));
       };
       vread(0, va[0]);
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        if (j + 1 < 4) vread(j + 1, va[(j + 1) & 1]);
+      for (int b = 0; b < 8; b++) {
+        if (b + 1 < 8) vread(b + 1, va[(b + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++)
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[j & 1][dt]), __builtin_bit_cast(bf16x8_t, pb[j]), o[dt], 0, 0, 0);
+        for (int i = 0; i < 4; i++) {
+          const int dt = 4 * (b & 1) + i;
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[b & 1][i]), __builtin_bit_cast(bf16x8_t, pb[b >> 1]), o[dt], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
