@@ -307,11 +307,12 @@ static int run_conv1d_prefill(Kernel& k, const uint64_t* s) {
   return launch_conv1d_prefill(P<void>(s[0]), P<void>(s[1]), P<void>(s[2]), P<void>(s[3]), P<void>(s[4]), (int)k.get("QKVD", 0),
                                (int)k.get("T", 0));
 }
-// gdn_prefill      slots as gdn_delta_rule with T rows in conv_out, z, a_p, b_p, out and one state     params: LVH, T
+// gdn_prefill      slots as gdn_delta_rule with T rows in conv_out, z, a_p, b_p, out and one state     params: LVH, T,
+//                  chunked=0 (1: the recurrence in chunks of 64 tokens on the f32 matrix instruction — the scan's results up to the order of the additions)
 static int run_gdn_prefill(Kernel& k, const uint64_t* s) {
   return launch_gdn_prefill(P<void>(s[0]), P<void>(s[1]), P<float>(s[2]), P<void>(s[3]), P<float>(s[4]), P<float>(s[5]),
                             P<float>(s[6]), P<float>(s[7]), P<void>(s[8]), P<float>(s[9]), k.scratch, k.scratch_bytes,
-                            (int)k.get("LVH", 0), (int)k.get("T", 0));
+                            (int)k.get("LVH", 0), (int)k.get("T", 0), k.get("chunked", 0) != 0);
 }
 // fa2_prefill      the norm + rotation + cache append of fa2_fused for T tokens at positions pos[t], then causal attention:
 //                  token t attends to cache positions 0 .. pos[t] of the sequence whose pages block_table lists.
@@ -422,7 +423,7 @@ static int build_kernel(Kernel& k) {
   if (k.op == "gdn_prefill") {
     if ((rc = need(k, "LVH")) || (rc = need(k, "T"))) return rc;
     BK_REQUIRE(k.get("LVH", 0) >= 1 && k.get("T", 0) >= 1 && k.get("T", 0) <= 65535, "gdn_prefill: bad LVH/T");
-    if ((rc = alloc_scratch(k, gdn_prefill_workspace_bytes((int)k.get("LVH", 0), (int)k.get("T", 0))))) return rc;
+    if ((rc = alloc_scratch(k, gdn_prefill_workspace_bytes((int)k.get("LVH", 0), (int)k.get("T", 0), k.get("chunked", 0) != 0)))) return rc;
     k.run = run_gdn_prefill; k.nslots = 10;
     return BK_OK;
   }

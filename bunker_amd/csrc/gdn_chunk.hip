@@ -1,0 +1,288 @@
+// Gated DeltaNet over a run of T prompt tokens in the chunked form (the form of the reference's prefill prototypes:
+// prototypes/gdn_fast.ts kernels kkt_fwd / solve_tril / recompute_w_u / fwd_h / fwd_o, prototypes/gdn_solve_tril.ts),
+// as an alternative to the token-by-token scan of gdn_prefill.hip.  The recurrence
+//     S_t = d_t S_{t-1} + k_t u_t^T,   u_t = beta_t (v_t - d_t S_{t-1}^T k_t),   o_t = S_t^T q_t
+// is cut into chunks of 64 tokens.  With g_t the sum of log d over the chunk up to t and S_0 the state at its start:
+//     (I + N) U = diag(beta) V - diag(beta e^g) K S_0,     N[t][j] = beta_t e^(g_t - g_j) (k_t . k_j)  for j < t
+//     => U = Uv - W S_0,   T = (I + N)^-1,   Uv = T diag(beta) V,   W = T diag(beta e^g) K        (chunks in parallel)
+//     S_C = e^(g_C) S_0 + K^T diag(e^(g_C - g)) U                                                 (chunk after chunk)
+//     O = diag(e^g) Q S_0 + M U,   M[t][j] = e^(g_t - g_j) (q_t . k_j)  for j <= t               (chunks in parallel)
+// Every product runs on the f32 matrix instruction (v_mfma_f32_32x32x2_f32: f32 operands, f32 sums), so the results
+// differ from the scan's by the order of the additions only — about 1e-6 relative on the state — but not to the bit:
+// the scan stays the default of the prompt path, this form is chosen with chunked=1.
+// The reference multiplies in f16 (dot16, gdn_fast.ts:15); f32 operands are the tighter choice the hardware offers at
+// the same instruction count.
+#include "ops.h"
+
+namespace bk {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int GC_C = 64;       // tokens per chunk
+constexpr int GC_D = 128;      // key and value width of a head
+constexpr int GC_LD = GC_D + 1;   // row stride of the [64][128] operands in LDS: the 32 rows of an operand read fall into different banks
+
+struct GdnChunkArgs {
+  const uint16_t* conv_out;   // bf16 [T, 3*Hg*128]: q | k | v
+  const float* A_log;         // f32 [Hg]
+  const uint16_t* dt_bias;    // bf16 [Hg]
+  const float* a_p;           // f32 [T, Hg]
+  const float* qk;            // f32 [T, Hg, 2, 128]: q^ (scaled), k^   (gdn_prefill_prep_kernel)
+  const float* gates;         // f32 [T, Hg, 2]: decay, beta
+  const float* S_in;          // f32 [Hg, 128, 128]
+  float* S_out;
+  float* G;                   // f32 [Hg, nC, 64]: sum of log decay from the chunk's first token
+  float* W;                   // f32 [Hg, nC, 64, 128]
+  float* U;                   // f32 [Hg, nC, 64, 128]: Uv, replaced by U as the states pass
+  float* Hs;                  // f32 [Hg, nC, 128, 128]: the state at the start of every chunk
+  float* o_raw;               // f32 [T, Hg, 128]
+  int Hg, T, nC;
+};
+
+// row of the 32x32 result held in register r of a lane in half `half` of the wave (its column is lane % 32)
+__device__ __forceinline__ int mrow(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
+
+__device__ __forceinline__ f32x16_t zero16() {
+  f32x16_t z;
+#pragma unroll
+  for (int r = 0; r < 16; r++) z[r] = 0.0f;
+  return z;
+}
+
+// ---- kernel 1, per (head, chunk): g, T = (I + N)^-1, W, Uv
+__global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
+  __shared__ float Ks[GC_C][GC_LD], Vs[GC_C][GC_LD];
+  __shared__ float Ns[GC_C][GC_C + 1], Ts[GC_C][GC_C + 1];
+  __shared__ float g_s[GC_C], beta_s[GC_C], cw_s[GC_C];
+  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const int t0 = c * GC_C, KEYDIM = A.Hg * GC_D;
+  for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
+    const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
+    const bool valid = t < A.T;
+    Ks[tt][i] = valid ? A.qk[(((int64_t)t * A.Hg + h) * 2 + 1) * GC_D + i] : 0.0f;
+    Vs[tt][i] = valid ? bf16_to_f32(A.conv_out[(int64_t)t * 3 * KEYDIM + 2 * KEYDIM + h * GC_D + i]) : 0.0f;
+  }
+  if (tid < GC_C) {
+    const int t = t0 + tid;
+    const bool valid = t < A.T;
+    const int64_t th = (int64_t)min(t, A.T - 1) * A.Hg + h;
+    // log of the decay, as gdn_prefill_prep_kernel forms the decay itself; a token past the run leaves the state alone
+    const float sp_in = A.a_p[th] + bf16_to_f32(A.dt_bias[h]);
+    const float softplus = (float)log1p(exp((double)sp_in));
+    float g = valid ? -((float)exp((double)A.A_log[h]) * softplus) : 0.0f;
+    const float beta = valid ? A.gates[th * 2 + 1] : 0.0f;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float up = __shfl_up(g, off);
+      if (lane >= off) g += up;
+    }
+    g_s[tid] = g; beta_s[tid] = beta; cw_s[tid] = beta * expf(g);
+    A.G[((int64_t)h * A.nC + c) * GC_C + tid] = g;
+  }
+  __syncthreads();
+  // K K^T: wave w owns tile (w / 2, w % 2); tile (0, 1) lies above the diagonal
+  {
+    const int ti = wave >> 1, tj = wave & 1;
+    f32x16_t acc = zero16();
+    if (wave != 1) {
+#pragma unroll 8
+      for (int s = 0; s < GC_D / 2; s++)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ks[32 * ti + col][2 * s + half], Ks[32 * tj + col][2 * s + half], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int t = 32 * ti + mrow(r, half), j = 32 * tj + col;
+      Ns[t][j] = j < t ? beta_s[t] * expf(g_s[t] - g_s[j]) * acc[r] : 0.0f;
+    }
+  }
+  __syncthreads();
+  // T = (I + N)^-1 by forward substitution, one wave: lane = column, row i needs rows 0 .. i-1
+  if (wave == 0) {
+    float Tr[GC_C];
+#pragma unroll
+    for (int i = 0; i < GC_C; i++) {
+      const float nrow = Ns[i][lane];
+      float a = lane == i ? 1.0f : 0.0f;
+#pragma unroll
+      for (int j = 0; j < i; j++) a -= __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(nrow), j)) * Tr[j];
+      Tr[i] = a;
+      Ts[i][lane] = a;
+    }
+  }
+  __syncthreads();
+  // W = T diag(beta e^g) K and Uv = T diag(beta) V: wave w owns the 32 columns 32 w .. of both, T's zeros above the diagonal skipped
+  const int64_t hc = (int64_t)h * A.nC + c;
+#pragma unroll
+  for (int which = 0; which < 2; which++)
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) {
+      f32x16_t acc = zero16();
+      const float (*B)[GC_LD] = which ? Vs : Ks;
+      const float* coef = which ? beta_s : cw_s;
+      const int steps = 16 * (tt + 1);
+#pragma unroll 8
+      for (int s = 0; s < steps; s++) {
+        const int j = 2 * s + half;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ts[32 * tt + col][j] * coef[j], B[j][32 * wave + col], acc, 0, 0, 0);
+      }
+      float* dst = (which ? A.U : A.W) + (hc * GC_C + 32 * tt) * GC_D + 32 * wave + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) dst[(int64_t)mrow(r, half) * GC_D] = acc[r];
+    }
+}
+
+// ---- kernel 2, per (head, slab of 32 value columns): the states, chunk after chunk.  Wave w keeps rows 32 w .. + 32
+// of the slab in the accumulators of one 32x32 tile.
+__global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
+  __shared__ float Wc[GC_C][GC_LD], Kc[GC_C][GC_LD];
+  __shared__ float red[4][GC_C][33];
+  __shared__ float Ut[GC_C][33];
+  __shared__ float g_s[GC_C];
+  const int h = blockIdx.x, sl = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  f32x16_t S;
+  {
+    const float* Si = A.S_in + (int64_t)h * GC_D * GC_D + 32 * sl + col;
+#pragma unroll
+    for (int r = 0; r < 16; r++) S[r] = Si[(int64_t)(32 * wave + mrow(r, half)) * GC_D];
+  }
+  for (int c = 0; c < A.nC; c++) {
+    const int64_t hc = (int64_t)h * A.nC + c;
+    const int t0 = c * GC_C;
+    __syncthreads();                                   // the previous chunk's readers are done
+    for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
+      const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
+      Wc[tt][i] = A.W[(hc * GC_C + tt) * GC_D + i];
+      Kc[tt][i] = t < A.T ? A.qk[(((int64_t)t * A.Hg + h) * 2 + 1) * GC_D + i] : 0.0f;
+    }
+    if (tid < GC_C) g_s[tid] = A.G[hc * GC_C + tid];
+    {
+      float* Ho = A.Hs + hc * GC_D * GC_D + 32 * sl + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) Ho[(int64_t)(32 * wave + mrow(r, half)) * GC_D] = S[r];
+    }
+    __syncthreads();
+    // this wave's share of W S: the sum over its 32 rows of S, taken in the order the accumulator holds them
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) {
+      f32x16_t P = zero16();
+#pragma unroll
+      for (int r = 0; r < 16; r++) P = __builtin_amdgcn_mfma_f32_32x32x2f32(Wc[32 * tt + col][32 * wave + mrow(r, half)], S[r], P, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 16; r++) red[wave][32 * tt + mrow(r, half)][col] = P[r];
+    }
+    __syncthreads();
+    const float gC = g_s[GC_C - 1];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int e = tid + 256 * i, t = e >> 5, n = e & 31;
+      float* up = A.U + (hc * GC_C + t) * GC_D + 32 * sl + n;
+      const float u = *up - (((red[0][t][n] + red[1][t][n]) + red[2][t][n]) + red[3][t][n]);
+      *up = u;
+      Ut[t][n] = u * expf(gC - g_s[t]);
+    }
+    __syncthreads();
+    const float dC = expf(gC);
+#pragma unroll
+    for (int r = 0; r < 16; r++) S[r] *= dC;
+#pragma unroll 8
+    for (int s = 0; s < GC_C / 2; s++) S = __builtin_amdgcn_mfma_f32_32x32x2f32(Kc[2 * s + half][32 * wave + col], Ut[2 * s + half][col], S, 0, 0, 0);
+  }
+  float* So = A.S_out + (int64_t)h * GC_D * GC_D + 32 * sl + col;
+#pragma unroll
+  for (int r = 0; r < 16; r++) So[(int64_t)(32 * wave + mrow(r, half)) * GC_D] = S[r];
+}
+
+// ---- kernel 3, per (head, chunk): the outputs
+__global__ __launch_bounds__(256) void gdn_chunk_out_kernel(GdnChunkArgs A) {
+  __shared__ float Qs[GC_C][GC_LD], Ks[GC_C][GC_LD], Us[GC_C][GC_LD];
+  __shared__ float Ms[GC_C][GC_C + 1];
+  __shared__ float g_s[GC_C];
+  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const int t0 = c * GC_C;
+  const int64_t hc = (int64_t)h * A.nC + c;
+  for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
+    const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
+    const bool valid = t < A.T;
+    const float* qk = A.qk + ((int64_t)min(t, A.T - 1) * A.Hg + h) * 2 * GC_D;
+    Qs[tt][i] = valid ? qk[i] : 0.0f;
+    Ks[tt][i] = valid ? qk[GC_D + i] : 0.0f;
+    Us[tt][i] = A.U[(hc * GC_C + tt) * GC_D + i];
+  }
+  if (tid < GC_C) g_s[tid] = A.G[hc * GC_C + tid];
+  __syncthreads();
+  {
+    const int ti = wave >> 1, tj = wave & 1;
+    f32x16_t acc = zero16();
+    if (wave != 1) {
+#pragma unroll 8
+      for (int s = 0; s < GC_D / 2; s++)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[32 * ti + col][2 * s + half], Ks[32 * tj + col][2 * s + half], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int t = 32 * ti + mrow(r, half), j = 32 * tj + col;
+      Ms[t][j] = j <= t ? expf(g_s[t] - g_s[j]) * acc[r] : 0.0f;
+    }
+  }
+  __syncthreads();
+  // wave w owns value columns 32 w .. + 32: diag(e^g) Q S_0, the state read straight from memory as the B operand
+  // (a lane's 64 loads per tile are issued 16 ahead of the 16 instructions that use them), then M U
+  const float* Hc = A.Hs + hc * GC_D * GC_D + 32 * wave + col;
+#pragma unroll
+  for (int tt = 0; tt < 2; tt++) {
+    f32x16_t acc = zero16();
+    float sb[2][16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) sb[0][i] = Hc[(int64_t)(2 * i + half) * GC_D];
+#pragma unroll
+    for (int bt = 0; bt < 4; bt++) {
+      if (bt + 1 < 4) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) sb[(bt + 1) & 1][i] = Hc[(int64_t)(2 * (16 * (bt + 1) + i) + half) * GC_D];
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[32 * tt + col][2 * (16 * bt + i) + half], sb[bt & 1][i], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] *= expf(g_s[32 * tt + mrow(r, half)]);
+    const int steps = 16 * (tt + 1);
+#pragma unroll 8
+    for (int s = 0; s < steps; s++) {
+      const int j = 2 * s + half;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ms[32 * tt + col][j], Us[j][32 * wave + col], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int t = t0 + 32 * tt + mrow(r, half);
+      if (t < A.T) A.o_raw[((int64_t)t * A.Hg + h) * GC_D + 32 * wave + col] = acc[r];
+    }
+  }
+}
+
+size_t gdn_chunk_workspace_bytes(int Hg, int T) {
+  const size_t nC = (size_t)(T + GC_C - 1) / GC_C;
+  return (size_t)Hg * nC * (GC_C + 2 * GC_C * GC_D + GC_D * GC_D) * sizeof(float);
+}
+
+// Called by launch_gdn_prefill after its preparation kernel and before its output norm; `workspace` is this form's own.
+int launch_gdn_chunked_core(const void* conv_out, const float* A_log, const void* dt_bias, const float* a_p, const float* qk, const float* gates,
+                            const float* S_in, float* S_out, float* o_raw, void* workspace, size_t workspace_bytes, int Hg, int T) {
+  BK_REQUIRE(workspace && workspace_bytes >= gdn_chunk_workspace_bytes(Hg, T), "gdn_prefill (chunked): workspace of %zu bytes, need %zu",
+             workspace_bytes, gdn_chunk_workspace_bytes(Hg, T));
+  GdnChunkArgs A{};
+  A.conv_out = (const uint16_t*)conv_out; A.A_log = A_log; A.dt_bias = (const uint16_t*)dt_bias; A.a_p = a_p; A.qk = qk; A.gates = gates;
+  A.S_in = S_in; A.S_out = S_out; A.o_raw = o_raw; A.Hg = Hg; A.T = T; A.nC = (T + GC_C - 1) / GC_C;
+  BK_REQUIRE(A.nC <= 65535, "gdn_prefill (chunked): T=%d is too long for one launch", T);
+  const size_t per = (size_t)Hg * A.nC;
+  A.G = (float*)workspace;
+  A.W = A.G + per * GC_C;
+  A.U = A.W + per * GC_C * GC_D;
+  A.Hs = A.U + per * GC_C * GC_D;
+  hipLaunchKernelGGL(gdn_chunk_wu_kernel, dim3(Hg, A.nC), dim3(256), 0, stream(), A);
+  hipLaunchKernelGGL(gdn_chunk_state_kernel, dim3(Hg, GC_D / 32), dim3(256), 0, stream(), A);
+  hipLaunchKernelGGL(gdn_chunk_out_kernel, dim3(Hg, A.nC), dim3(256), 0, stream(), A);
+  return BK_OK;
+}
+
+}  // namespace bk

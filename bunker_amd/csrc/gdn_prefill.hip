@@ -222,17 +222,19 @@ __global__ __launch_bounds__(128) void gdn_prefill_outnorm_kernel(GdnPrefillArgs
   A.out[th * GP_D + tid] = f32_to_bf16(((o * orstd) * A.norm_w[tid]) * zs);
 }
 
-size_t gdn_prefill_workspace_bytes(int Hg, int T) {
-  return (size_t)T * Hg * (2 * GP_D + GP_D + 2) * sizeof(float);
+static size_t gdn_prefill_base_bytes(int Hg, int T) { return (((size_t)T * Hg * (2 * GP_D + GP_D + 2) * sizeof(float)) + 255) & ~(size_t)255; }
+
+size_t gdn_prefill_workspace_bytes(int Hg, int T, bool chunked) {
+  return gdn_prefill_base_bytes(Hg, T) + (chunked ? gdn_chunk_workspace_bytes(Hg, T) : 0);
 }
 
 int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
                        const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, void* workspace,
-                       size_t workspace_bytes, int Hg, int T) {
+                       size_t workspace_bytes, int Hg, int T, bool chunked) {
   BK_REQUIRE(conv_out && z && A_log && dt_bias && a_p && b_p && norm_w && S_in && out && S_out && workspace, "gdn_prefill: null pointer");
   BK_REQUIRE(Hg > 0 && Hg <= 65535 && T > 0 && T <= 65535, "gdn_prefill: bad Hg=%d T=%d", Hg, T);
-  BK_REQUIRE(workspace_bytes >= gdn_prefill_workspace_bytes(Hg, T), "gdn_prefill: workspace of %zu bytes, need %zu", workspace_bytes,
-             gdn_prefill_workspace_bytes(Hg, T));
+  BK_REQUIRE(workspace_bytes >= gdn_prefill_workspace_bytes(Hg, T, chunked), "gdn_prefill: workspace of %zu bytes, need %zu", workspace_bytes,
+             gdn_prefill_workspace_bytes(Hg, T, chunked));
   BK_REQUIRE(((uintptr_t)workspace & 15) == 0, "gdn_prefill: workspace must be 16-byte aligned");
   GdnPrefillArgs A{};
   A.conv_out = (const uint16_t*)conv_out; A.z = (const uint16_t*)z; A.A_log = A_log; A.dt_bias = (const uint16_t*)dt_bias;
@@ -242,7 +244,15 @@ int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, 
   A.gates = A.o_raw + (size_t)T * Hg * GP_D;
   A.Hg = Hg; A.T = T;
   hipLaunchKernelGGL(gdn_prefill_prep_kernel, dim3(Hg, T), dim3(256), 0, stream(), A);
-  hipLaunchKernelGGL(gdn_prefill_scan_kernel, dim3(Hg, GP_SLABS), dim3(256), 0, stream(), A);
+  if (chunked) {
+    // the chunked form of the recurrence (gdn_chunk.hip) between the same preparation and output norm
+    const size_t base = gdn_prefill_base_bytes(Hg, T);
+    const int rc = launch_gdn_chunked_core(conv_out, A_log, dt_bias, a_p, A.qk, A.gates, S_in, S_out, A.o_raw, (uint8_t*)workspace + base,
+                                           workspace_bytes - base, Hg, T);
+    if (rc) return rc;
+  } else {
+    hipLaunchKernelGGL(gdn_prefill_scan_kernel, dim3(Hg, GP_SLABS), dim3(256), 0, stream(), A);
+  }
   hipLaunchKernelGGL(gdn_prefill_outnorm_kernel, dim3(Hg, T), dim3(128), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;

@@ -21,11 +21,15 @@ int launch_dequant_legacy_i8(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_nibbles(const void* blocks, void* out, int64_t nblocks);
 int launch_q4k_dequant_f32(const void* blocks, void* out, int64_t nblocks);
 
+// gdn_chunk.hip: the chunked form of the recurrence (f32 matrix instruction), between gdn_prefill's preparation and output norm
+size_t gdn_chunk_workspace_bytes(int Hg, int T);
+int launch_gdn_chunked_core(const void* conv_out, const float* A_log, const void* dt_bias, const float* a_p, const float* qk, const float* gates,
+                            const float* S_in, float* S_out, float* o_raw, void* workspace, size_t workspace_bytes, int Hg, int T);
 // gdn_prefill.hip
-size_t gdn_prefill_workspace_bytes(int Hg, int T);
+size_t gdn_prefill_workspace_bytes(int Hg, int T, bool chunked = false);
 int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
                        const float* b_p, const float* norm_w, const float* S_in, void* out, float* S_out, void* workspace,
-                       size_t workspace_bytes, int Hg, int T);
+                       size_t workspace_bytes, int Hg, int T, bool chunked = false);
 
 // quant_q4k.hip
 int launch_quantize_q4k(const void* w, int w_dtype, void* out, int64_t rows, int K);

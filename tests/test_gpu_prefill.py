@@ -70,6 +70,37 @@ def test_gdn_prefill_is_T_decode_steps(orc, Hg, T):
         rt.cuFree(p)
 
 
+@pytest.mark.parametrize("Hg,T", [(2, 1), (3, 5), (2, 64), (4, 65), (3, 200), (16, 1024)])
+def test_gdn_prefill_chunked_form_against_the_scan(Hg, T):
+    """chunked=1 (chunks of 64 tokens, f32 matrix instruction) against the scan, which has the checker's bits: the
+    state within 2e-5 of the largest state element, the bf16 outputs within one step of bf16 (2^-7 relative) — the two
+    forms add the same f32 terms in different orders.  Covers a lone token, a partial chunk, exactly one chunk, a
+    partial chunk behind full ones, and a 16-chunk run with strong and weak decays in the same head."""
+    print(f"gdn_prefill chunked Hg={Hg} T={T}", flush=True)
+    g = synth.rng(8200 + Hg + T)
+    C = 3 * Hg * 128
+    conv = bf(g.standard_normal((T, C)).astype(np.float32))
+    z = bf(g.standard_normal((T, Hg * 128)).astype(np.float32))
+    A_log = g.uniform(-2, 1, Hg).astype(np.float32)
+    dt_bias = bf(g.standard_normal(Hg).astype(np.float32))
+    a_p = (g.standard_normal((T, Hg)) * 2).astype(np.float32); b_p = g.standard_normal((T, Hg)).astype(np.float32)
+    norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    S = (g.standard_normal((Hg, 128, 128)) * 0.02).astype(np.float32)
+    res = []
+    for chunked in (0, 1):
+        ptrs = [rt.to_device(a) for a in (conv, z, A_log, dt_bias, a_p, b_p, norm_w, S)]
+        dout = rt.cuAlloc(T * Hg * 128 * 2)
+        rt.cuMemset(dout, 0xff, T * Hg * 128 * 2)
+        _launch(f"gdn_prefill LVH={Hg} T={T} chunked={chunked}", ptrs + [dout, ptrs[7]])
+        res.append((f32(rt.from_device(dout, (T, Hg * 128), np.uint16)).astype(np.float64), rt.from_device(ptrs[7], S.shape, np.float32).astype(np.float64)))
+        for p in ptrs + [dout]:
+            rt.cuFree(p)
+    (o0, S0), (o1, S1) = res
+    assert np.isfinite(o1).all() and np.isfinite(S1).all()
+    assert np.abs(S1 - S0).max() <= 2e-5 * np.abs(S0).max(), (np.abs(S1 - S0).max(), np.abs(S0).max())
+    assert np.all(np.abs(o1 - o0) <= 2.0 ** -7 * np.abs(o0) + 1e-4), np.abs(o1 - o0).max()
+
+
 @pytest.mark.parametrize("T,pos0,splits", [(6, 0, 0), (37, 12, 0), (37, 60, 3), (2, 15, 2)])
 def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits):
     """The matrix-instruction form (exact=0): two consecutive tokens per workgroup (their heads side by side in the 16 columns of the products, each column
