@@ -49,18 +49,39 @@ __device__ __forceinline__ f32x16_t zero16() {
   return z;
 }
 
+// Rows of 128 f32 from memory (`stride` floats apart) straight into the padded rows of an LDS operand: lane l of a wave
+// fills float l of a half row (global_load_lds_dword), the waves of the workgroup take the half rows in turn.  Nothing
+// waits here; the caller waits for its own requests (vmcnt) and then for the other waves' (barrier).
+__device__ __forceinline__ void rows_to_lds(const float* src, int64_t stride, int row_last, float (*dst)[GC_LD], int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < GC_C * 2 / 4; i++) {
+    const int piece = 4 * i + wave, r = piece >> 1, hh = piece & 1;
+    __builtin_amdgcn_global_load_lds(src + (int64_t)min(r, row_last) * stride + 64 * hh + lane, &dst[r][64 * hh], 4, 0, 0);
+  }
+}
+__device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }      // vmcnt(0)
+
 // ---- kernel 1, per (head, chunk): g, T = (I + N)^-1, W, Uv
 __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
   __shared__ float Ks[GC_C][GC_LD], Vs[GC_C][GC_LD];
   __shared__ float Ns[GC_C][GC_C + 1], Ts[GC_C][GC_C + 1];
   __shared__ float g_s[GC_C], beta_s[GC_C], cw_s[GC_C];
-  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5,
+            col = lane & 31;
   const int t0 = c * GC_C, KEYDIM = A.Hg * GC_D;
-  for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
-    const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
-    const bool valid = t < A.T;
-    Ks[tt][i] = valid ? A.qk[(((int64_t)t * A.Hg + h) * 2 + 1) * GC_D + i] : 0.0f;
-    Vs[tt][i] = valid ? bf16_to_f32(A.conv_out[(int64_t)t * 3 * KEYDIM + 2 * KEYDIM + h * GC_D + i]) : 0.0f;
+  // k^ of the chunk's tokens (rows past the run repeat the last token: beta = 0 keeps them out of every sum); v as f32
+  const int last = min(GC_C, A.T - t0) - 1;
+  rows_to_lds(A.qk + (((int64_t)t0 * A.Hg + h) * 2 + 1) * GC_D, (int64_t)A.Hg * 2 * GC_D, last, Ks, wave, lane);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int e = tid + 256 * i, tt = e >> 4, i8 = (e & 15) * 8;
+    const uint4 raw = *(const uint4*)(A.conv_out + (int64_t)(t0 + min(tt, last)) * 3 * KEYDIM + 2 * KEYDIM + h * GC_D + i8);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      Vs[tt][i8 + 2 * q] = __uint_as_float(w[q] << 16);
+      Vs[tt][i8 + 2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u);
+    }
   }
   if (tid < GC_C) {
     const int t = t0 + tid;
@@ -79,6 +100,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
     g_s[tid] = g; beta_s[tid] = beta; cw_s[tid] = beta * expf(g);
     A.G[((int64_t)h * A.nC + c) * GC_C + tid] = g;
   }
+  wait_own_loads();
   __syncthreads();
   // K K^T: wave w owns tile (w / 2, w % 2); tile (0, 1) lies above the diagonal
   {
@@ -132,35 +154,41 @@ __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
 }
 
 // ---- kernel 2, per (head, slab of 32 value columns): the states, chunk after chunk.  Wave w keeps rows 32 w .. + 32
-// of the slab in the accumulators of one 32x32 tile.
+// of the slab in the accumulators of one 32x32 tile.  W and k^ of a chunk arrive in LDS while the chunk before is worked
+// on: k^ in one of two buffers, requested a whole chunk ahead; W in its single buffer as soon as the last reader of the
+// previous W is done.
 __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
-  __shared__ float Wc[GC_C][GC_LD], Kc[GC_C][GC_LD];
+  __shared__ float Wc[GC_C][GC_LD], Kc[2][GC_C][GC_LD];
   __shared__ float red[4][GC_C][33];
   __shared__ float Ut[GC_C][33];
-  __shared__ float g_s[GC_C];
-  const int h = blockIdx.x, sl = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  __shared__ float g_s[2][GC_C];
+  const int h = blockIdx.x, sl = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5,
+            col = lane & 31;
+  const int64_t kstride = (int64_t)A.Hg * 2 * GC_D;
+  auto k_rows = [&](int c) { return A.qk + (((int64_t)c * GC_C * A.Hg + h) * 2 + 1) * GC_D; };
+  auto last_row = [&](int c) { return min(GC_C, A.T - c * GC_C) - 1; };
   f32x16_t S;
   {
     const float* Si = A.S_in + (int64_t)h * GC_D * GC_D + 32 * sl + col;
 #pragma unroll
     for (int r = 0; r < 16; r++) S[r] = Si[(int64_t)(32 * wave + mrow(r, half)) * GC_D];
   }
+  rows_to_lds(A.W + (int64_t)h * A.nC * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
+  rows_to_lds(k_rows(0), kstride, last_row(0), Kc[0], wave, lane);
+  if (tid < GC_C) g_s[0][tid] = A.G[(int64_t)h * A.nC * GC_C + tid];
   for (int c = 0; c < A.nC; c++) {
     const int64_t hc = (int64_t)h * A.nC + c;
-    const int t0 = c * GC_C;
-    __syncthreads();                                   // the previous chunk's readers are done
-    for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
-      const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
-      Wc[tt][i] = A.W[(hc * GC_C + tt) * GC_D + i];
-      Kc[tt][i] = t < A.T ? A.qk[(((int64_t)t * A.Hg + h) * 2 + 1) * GC_D + i] : 0.0f;
+    wait_own_loads();
+    __syncthreads();                                   // W, k^ and g of this chunk are in LDS; the previous chunk's readers are done
+    if (c + 1 < A.nC) {
+      rows_to_lds(k_rows(c + 1), kstride, last_row(c + 1), Kc[(c + 1) & 1], wave, lane);
+      if (tid < GC_C) g_s[(c + 1) & 1][tid] = A.G[(hc + 1) * GC_C + tid];
     }
-    if (tid < GC_C) g_s[tid] = A.G[hc * GC_C + tid];
     {
       float* Ho = A.Hs + hc * GC_D * GC_D + 32 * sl + col;
 #pragma unroll
       for (int r = 0; r < 16; r++) Ho[(int64_t)(32 * wave + mrow(r, half)) * GC_D] = S[r];
     }
-    __syncthreads();
     // this wave's share of W S: the sum over its 32 rows of S, taken in the order the accumulator holds them
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
@@ -171,21 +199,24 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
       for (int r = 0; r < 16; r++) red[wave][32 * tt + mrow(r, half)][col] = P[r];
     }
     __syncthreads();
-    const float gC = g_s[GC_C - 1];
+    if (c + 1 < A.nC) rows_to_lds(A.W + (hc + 1) * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
+    const float* gc = g_s[c & 1];
+    const float gC = gc[GC_C - 1];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const int e = tid + 256 * i, t = e >> 5, n = e & 31;
       float* up = A.U + (hc * GC_C + t) * GC_D + 32 * sl + n;
       const float u = *up - (((red[0][t][n] + red[1][t][n]) + red[2][t][n]) + red[3][t][n]);
       *up = u;
-      Ut[t][n] = u * expf(gC - g_s[t]);
+      Ut[t][n] = u * expf(gC - gc[t]);
     }
     __syncthreads();
     const float dC = expf(gC);
 #pragma unroll
     for (int r = 0; r < 16; r++) S[r] *= dC;
+    const float (*Kcur)[GC_LD] = Kc[c & 1];
 #pragma unroll 8
-    for (int s = 0; s < GC_C / 2; s++) S = __builtin_amdgcn_mfma_f32_32x32x2f32(Kc[2 * s + half][32 * wave + col], Ut[2 * s + half][col], S, 0, 0, 0);
+    for (int s = 0; s < GC_C / 2; s++) S = __builtin_amdgcn_mfma_f32_32x32x2f32(Kcur[2 * s + half][32 * wave + col], Ut[2 * s + half][col], S, 0, 0, 0);
   }
   float* So = A.S_out + (int64_t)h * GC_D * GC_D + 32 * sl + col;
 #pragma unroll
@@ -197,18 +228,20 @@ __global__ __launch_bounds__(256) void gdn_chunk_out_kernel(GdnChunkArgs A) {
   __shared__ float Qs[GC_C][GC_LD], Ks[GC_C][GC_LD], Us[GC_C][GC_LD];
   __shared__ float Ms[GC_C][GC_C + 1];
   __shared__ float g_s[GC_C];
-  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const int h = blockIdx.x, c = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5,
+            col = lane & 31;
   const int t0 = c * GC_C;
   const int64_t hc = (int64_t)h * A.nC + c;
-  for (int idx = tid; idx < GC_C * GC_D; idx += 256) {
-    const int tt = idx >> 7, i = idx & 127, t = t0 + tt;
-    const bool valid = t < A.T;
-    const float* qk = A.qk + ((int64_t)min(t, A.T - 1) * A.Hg + h) * 2 * GC_D;
-    Qs[tt][i] = valid ? qk[i] : 0.0f;
-    Ks[tt][i] = valid ? qk[GC_D + i] : 0.0f;
-    Us[tt][i] = A.U[(hc * GC_C + tt) * GC_D + i];
+  {
+    // (rows past the run repeat the last token; their U rows are zero and their outputs are not stored)
+    const int last = min(GC_C, A.T - t0) - 1;
+    const float* qk = A.qk + ((int64_t)t0 * A.Hg + h) * 2 * GC_D;
+    rows_to_lds(qk, (int64_t)A.Hg * 2 * GC_D, last, Qs, wave, lane);
+    rows_to_lds(qk + GC_D, (int64_t)A.Hg * 2 * GC_D, last, Ks, wave, lane);
+    rows_to_lds(A.U + hc * GC_C * GC_D, GC_D, GC_C - 1, Us, wave, lane);
   }
   if (tid < GC_C) g_s[tid] = A.G[hc * GC_C + tid];
+  wait_own_loads();
   __syncthreads();
   {
     const int ti = wave >> 1, tj = wave & 1;
