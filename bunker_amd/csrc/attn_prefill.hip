@@ -45,7 +45,7 @@ struct PrefillAttnArgs {
   float scale_log2;                // softmax scale times log2(e)
 };
 
-// K/V tiles travel from memory straight into LDS (global_load_lds_dwordx4: lane l of a wave fills the l-th 16-byte
+// K/V tiles travel from memory straight into LDS (lds_dma16: lane l of a wave fills the l-th 16-byte
 // slot of a 1 KiB piece of LDS from an address of its own choosing), two tiles deep: no registers hold them and no
 // wave spends instructions on the copy.  A slot's position is fixed by the lane, so rows cannot be padded against bank
 // conflicts; instead the 16-byte units of a row are stored exclusive-or'ed with a few bits of the row number
@@ -100,14 +100,14 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
       const int piece = 4 * i + wave;
       const int row = 2 * piece + (lane >> 5), unit = (lane & 31) ^ (row & 15);
       const uint16_t* src = A.kc + page_base(tile * 4 + (row >> 4)) + (row & 15) * ATT_HD + unit * 8;
-      __builtin_amdgcn_global_load_lds(src, kb + piece * 1024, 16, 0, 0);
+      lds_dma16(src, kb + piece * 1024);
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const int piece = 4 * i + wave;
       const int dim = 8 * piece + (lane >> 3), unit = (lane & 7) ^ ((dim >> 1) & 7);     // unit = 2 * page + half of the page's tokens
       const uint16_t* src = A.vc + page_base(tile * 4 + (unit >> 1)) + dim * ATT_PAGE + (unit & 1) * 8;
-      __builtin_amdgcn_global_load_lds(src, vb + piece * 1024, 16, 0, 0);
+      lds_dma16(src, vb + piece * 1024);
     }
   };
   // What the cache holds behind the longest row need not be a number, and 0 * NaN would reach the output: the values

@@ -254,4 +254,20 @@ __device__ __forceinline__ double block_sum_f64(double v, double* lds) {
 }
 
 #endif  // __HIPCC__
+// Memory -> LDS without a register in between: lane l of the wave fills the l-th 16-byte (4-byte) slot of the LDS piece
+// that starts at `lds_piece` (the same address in every lane) from an address of its own choosing.  Written as
+// instructions, not through the compiler's builtin: the compiler would put a wait for the whole transfer in front of the
+// next LDS access of any kind (it cannot tell which LDS bytes a transfer in flight will write), and a tile requested
+// a step ahead would be waited for at once.  The caller waits itself (s_waitcnt vmcnt) before the barrier that hands
+// the piece to its readers.  m0 carries the LDS address; nothing else in these kernels uses that register.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lds_dma16(const void* src, const void* lds_piece) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma4(const void* src, const void* lds_piece) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 }  // namespace bk

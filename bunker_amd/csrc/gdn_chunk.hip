@@ -49,17 +49,47 @@ __device__ __forceinline__ f32x16_t zero16() {
   return z;
 }
 
+// acc += sum over STEPS steps of A-operand fa(step) x B-operand fb(step): the operands of 16 steps are fetched (from LDS,
+// memory or registers, as fa / fb say) before the 16 matrix instructions of the 16 steps before them are issued, so a
+// wave that has nothing else to run does not sit out an operand's latency in front of every instruction.
+template <int STEPS, class FA, class FB>
+__device__ __forceinline__ f32x16_t mfma_run(f32x16_t acc, FA fa, FB fb) {
+  static_assert(STEPS % 16 == 0, "whole batches");
+  float a[2][16], b[2][16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) { a[0][i] = fa(i); b[0][i] = fb(i); }
+#pragma unroll
+  for (int bt = 0; bt < STEPS / 16; bt++) {
+    if (bt + 1 < STEPS / 16) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) { a[(bt + 1) & 1][i] = fa(16 * (bt + 1) + i); b[(bt + 1) & 1][i] = fb(16 * (bt + 1) + i); }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[bt & 1][i], b[bt & 1][i], acc, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  return acc;
+}
+
 // Rows of 128 f32 from memory (`stride` floats apart) straight into the padded rows of an LDS operand: lane l of a wave
-// fills float l of a half row (global_load_lds_dword), the waves of the workgroup take the half rows in turn.  Nothing
+// fills float l of a half row (lds_dma4), the waves of the workgroup take the half rows in turn.  Nothing
 // waits here; the caller waits for its own requests (vmcnt) and then for the other waves' (barrier).
 __device__ __forceinline__ void rows_to_lds(const float* src, int64_t stride, int row_last, float (*dst)[GC_LD], int wave, int lane) {
 #pragma unroll
   for (int i = 0; i < GC_C * 2 / 4; i++) {
     const int piece = 4 * i + wave, r = piece >> 1, hh = piece & 1;
-    __builtin_amdgcn_global_load_lds(src + (int64_t)min(r, row_last) * stride + 64 * hh + lane, &dst[r][64 * hh], 4, 0, 0);
+    lds_dma4(src + (int64_t)min(r, row_last) * stride + 64 * hh + lane, &dst[r][64 * hh]);
   }
 }
 __device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }      // vmcnt(0)
+// A workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global store of the wave
+// (its fence covers all memory), which the state kernel would pay three times per chunk for stores nobody here reads.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 // ---- kernel 1, per (head, chunk): g, T = (I + N)^-1, W, Uv
 __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
@@ -106,11 +136,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
   {
     const int ti = wave >> 1, tj = wave & 1;
     f32x16_t acc = zero16();
-    if (wave != 1) {
-#pragma unroll 8
-      for (int s = 0; s < GC_D / 2; s++)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ks[32 * ti + col][2 * s + half], Ks[32 * tj + col][2 * s + half], acc, 0, 0, 0);
-    }
+    if (wave != 1)
+      acc = mfma_run<GC_D / 2>(acc, [&](int s) { return Ks[32 * ti + col][2 * s + half]; }, [&](int s) { return Ks[32 * tj + col][2 * s + half]; });
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int t = 32 * ti + mrow(r, half), j = 32 * tj + col;
@@ -118,18 +145,35 @@ __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
     }
   }
   __syncthreads();
-  // T = (I + N)^-1 by forward substitution, one wave: lane = column, row i needs rows 0 .. i-1
-  if (wave == 0) {
-    float Tr[GC_C];
+  // T = (I + N)^-1 in two levels.  Waves 0 and 1 invert the diagonal 32x32 blocks by forward substitution (lane =
+  // column, row i needs rows 0 .. i-1); the block under the diagonal is then T21 = -T22 (N21 T11), two matrix products.
+  if (wave < 2) {
+    const int o32 = 32 * wave;
+    float Tr[32];
 #pragma unroll
-    for (int i = 0; i < GC_C; i++) {
-      const float nrow = Ns[i][lane];
-      float a = lane == i ? 1.0f : 0.0f;
+    for (int i = 0; i < 32; i++) {
+      const float nrow = Ns[o32 + i][o32 + col];
+      float a = col == i ? 1.0f : 0.0f;
 #pragma unroll
       for (int j = 0; j < i; j++) a -= __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(nrow), j)) * Tr[j];
       Tr[i] = a;
-      Ts[i][lane] = a;
+      if (half == 0) { Ts[o32 + i][o32 + col] = a; if (wave == 0) Ts[i][32 + col] = 0.0f; }
     }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    f32x16_t X = mfma_run<16>(zero16(), [&](int s) { return Ns[32 + col][2 * s + half]; }, [&](int s) { return Ts[2 * s + half][col]; });
+    // X = N21 T11 takes N21's place (this wave is its only reader), then T21 = -(T22 X)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < 16; r++) Ns[32 + mrow(r, half)][col] = X[r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    f32x16_t Y = mfma_run<16>(zero16(), [&](int s) { return Ts[32 + col][32 + 2 * s + half]; }, [&](int s) { return Ns[32 + 2 * s + half][col]; });
+#pragma unroll
+    for (int r = 0; r < 16; r++) Ts[32 + mrow(r, half)][col] = -Y[r];
   }
   __syncthreads();
   // W = T diag(beta e^g) K and Uv = T diag(beta) V: wave w owns the 32 columns 32 w .. of both, T's zeros above the diagonal skipped
@@ -138,15 +182,11 @@ __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
   for (int which = 0; which < 2; which++)
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
-      f32x16_t acc = zero16();
       const float (*B)[GC_LD] = which ? Vs : Ks;
       const float* coef = which ? beta_s : cw_s;
-      const int steps = 16 * (tt + 1);
-#pragma unroll 8
-      for (int s = 0; s < steps; s++) {
-        const int j = 2 * s + half;
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ts[32 * tt + col][j] * coef[j], B[j][32 * wave + col], acc, 0, 0, 0);
-      }
+      auto fa = [&](int s) { const int j = 2 * s + half; return Ts[32 * tt + col][j] * coef[j]; };
+      auto fb = [&](int s) { return B[2 * s + half][32 * wave + col]; };
+      const f32x16_t acc = tt ? mfma_run<32>(zero16(), fa, fb) : mfma_run<16>(zero16(), fa, fb);
       float* dst = (which ? A.U : A.W) + (hc * GC_C + 32 * tt) * GC_D + 32 * wave + col;
 #pragma unroll
       for (int r = 0; r < 16; r++) dst[(int64_t)mrow(r, half) * GC_D] = acc[r];
@@ -176,13 +216,19 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
   rows_to_lds(A.W + (int64_t)h * A.nC * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
   rows_to_lds(k_rows(0), kstride, last_row(0), Kc[0], wave, lane);
   if (tid < GC_C) g_s[0][tid] = A.G[(int64_t)h * A.nC * GC_C + tid];
+  wait_own_loads();
   for (int c = 0; c < A.nC; c++) {
     const int64_t hc = (int64_t)h * A.nC + c;
-    wait_own_loads();
-    __syncthreads();                                   // W, k^ and g of this chunk are in LDS; the previous chunk's readers are done
-    if (c + 1 < A.nC) {
-      rows_to_lds(k_rows(c + 1), kstride, last_row(c + 1), Kc[(c + 1) & 1], wave, lane);
-      if (tid < GC_C) g_s[(c + 1) & 1][tid] = A.G[(hc + 1) * GC_C + tid];
+    lds_barrier();                                   // W, k^ and g of this chunk are in LDS; the previous chunk's readers are done
+    // requests of this step, oldest first: k^ of the next chunk, its g, this chunk's Uv (used after the first product)
+    const bool more = c + 1 < A.nC;
+    if (more) rows_to_lds(k_rows(c + 1), kstride, last_row(c + 1), Kc[(c + 1) & 1], wave, lane);
+    const float gnext = A.G[(hc + (more ? 1 : 0)) * GC_C + (tid & 63)];
+    float uv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int e = tid + 256 * i;
+      uv[i] = A.U[(hc * GC_C + (e >> 5)) * GC_D + 32 * sl + (e & 31)];
     }
     {
       float* Ho = A.Hs + hc * GC_D * GC_D + 32 * sl + col;
@@ -192,31 +238,31 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
     // this wave's share of W S: the sum over its 32 rows of S, taken in the order the accumulator holds them
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
-      f32x16_t P = zero16();
-#pragma unroll
-      for (int r = 0; r < 16; r++) P = __builtin_amdgcn_mfma_f32_32x32x2f32(Wc[32 * tt + col][32 * wave + mrow(r, half)], S[r], P, 0, 0, 0);
+      const f32x16_t P = mfma_run<16>(zero16(), [&](int r) { return Wc[32 * tt + col][32 * wave + mrow(r, half)]; }, [&](int r) { return S[r]; });
 #pragma unroll
       for (int r = 0; r < 16; r++) red[wave][32 * tt + mrow(r, half)][col] = P[r];
     }
-    __syncthreads();
-    if (c + 1 < A.nC) rows_to_lds(A.W + (hc + 1) * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
+    lds_barrier();
+    if (more) rows_to_lds(A.W + (hc + 1) * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
     const float* gc = g_s[c & 1];
     const float gC = gc[GC_C - 1];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const int e = tid + 256 * i, t = e >> 5, n = e & 31;
-      float* up = A.U + (hc * GC_C + t) * GC_D + 32 * sl + n;
-      const float u = *up - (((red[0][t][n] + red[1][t][n]) + red[2][t][n]) + red[3][t][n]);
-      *up = u;
+      const float u = uv[i] - (((red[0][t][n] + red[1][t][n]) + red[2][t][n]) + red[3][t][n]);
       Ut[t][n] = u * expf(gC - gc[t]);
+      A.U[(hc * GC_C + t) * GC_D + 32 * sl + n] = u;
     }
-    __syncthreads();
+    if (tid < GC_C) g_s[(c + 1) & 1][tid] = gnext;
+    lds_barrier();
     const float dC = expf(gC);
 #pragma unroll
     for (int r = 0; r < 16; r++) S[r] *= dC;
     const float (*Kcur)[GC_LD] = Kc[c & 1];
-#pragma unroll 8
-    for (int s = 0; s < GC_C / 2; s++) S = __builtin_amdgcn_mfma_f32_32x32x2f32(Kcur[2 * s + half][32 * wave + col], Ut[2 * s + half][col], S, 0, 0, 0);
+    S = mfma_run<GC_C / 2>(S, [&](int s) { return Kcur[2 * s + half][32 * wave + col]; }, [&](int s) { return Ut[2 * s + half][col]; });
+    // the 8 stores of U are the youngest requests of this wave; everything older — the next chunk's W and k^ among
+    // it — has to be in LDS before the barrier at the top, the stores may stay in flight
+    __builtin_amdgcn_s_waitcnt(0x0F70 | 8);            // vmcnt(8)
   }
   float* So = A.S_out + (int64_t)h * GC_D * GC_D + 32 * sl + col;
 #pragma unroll
@@ -246,11 +292,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_out_kernel(GdnChunkArgs A) {
   {
     const int ti = wave >> 1, tj = wave & 1;
     f32x16_t acc = zero16();
-    if (wave != 1) {
-#pragma unroll 8
-      for (int s = 0; s < GC_D / 2; s++)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[32 * ti + col][2 * s + half], Ks[32 * tj + col][2 * s + half], acc, 0, 0, 0);
-    }
+    if (wave != 1)
+      acc = mfma_run<GC_D / 2>(acc, [&](int s) { return Qs[32 * ti + col][2 * s + half]; }, [&](int s) { return Ks[32 * tj + col][2 * s + half]; });
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int t = 32 * ti + mrow(r, half), j = 32 * tj + col;
@@ -259,31 +302,18 @@ __global__ __launch_bounds__(256) void gdn_chunk_out_kernel(GdnChunkArgs A) {
   }
   __syncthreads();
   // wave w owns value columns 32 w .. + 32: diag(e^g) Q S_0, the state read straight from memory as the B operand
-  // (a lane's 64 loads per tile are issued 16 ahead of the 16 instructions that use them), then M U
+  // (mfma_run keeps a lane's loads 16 ahead of the instructions that use them), then M U
   const float* Hc = A.Hs + hc * GC_D * GC_D + 32 * wave + col;
 #pragma unroll
   for (int tt = 0; tt < 2; tt++) {
-    f32x16_t acc = zero16();
-    float sb[2][16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) sb[0][i] = Hc[(int64_t)(2 * i + half) * GC_D];
-#pragma unroll
-    for (int bt = 0; bt < 4; bt++) {
-      if (bt + 1 < 4) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) sb[(bt + 1) & 1][i] = Hc[(int64_t)(2 * (16 * (bt + 1) + i) + half) * GC_D];
-      }
-#pragma unroll
-      for (int i = 0; i < 16; i++)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[32 * tt + col][2 * (16 * bt + i) + half], sb[bt & 1][i], acc, 0, 0, 0);
-    }
+    f32x16_t acc = mfma_run<GC_D / 2>(zero16(), [&](int s) { return Qs[32 * tt + col][2 * s + half]; },
+                                      [&](int s) { return Hc[(int64_t)(2 * s + half) * GC_D]; });
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] *= expf(g_s[32 * tt + mrow(r, half)]);
-    const int steps = 16 * (tt + 1);
-#pragma unroll 8
-    for (int s = 0; s < steps; s++) {
-      const int j = 2 * s + half;
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ms[32 * tt + col][j], Us[j][32 * wave + col], acc, 0, 0, 0);
+    {
+      auto fa = [&](int s) { return Ms[32 * tt + col][2 * s + half]; };
+      auto fb = [&](int s) { return Us[2 * s + half][32 * wave + col]; };
+      acc = tt ? mfma_run<32>(acc, fa, fb) : mfma_run<16>(acc, fa, fb);
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) {
