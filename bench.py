@@ -280,7 +280,21 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     pf.run(prompt, 0, 0)
     wall = time.perf_counter() - t0
     pf.close()
-    out["prefill"]["with_bf16_mfma_attention"] = {"tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2)}
+    out["prefill"]["with_bf16_mfma_attention"] = {"tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
+                                                  "attention": "query tile x K/V tile on the bf16 matrix cores (fa2_prefill exact=0)"}
+    # the reference's prefill forms on both ops that couple tokens: tiled bf16 attention and the chunked GDN recurrence
+    runner.ATTN_EXACT = False
+    pf = prefill.Prefill(D, envs[0], chunk=chunk, gdn_chunked=True)
+    runner.ATTN_EXACT = True
+    pf.run(prompt, 0, 0)
+    rt.cuSync()
+    t0 = time.perf_counter()
+    tok_c, _ = pf.run(prompt, 0, 0)
+    wall = time.perf_counter() - t0
+    pf.close()
+    out["prefill"]["with_tiled_attention_and_chunked_gdn"] = {"tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
+                                                              "first_generated_token": tok_c,
+                                                              "gdn": "chunks of 64 tokens on the f32 matrix instruction (gdn_prefill chunked=1)"}
     for env in envs:
         env.close()
     # the reference model's own dimensions (src/model.ts:14-18), random Q4_K weights, KV at 4096: batch 1 only

@@ -44,14 +44,18 @@ class _Slot:
 
 
 class Prefill:
-    def __init__(self, D: Dims, env: DecodeEnv, chunk: int = 1024, on_attention: Callable | None = None, overlap: bool | int = True):
+    def __init__(self, D: Dims, env: DecodeEnv, chunk: int = 1024, on_attention: Callable | None = None, overlap: bool | int = True,
+                 gdn_chunked: bool = False):
         """``env`` supplies the weights and the state buffers (those of sequence ``seq`` are updated in place).
         ``on_attention(layer, first_token_index, rows)`` receives each full-attention layer's output
         (uint16 bf16 bits ``[T, NH*HD]``) as it is produced — for tests.  ``overlap``: chunks in flight (True = 2,
-        False = 1: everything on the library's first stream)."""
+        False = 1: everything on the library's first stream).  ``gdn_chunked``: the Gated-DeltaNet recurrence in chunks of
+        64 tokens on the f32 matrix instruction (the form of the reference's prefill prototypes) instead of the scan;
+        state and outputs then agree with T decode steps to ~1e-6 relative, not to the bit."""
         if chunk < 1 or chunk > 4096:
             raise ValueError("Prefill: chunk must be 1..4096 tokens")
         self.D, self.env, self.chunk, self.on_attention = D, env, int(chunk), on_attention
+        self.gdn_chunked = bool(gdn_chunked)
         self.attn_exact = bool(_runner.ATTN_EXACT)       # double-precision attention, or the matrix-instruction form (runner.ATTN_EXACT)
         self._owned: list[int] = []
         in_flight = 2 if overlap is True else max(int(overlap), 1)
@@ -99,7 +103,7 @@ class Prefill:
             "embed": c(f"embed H={D.H} VOCAB={D.VOCAB} ids_dev=1" + bp),
             "gdn_in": c(f"gemv_fused K={D.H} pro=2 G=4 N0={D.QKVD} epi0=1 N1={D.ZD} epi1=1 N2={D.LVH} epi2=0 N3={D.LVH} epi3=0" + bp),
             "conv": c(f"conv1d_prefill QKVD={D.QKVD} T={T}"),
-            "gdn": c(f"gdn_prefill LVH={D.LVH} T={T}"),
+            "gdn": c(f"gdn_prefill LVH={D.LVH} T={T}" + (" chunked=1" if self.gdn_chunked else "")),
             "gdn_out": c(f"gemv_fused K={D.ZD} pro=1 G=1 N0={D.H} epi0=2" + bp),
             "fa_in": c(f"gemv_fused K={D.H} pro=2 G=3 N0={D.QGATE} epi0=1 N1={D.KV_DIM} epi1=1 N2={D.KV_DIM} epi2=1" + bp),
             "fa": c(f"fa2_prefill HD={D.HD} NH={D.NH} NKV={D.NKV} MAX_LEN={D.MAX_LEN} ROT_HALF={D.ROT_HALF} T={T}"

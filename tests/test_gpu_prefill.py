@@ -321,3 +321,48 @@ def test_prefill_two_chunks_in_flight_equals_one(orc, n_prompt, chunk):
     for other in results[1:]:
         for key, v in results[0].items():
             assert np.array_equal(v, other[key]), key
+
+
+def test_prefill_in_the_chunked_and_tiled_forms_stays_close_to_the_exact_one():
+    """A TINY-model prompt through the forms of the reference's prefill prototypes (fa2_prefill exact=0: tiled bf16
+    attention; gdn_prefill chunked=1: chunks of 64 tokens in f32) against the default forms, which leave the bits of
+    token-by-token decoding: the conv rows are the same bytes (that op has one form), the GDN states agree to 1e-3 of
+    their largest element and the logits of the last prompt token to 0.05 — the differences are the rounding of
+    attention weights to bf16 and the order of the f32 additions, carried through the layers by the bf16 activations."""
+    print("prefill chunked/tiled vs exact", flush=True)
+    from dataclasses import replace
+    D = replace(TINY, MAX_LEN=256)
+    B, seq, n_prompt, chunk = 2, 1, 150, 96
+    W = synth_model.synth_weights(D, seed=61)
+    S = synth_model.synth_state(D, B, seed=62)
+    for key in S:
+        if key.endswith("conv_state") or key.endswith("s_state"):
+            S[key][seq] = 0
+    prompt = synth.rng(63).integers(0, D.VOCAB, n_prompt).astype(np.int32)
+    g = model.buildModelGraph(D, B)
+    results = []
+    for fast in (False, True):
+        env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
+        runner.ATTN_EXACT = not fast
+        try:
+            pf = prefill.Prefill(D, env, chunk=chunk, gdn_chunked=fast)
+        finally:
+            runner.ATTN_EXACT = True
+        tok, val = pf.run(prompt, seq=seq, pos0=0)
+        state = {"logits": rt.from_device(pf.d_logits, (D.VOCAB,), np.float32).astype(np.float64), "tok": tok}
+        for l in range(D.NL):
+            p = f"model.layers.{l}"
+            if not D.is_full_attention(l):
+                state[p + ".S"] = env.read_state(f"{p}.s_state", (B, D.LVH, 128, 128), np.float32).astype(np.float64)
+                state[p + ".conv"] = env.read_state(f"{p}.conv_state", (B, 3, D.QKVD), np.uint16)
+        results.append(state)
+        pf.close()
+        env.close()
+    exact, fast = results
+    first_gdn = next(l for l in range(D.NL) if not D.is_full_attention(l))
+    assert np.array_equal(exact[f"model.layers.{first_gdn}.conv"], fast[f"model.layers.{first_gdn}.conv"])     # same inputs, one form
+    for key, v in exact.items():
+        if key.endswith(".S"):
+            assert np.abs(fast[key] - v).max() <= 1e-3 * np.abs(v).max(), (key, np.abs(fast[key] - v).max(), np.abs(v).max())
+    assert np.isfinite(fast["logits"]).all()
+    assert np.abs(fast["logits"] - exact["logits"]).max() <= 0.05, np.abs(fast["logits"] - exact["logits"]).max()
