@@ -220,11 +220,18 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
       pb[j] = make_uint4(pk_bf16(p[0], p[1]), pk_bf16(p[2], p[3]), pk_bf16(p[4], p[5]), pk_bf16(p[6], p[7]));
     }
     lrow = lrow * alpha + psum;
-    if (__ballot(alpha != 1.0f) != 0ull) {
+    if (__builtin_expect(__ballot(alpha != 1.0f) != 0ull, 0)) {        // (rare after the first tiles, see above)
 #pragma unroll
       for (int dt = 0; dt < 8; dt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+        for (int r = 0; r < 16; r++) {
+          // (the accumulators live in the matrix unit's registers; the empty statement pins each one there at this
+          // point, so that the copy to a vector register the multiply needs is made here, in the rare branch, and
+          // not for all 128 at the top of every tile)
+          float x = o[dt][r];
+          asm volatile("" : "+a"(x));
+          o[dt][r] = x * alpha;
+        }
     }
     // ---- values: O^T[dim 32 dt + .., row] += V^T . P^T over the four 16-token slices, the A operands again a batch
     // (one slice, eight dim tiles) ahead
