@@ -464,6 +464,69 @@ def bench_kernels(rt, synth, use_graph=True, iters=50):
         dws = 0
         for p in kcs + vcs + [dq, dbt, dctx, dout, dlse] + ([dws] if dws else []):
             rt.cuFree(p)
+    res.update(bench_prefill_ops(rt, synth))
+    return res
+
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
+MFMA_F32_PEAK_TFLOPS = 157.3       # MI355X f32 matrix
+
+
+def bench_prefill_ops(rt, synth, iters=5):
+    """The two prompt ops that couple the tokens of a sequence, each in its forms: causal attention of 1024 prompt tokens
+    behind 15360 cached ones (fa2_prefill: norms, rotation and cache append included) and the Gated-DeltaNet recurrence
+    over 1024 tokens of 16 heads (gdn_prefill: gates, norms and the output norm included)."""
+    g = synth.rng(15)
+    bf = synth.f32_to_bf16
+    res = {}
+
+    def timed(spec, args):
+        h = rt.compileAndLoad(spec)
+        for _ in range(2):
+            rt.cuLaunch(h, [1, 1, 1], [128, 1, 1], args)
+        us = _time_launches(rt, lambda: [rt.cuLaunch(h, [1, 1, 1], [128, 1, 1], args) for _ in range(iters)], False) / iters
+        rt.unloadKernel(h)
+        return us
+
+    NH, NKV, HD, HALF, MAXL, T, pos0 = 16, 2, 256, 32, 16384, 1024, 15360
+    pages = MAXL // 16
+    page = bf(g.standard_normal((64, NKV, 16, HD), dtype=np.float32))
+    cache = np.tile(page, (pages // 64, 1, 1, 1))
+    host = (bf(g.standard_normal((T, NH, 2, HD), dtype=np.float32)), bf(g.standard_normal((T, NKV, HD), dtype=np.float32)),
+            bf(g.standard_normal((T, NKV, HD), dtype=np.float32)), bf((g.standard_normal(HD) * 0.1).astype(np.float32)),
+            bf((g.standard_normal(HD) * 0.1).astype(np.float32)), g.uniform(-1, 1, (MAXL, HALF)).astype(np.float32),
+            g.uniform(-1, 1, (MAXL, HALF)).astype(np.float32), (pos0 + np.arange(T)).astype(np.int32), np.arange(pages, dtype=np.int32))
+    ptrs = [rt.to_device(a) for a in host] + [rt.to_device(cache), rt.to_device(cache), rt.cuAlloc(T * NH * HD * 2)]
+    spec = f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T}"
+    flop = float(sum(pos0 + t + 1 for t in range(T))) * NH * 4 * HD            # 2 products x 2 flop per (row, token, dim)
+    row = {"prompt_tokens": T, "cached_tokens": pos0, "flop": flop}
+    for key, flags in (("tiled_bf16_mfma", " exact=0"), ("decode_kernel_per_token_pair", " exact=0 tiled=0"), ("double_precision", "")):
+        us = timed(spec + flags, ptrs)
+        row[key] = {"us": round(us, 1), "TFLOPs": round(flop / us / 1e6, 1)}
+    row["tiled_bf16_mfma"]["frac_bf16_mfma_peak"] = round(row["tiled_bf16_mfma"]["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4)
+    res["fa2_prefill_T1024_behind_15360"] = row
+    for p in ptrs:
+        rt.cuFree(p)
+
+    Hg, T = 16, 1024
+    C = 3 * Hg * 128
+    host = (bf(g.standard_normal((T, C), dtype=np.float32)), bf(g.standard_normal((T, Hg * 128), dtype=np.float32)),
+            g.uniform(-2, 1, Hg).astype(np.float32), bf(g.standard_normal(Hg).astype(np.float32)),
+            (g.standard_normal((T, Hg)) * 2).astype(np.float32), g.standard_normal((T, Hg)).astype(np.float32),
+            (1 + 0.1 * g.standard_normal(128)).astype(np.float32), (g.standard_normal((Hg, 128, 128)) * 0.02).astype(np.float32))
+    ptrs = [rt.to_device(a) for a in host]
+    args = ptrs + [rt.cuAlloc(T * Hg * 128 * 2), rt.cuAlloc(host[7].nbytes)]
+    # chunked form: per chunk of 64 tokens and head, products of 64x64x128 (K K^T, Q K^T), 2 x 64x64x128 (W, Uv),
+    # 2 x 64x128x128 (W S, K^T U), 64x128x128 (Q S) and 64x64x128 (M U): 11 M multiply-adds
+    flop_chunked = 2.0 * 11 * 64 * 64 * 128 * (T // 64) * Hg
+    row = {"tokens": T, "heads": Hg,
+           "scan": {"us": round(timed(f"gdn_prefill LVH={Hg} T={T}", args), 1)},
+           "chunked_f32_mfma": {"us": round(timed(f"gdn_prefill LVH={Hg} T={T} chunked=1", args), 1)}}
+    row["chunked_f32_mfma"]["TFLOPs"] = round(flop_chunked / row["chunked_f32_mfma"]["us"] / 1e6, 2)
+    row["chunked_f32_mfma"]["frac_f32_mfma_peak"] = round(row["chunked_f32_mfma"]["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4)
+    res["gdn_prefill_T1024_H16"] = row
+    for p in args:
+        rt.cuFree(p)
     return res
 
 
