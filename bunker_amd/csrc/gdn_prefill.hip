@@ -38,26 +38,39 @@ struct GdnPrefillArgs {
   int Hg, T;
 };
 
+// One wave per (token, head, q | k) row of 128 values, two per lane; a workgroup's four waves take 64 consecutive rows,
+// i.e. 32 (token, head) pairs, whose gates — a chain of double-precision exponentials and logarithms, several hundred
+// instructions long whether one lane runs it or 64 — are worked out side by side by 32 lanes of the first wave.
+// (The squares of bf16 values are exact in f32 and their sum over a row is exact in f64, so the order of that sum —
+// here lane pairs first, in the single-token kernel 64-lane halves first — does not show in the result.)
+constexpr int GP_PREP_ROWS = 64;
 __global__ __launch_bounds__(256) void gdn_prefill_prep_kernel(GdnPrefillArgs A) {
-  __shared__ double red[4];
-  const int h = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int KEYDIM = A.Hg * GP_D;
-  const bool isk = tid >= 128;
-  const int i = tid & 127;
-  const uint16_t* row = A.conv_out + (int64_t)t * 3 * KEYDIM;
-  const float x = bf16_to_f32(row[(isk ? KEYDIM : 0) + h * GP_D + i]);
-  const double ss = wave_sum_f64((double)(x * x));       // square of a bf16 value: exact in f32
-  if ((tid & 63) == 0) red[tid >> 6] = ss;
-  __syncthreads();
-  const double tot = isk ? (red[2] + red[3]) : (red[0] + red[1]);
-  const float rs = rsqrt_f64(tot + 1e-6);
-  const int64_t th = (int64_t)t * A.Hg + h;
-  A.qk[(th * 2 + (isk ? 1 : 0)) * GP_D + i] = isk ? x * rs : x * (rs * 0.08838834764831845f);     // 1/sqrt(128)
-  if (tid == 0) {
-    const float sp_in = A.a_p[th] + bf16_to_f32(A.dt_bias[h]);
-    const float softplus = (float)log1p(exp((double)sp_in));
-    A.gates[th * 2] = (float)exp(-(double)((float)exp((double)A.A_log[h]) * softplus));
-    A.gates[th * 2 + 1] = sigmoid_f64(A.b_p[th]);
+  const int64_t nrows = (int64_t)A.T * A.Hg * 2;
+  const int64_t row0 = (int64_t)blockIdx.x * GP_PREP_ROWS;
+  if (wave == 0 && lane < GP_PREP_ROWS / 2) {
+    const int64_t th = (row0 >> 1) + lane;
+    if (th < (int64_t)A.T * A.Hg) {
+      const int h = (int)(th % A.Hg);
+      const float sp_in = A.a_p[th] + bf16_to_f32(A.dt_bias[h]);
+      const float softplus = (float)log1p(exp((double)sp_in));
+      A.gates[th * 2] = (float)exp(-(double)((float)exp((double)A.A_log[h]) * softplus));
+      A.gates[th * 2 + 1] = sigmoid_f64(A.b_p[th]);
+    }
+  }
+  for (int it = 0; it < GP_PREP_ROWS / 4; it++) {
+    const int64_t rowi = row0 + 4 * it + wave;       // (t, h, q | k) in the order of A.qk
+    if (rowi >= nrows) break;
+    const int isk = (int)(rowi & 1);
+    const int64_t th = rowi >> 1;
+    const int t = (int)(th / A.Hg), h = (int)(th - (int64_t)t * A.Hg);
+    const uint32_t pair = *(const uint32_t*)(A.conv_out + (int64_t)t * 3 * KEYDIM + (isk ? KEYDIM : 0) + h * GP_D + 2 * lane);
+    const float x0 = __uint_as_float(pair << 16), x1 = __uint_as_float(pair & 0xffff0000u);
+    const double tot = wave_sum_f64((double)(x0 * x0) + (double)(x1 * x1));
+    const float rs = rsqrt_f64(tot + 1e-6);
+    const float f = isk ? rs : rs * 0.08838834764831845f;     // 1/sqrt(128) on q
+    *(float2*)(A.qk + rowi * GP_D + 2 * lane) = make_float2(x0 * f, x1 * f);
   }
 }
 
@@ -208,18 +221,24 @@ __global__ __launch_bounds__(256) void gdn_prefill_scan_kernel(GdnPrefillArgs A)
   for (int r = 0; r < GP_ROWS; r++) So[(int64_t)r * GP_D] = st.S[r];
 }
 
-__global__ __launch_bounds__(128) void gdn_prefill_outnorm_kernel(GdnPrefillArgs A) {
-  __shared__ double red[2];
-  const int h = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
-  const int64_t th = (int64_t)t * A.Hg + h;
-  const float o = A.o_raw[th * GP_D + tid];
-  const float zin = bf16_to_f32(A.z[th * GP_D + tid]);
-  const double oss = wave_sum_f64((double)o * (double)o);
-  if ((tid & 63) == 0) red[tid >> 6] = oss;
-  __syncthreads();
-  const float orstd = rsqrt_f64((red[0] + red[1]) / (double)GP_D + 1e-6);
-  const float zs = zin * sigmoid_f64(zin);
-  A.out[th * GP_D + tid] = f32_to_bf16(((o * orstd) * A.norm_w[tid]) * zs);
+// One wave per (token, head): the 128 outputs two per lane, 16 rows per workgroup.  (The sum of squares is taken in
+// double; its last bit may depend on the order of the additions, which the rounding of its inverse root to f32 absorbs.)
+__global__ __launch_bounds__(256) void gdn_prefill_outnorm_kernel(GdnPrefillArgs A) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t nrows = (int64_t)A.T * A.Hg;
+  for (int it = 0; it < GP_PREP_ROWS / 4; it++) {
+    const int64_t th = (int64_t)blockIdx.x * GP_PREP_ROWS + 4 * it + wave;
+    if (th >= nrows) break;
+    const float2 o = *(const float2*)(A.o_raw + th * GP_D + 2 * lane);
+    const uint32_t zp = *(const uint32_t*)(A.z + th * GP_D + 2 * lane);
+    const float2 nw = *(const float2*)(A.norm_w + 2 * lane);
+    const float z0 = __uint_as_float(zp << 16), z1 = __uint_as_float(zp & 0xffff0000u);
+    const double oss = wave_sum_f64((double)o.x * (double)o.x + (double)o.y * (double)o.y);
+    const float orstd = rsqrt_f64(oss / (double)GP_D + 1e-6);
+    const float zs0 = z0 * sigmoid_f64(z0), zs1 = z1 * sigmoid_f64(z1);
+    const uint32_t r0 = f32_to_bf16(((o.x * orstd) * nw.x) * zs0), r1 = f32_to_bf16(((o.y * orstd) * nw.y) * zs1);
+    *(uint32_t*)(A.out + th * GP_D + 2 * lane) = r0 | (r1 << 16);
+  }
 }
 
 static size_t gdn_prefill_base_bytes(int Hg, int T) { return (((size_t)T * Hg * (2 * GP_D + GP_D + 2) * sizeof(float)) + 255) & ~(size_t)255; }
@@ -243,7 +262,7 @@ int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, 
   A.o_raw = A.qk + (size_t)T * Hg * 2 * GP_D;
   A.gates = A.o_raw + (size_t)T * Hg * GP_D;
   A.Hg = Hg; A.T = T;
-  hipLaunchKernelGGL(gdn_prefill_prep_kernel, dim3(Hg, T), dim3(256), 0, stream(), A);
+  hipLaunchKernelGGL(gdn_prefill_prep_kernel, dim3((unsigned)(((int64_t)T * Hg * 2 + GP_PREP_ROWS - 1) / GP_PREP_ROWS)), dim3(256), 0, stream(), A);
   if (chunked) {
     // the chunked form of the recurrence (gdn_chunk.hip) between the same preparation and output norm
     const size_t base = gdn_prefill_base_bytes(Hg, T);
@@ -253,7 +272,7 @@ int launch_gdn_prefill(const void* conv_out, const void* z, const float* A_log, 
   } else {
     hipLaunchKernelGGL(gdn_prefill_scan_kernel, dim3(Hg, GP_SLABS), dim3(256), 0, stream(), A);
   }
-  hipLaunchKernelGGL(gdn_prefill_outnorm_kernel, dim3(Hg, T), dim3(128), 0, stream(), A);
+  hipLaunchKernelGGL(gdn_prefill_outnorm_kernel, dim3((unsigned)(((int64_t)T * Hg + GP_PREP_ROWS - 1) / GP_PREP_ROWS)), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
