@@ -17,16 +17,20 @@ CSRC = os.path.join(ROOT, "bunker_amd", "csrc")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
-@pytest.fixture(scope="module")
-def exact_asm(tmp_path_factory):
+def _compile_to_asm(tmp_path_factory, source):
     if not (os.path.exists(HIPCC) or shutil.which(HIPCC)):
         pytest.skip("hipcc not found")
-    out = str(tmp_path_factory.mktemp("isa") / "attn_exact.s")
+    out = str(tmp_path_factory.mktemp("isa") / (source + ".s"))
     flags = re.search(r"^HIPFLAGS \?= (.*?)(?<!\\)$", open(os.path.join(CSRC, "Makefile")).read(), flags=re.M | re.S).group(1)
     flags = flags.replace("\\\n", " ").replace("$(ARCH)", "gfx950").split()
-    subprocess.check_call([HIPCC, *flags, "-S", "--cuda-device-only", "-o", out, os.path.join(CSRC, "attn_exact.hip")],
+    subprocess.check_call([HIPCC, *flags, "-S", "--cuda-device-only", "-o", out, os.path.join(CSRC, source)],
                           stderr=subprocess.DEVNULL)
     return open(out).read()
+
+
+@pytest.fixture(scope="module")
+def exact_asm(tmp_path_factory):
+    return _compile_to_asm(tmp_path_factory, "attn_exact.hip")
 
 
 def _kernels(asm):
@@ -60,3 +64,31 @@ def test_dpp_groups_in_the_exact_attention_are_hazard_free(exact_asm):
         meta = re.search(r"\.name:\s+%s\n(.*?)\.wavefront_size" % re.escape(name), exact_asm, flags=re.S).group(1)
         assert int(re.search(r"\.vgpr_count:\s+(\d+)", meta).group(1)) <= 128
         assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0
+
+
+@pytest.mark.parametrize("source,kernels,transfer,mfma,min_mfma", [
+    ("attn_prefill.hip", ["attn_prefill_kernel"], "global_load_lds_dwordx4", "v_mfma_f32_32x32x16_bf16", 64),
+    ("gdn_chunk.hip", ["gdn_chunk_wu_kernel", "gdn_chunk_state_kernel", "gdn_chunk_out_kernel"], "global_load_lds_dword", "v_mfma_f32_32x32x2_f32", 32),
+])
+def test_lds_transfers_written_as_instructions_own_m0(tmp_path_factory, source, kernels, transfer, mfma, min_mfma):
+    """lds_dma16 / lds_dma4 (common.h) set m0 themselves and tell the compiler so, but m0 is a register the compiler
+    reserves: the kernels that use them must contain no other use of it, every write of m0 must be followed (one idle
+    cycle later) by the transfer that reads it, and the compiler's own form of the transfer — behind which it waits for
+    the whole transfer before the next LDS access — must not have come back.  Also: no spills, no scratch, and the
+    matrix instruction the kernel is built around is there."""
+    asm = _compile_to_asm(tmp_path_factory, source)
+    bodies = _kernels(asm)
+    for kname in kernels:
+        name, body = next((k, v) for k, v in bodies.items() if kname in k)
+        lines = [l.strip() for l in body.split("\n") if l.strip() and not l.strip().startswith((";", "."))]
+        m0 = [i for i, l in enumerate(lines) if re.search(r"\bm0\b", l)]
+        assert m0, name
+        for i in m0:
+            assert lines[i].startswith("s_mov_b32 m0,"), (name, lines[i])
+            assert lines[i + 1].startswith("s_nop") and lines[i + 2].startswith(transfer + " "), (name, lines[i:i + 3])
+        assert sum(l.startswith(transfer + " ") for l in lines) == len(m0), name
+        assert sum(l.startswith(mfma + " ") for l in lines) >= min_mfma, name
+        meta = re.search(r"\.name:\s+%s\n(.*?)\.wavefront_size" % re.escape(name), asm, flags=re.S).group(1)
+        assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, name
+        assert int(re.search(r"\.sgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, name
+        assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", meta).group(1)) == 0, name
