@@ -268,6 +268,14 @@ __device__ __forceinline__ void lds_dma16(const void* src, const void* lds_piece
 __device__ __forceinline__ void lds_dma4(const void* src, const void* lds_piece) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
 }
+// An LDS address the compiler has to take as it comes: computed from this value, the addresses of a run of transfers
+// are one scalar addition each at the point of use; computed from the array's name they are loop invariants, all of them
+// kept in scalar registers across the loop (and spilled: a run has dozens).
+__device__ __forceinline__ const unsigned char* lds_opaque(const void* p) {
+  uint32_t a = (uint32_t)(uintptr_t)p;
+  asm volatile("" : "+s"(a));
+  return (const unsigned char*)(uintptr_t)a;
+}
 #pragma clang diagnostic pop
 
 }  // namespace bk

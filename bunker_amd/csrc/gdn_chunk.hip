@@ -76,10 +76,16 @@ __device__ __forceinline__ f32x16_t mfma_run(f32x16_t acc, FA fa, FB fb) {
 // fills float l of a half row (lds_dma4), the waves of the workgroup take the half rows in turn.  Nothing
 // waits here; the caller waits for its own requests (vmcnt) and then for the other waves' (barrier).
 __device__ __forceinline__ void rows_to_lds(const float* src, int64_t stride, int row_last, float (*dst)[GC_LD], int wave, int lane) {
+  const unsigned char* base = lds_opaque(dst);
+  const float* lane_src = src + lane;
 #pragma unroll
   for (int i = 0; i < GC_C * 2 / 4; i++) {
-    const int piece = 4 * i + wave, r = piece >> 1, hh = piece & 1;
-    lds_dma4(src + (int64_t)min(r, row_last) * stride + 64 * hh + lane, &dst[r][64 * hh]);
+    const int piece = 4 * i + wave, hh = piece & 1;
+    // (the row number passes through an empty statement: its address arithmetic — scalar, 64-bit — is then done
+    // here, between two transfers, instead of for all 32 pieces ahead of the first, which runs out of scalar registers)
+    int r = piece >> 1;
+    asm volatile("" : "+s"(r));
+    lds_dma4(lane_src + (int64_t)min(r, row_last) * stride + 64 * hh, base + ((piece >> 1) * GC_LD + 64 * hh) * 4);
   }
 }
 __device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }      // vmcnt(0)
