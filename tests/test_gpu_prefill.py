@@ -224,6 +224,42 @@ def test_fa2_prefill_tiled_attention_against_the_checker(orc, NH, NKV, T, pos0):
         rt.cuFree(p)
 
 
+def test_fa2_prefill_tiled_attention_rows_in_any_order_and_a_long_context(orc):
+    """The tiled kernel takes each row's length from pos[t] alone: rows whose positions are shuffled (every token is
+    appended before any row attends, so row t sees all tokens at positions <= pos[t]) and a chunk far into a long
+    cache (8000 tokens in front of it: 126 K/V tiles per workgroup) agree with the checker row by row."""
+    print("fa2_prefill tiled shuffled / long", flush=True)
+    g = synth.rng(8877)
+    NH, NKV, HD, HALF = 16, 2, 256, 32
+    for MAXL, T, pos0, shuffled in ((256, 90, 20, True), (8192, 48, 8000, False)):
+        pages = MAXL // 16
+        cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+        kc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+        vc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+        table = g.permutation(pages).astype(np.int32)
+        qgate = bf(g.standard_normal((T, NH, 2, HD)).astype(np.float32))
+        k = bf(g.standard_normal((T, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((T, NKV, HD)).astype(np.float32))
+        qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+        pos = (pos0 + (g.permutation(T) if shuffled else np.arange(T))).astype(np.int32)
+        ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
+        dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
+        dout = rt.cuAlloc(T * NH * HD * 2)
+        _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} exact=0", ptrs + [dkc, dvc, dout])
+        out = rt.from_device(dout, (T, NH, HD), np.uint16)
+        for t in range(T):                              # all appends first, as the op does
+            kn = orc.rope(orc.headnorm(k[t].ravel(), kw, NKV, HD, HD), cos_t, sin_t, pos[t], NKV, HD, HALF)
+            orc.kv_append(kn.reshape(NKV, HD), v[t], kc, vc, table, pos[t], NKV, HD, 16)
+        worst = 0.0
+        for t in range(T):
+            qn = orc.rope(orc.headnorm(qgate[t].ravel(), qw, NH, HD, 2 * HD), cos_t, sin_t, pos[t], NH, HD, HALF).reshape(1, NH, HD)
+            ro, _ = orc.attn_decode_paged(qn, kc, vc, table[None], np.array([pos[t] + 1], np.int32), 1, NH, NKV, HD, 16,
+                                          gate=qgate[t].ravel()[HD:], gate_bstride=0, gate_hstride=2 * HD)
+            worst = max(worst, float(np.abs(f32(out[t]).astype(np.float64) - f32(ro[0])).max()))
+        assert worst <= 2e-2, (MAXL, worst)
+        for p in ptrs + [dkc, dvc, dout]:
+            rt.cuFree(p)
+
+
 @pytest.mark.parametrize("n_prompt,chunk", [(23, 8), (9, 16)])
 def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
     """TINY model, two sequences in the cache; the prompt goes to sequence 1 in chunks (with a shorter last chunk),
