@@ -89,14 +89,6 @@ __device__ __forceinline__ void rows_to_lds(const float* src, int64_t stride, in
   }
 }
 __device__ __forceinline__ void wait_own_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }      // vmcnt(0)
-// A workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global store of the wave
-// (its fence covers all memory), which the state kernel would pay three times per chunk for stores nobody here reads.
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 // ---- kernel 1, per (head, chunk): g, T = (I + N)^-1, W, Uv
 __global__ __launch_bounds__(256) void gdn_chunk_wu_kernel(GdnChunkArgs A) {
   __shared__ float Ks[GC_C][GC_LD], Vs[GC_C][GC_LD];
@@ -225,7 +217,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
   wait_own_loads();
   for (int c = 0; c < A.nC; c++) {
     const int64_t hc = (int64_t)h * A.nC + c;
-    lds_barrier();                                   // W, k^ and g of this chunk are in LDS; the previous chunk's readers are done
+    __syncthreads();                                   // W, k^ and g of this chunk are in LDS; the previous chunk's readers are done
     // requests of this step, oldest first: k^ of the next chunk, its g, this chunk's Uv (used after the first product)
     const bool more = c + 1 < A.nC;
     if (more) rows_to_lds(k_rows(c + 1), kstride, last_row(c + 1), Kc[(c + 1) & 1], wave, lane);
@@ -248,7 +240,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
 #pragma unroll
       for (int r = 0; r < 16; r++) red[wave][32 * tt + mrow(r, half)][col] = P[r];
     }
-    lds_barrier();
+    __syncthreads();
     if (more) rows_to_lds(A.W + (hc + 1) * GC_C * GC_D, GC_D, GC_C - 1, Wc, wave, lane);
     const float* gc = g_s[c & 1];
     const float gC = gc[GC_C - 1];
@@ -260,7 +252,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_state_kernel(GdnChunkArgs A) {
       A.U[(hc * GC_C + t) * GC_D + 32 * sl + n] = u;
     }
     if (tid < GC_C) g_s[(c + 1) & 1][tid] = gnext;
-    lds_barrier();
+    __syncthreads();
     const float dC = expf(gC);
 #pragma unroll
     for (int r = 0; r < 16; r++) S[r] *= dC;
