@@ -27,6 +27,7 @@ import argparse
 import json
 import os
 import sys
+import tempfile
 import time
 
 import numpy as np
@@ -354,6 +355,47 @@ def bench_load(rt, synth):
     return out
 
 
+def bench_tokenizer():
+    """gt_encode / gt_encode_mt (host C++, no GPU work) on this repository's own documents, with a vocabulary trained on
+    them by the Hugging Face `tokenizers` library (whose encoder is timed beside ours); skipped where that library is absent."""
+    try:
+        from tokenizers import Regex, Tokenizer, models, pre_tokenizers, trainers
+    except ImportError:
+        return {"skipped": "the `tokenizers` package is not importable"}
+    from bunker_amd import tokenizer
+    root = os.path.dirname(os.path.abspath(__file__))
+    text = "".join(open(os.path.join(root, f), encoding="utf-8").read() for f in ("bench.py", "bunker_amd/runner.py", "bunker_amd/loader.py"))
+    qwen = r"(?i:'s|'t|'re|'ve|'m|'ll|'d)|[^\r\n\p{L}\p{N}]?\p{L}+|\p{N}| ?[^\s\p{L}\p{N}]+[\r\n]*|\s*[\r\n]+|\s+(?!\S)|\s+"
+    tok = Tokenizer(models.BPE())
+    tok.pre_tokenizer = pre_tokenizers.Sequence([pre_tokenizers.Split(Regex(qwen), behavior="isolated", invert=False),
+                                                 pre_tokenizers.ByteLevel(add_prefix_space=False, use_regex=False)])
+    tr = trainers.BpeTrainer(vocab_size=3000, special_tokens=["<|endoftext|>"], initial_alphabet=pre_tokenizers.ByteLevel.alphabet(),
+                             show_progress=False)
+    tok.train_from_iterator([text[i:i + 1500] for i in range(0, len(text), 1500)], tr)
+    tmp = tempfile.mkdtemp(prefix="bk_tok_")
+    path = os.path.join(tmp, "tokenizer.json")
+    tok.save(path)
+    t = tokenizer.Tokenizer(path)
+    big = text * 16
+    nbytes = len(big.encode("utf-8"))
+    res = {"bytes": nbytes, "threads_mt": os.cpu_count()}
+    ref_ids = None
+    for name, fn in (("gt_encode", lambda: t.encode(big)), ("gt_encode_mt", lambda: t.encode(big, mt=True)),
+                     ("hugging_face_tokenizers", lambda: np.asarray(tok.encode(big).ids))):
+        fn()
+        t0 = time.perf_counter()
+        ids = fn()
+        dt = time.perf_counter() - t0
+        res[name] = {"MB_per_s": round(nbytes / dt / 1e6, 1), "ids": int(len(ids))}
+        if name == "gt_encode":
+            ref_ids = ids
+        elif name == "hugging_face_tokenizers":
+            res["gt_encode"]["equal_to_hugging_face"] = bool(len(ids) == len(ref_ids) and np.array_equal(np.asarray(ids), np.asarray(ref_ids)))
+    t.close()
+    os.remove(path); os.rmdir(tmp)
+    return res
+
+
 def _time_launches(rt, enqueue, use_graph):
     """Microseconds for everything `enqueue` launches, by HIP events on the library's stream."""
     e0, e1 = rt.Event(), rt.Event()
@@ -538,8 +580,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sections", default="gemv,decode,kernels,gemm",
-                    help="comma list of gemv (headline, always on), decode (with prefill), kernels, gemm, calib, load (weights path)")
+    ap.add_argument("--sections", default="gemv,decode,kernels,gemm,load,tok",
+                    help="comma list of gemv (headline, always on), decode (with prefill), kernels, gemm, calib, load (weights path), "
+                         "tok (tokenizer, host only)")
     ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
                     help="GEMV section. graph: the K launches of a shape replayed from one HIP graph (the device's own launch "
                          "rate); stream: K individual launches per shape queued from the host (used under rocprofv3)")
@@ -717,6 +760,8 @@ def main():
         out["gemm_bs32"] = bench_gemm(rt, synth, use_graph=not args.no_graph)
     if "load" in sections:
         out["weights_path"] = bench_load(rt, synth)
+    if "tok" in sections:
+        out["tokenizer"] = bench_tokenizer()
     if not args.no_cpu_baseline:
         out["cpu_baseline"], parity = cpu_baseline(decode_inputs)
         for key, rep in (parity or {}).items():
