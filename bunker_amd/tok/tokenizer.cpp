@@ -235,6 +235,7 @@ struct Tokenizer {
   std::unordered_map<std::string, uint32_t> vocab;
   std::unordered_map<uint64_t, std::pair<uint32_t, uint32_t>, PairHash> merges;     // (left id, right id) -> (rank, merged id)
   std::vector<std::pair<std::string, uint32_t>> added;                              // content, id
+  bool added_first[256] = {};     // some added token begins with this byte
   uint32_t byte_id[256];          // id of the one-character token of every byte
   std::string byte_char[256];     // the printable character (UTF-8) a byte maps to
   bool ignore_merges = false;
@@ -284,7 +285,7 @@ struct Tokenizer {
     if (const JValue* at = root.get("added_tokens"))
       for (const JValue& t : at->arr) {
         const JValue *c = t.get("content"), *id = t.get("id");
-        if (c && id && !c->str.empty()) added.emplace_back(c->str, (uint32_t)id->num);
+        if (c && id && !c->str.empty()) { added.emplace_back(c->str, (uint32_t)id->num); added_first[(uint8_t)c->str[0]] = true; }
       }
     // the split pattern decides how many digits form one piece
     if (const JValue* pt = root.get("pre_tokenizer")) {
@@ -325,21 +326,52 @@ struct Tokenizer {
     out.insert(out.end(), sym.begin(), sym.end());
   }
 
-  void encode_plain(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
+  // Pieces repeat (words, indentation, punctuation runs): the ids of a piece of up to 24 bytes are kept for the rest of
+  // the call.  The table belongs to the call, not to the tokenizer, so calls on several threads share nothing.
+  struct PieceCache {
+    struct Entry { uint8_t len = 0xFF, nids = 0; uint8_t bytes[24]; uint32_t ids[8]; };
+    std::vector<Entry> slots = std::vector<Entry>(1 << 14);
+    static size_t hash(const uint8_t* s, size_t n) {
+      uint64_t h = 0xcbf29ce484222325ull ^ n;
+      for (size_t i = 0; i < n; i++) h = (h ^ s[i]) * 0x100000001b3ull;
+      return (size_t)(h ^ (h >> 29));
+    }
+  };
+
+  void encode_plain(const uint8_t* s, size_t n, std::vector<uint32_t>& out, PieceCache& cache) const {
     std::vector<Cp> cps;
     decode_utf8(s, n, 0, cps);
     size_t i = 0;
     while (i < cps.size()) {
       const size_t len = scan.next(cps, i);
       const size_t b0 = cps[i].off, b1 = i + len < cps.size() ? cps[i + len].off : n;
-      bpe(s + b0, b1 - b0, out);
+      const size_t pn = b1 - b0;
+      if (pn <= 24) {
+        PieceCache::Entry& e = cache.slots[PieceCache::hash(s + b0, pn) & (cache.slots.size() - 1)];
+        if (e.len == pn && !memcmp(e.bytes, s + b0, pn)) {
+          out.insert(out.end(), e.ids, e.ids + e.nids);
+        } else {
+          const size_t before = out.size();
+          bpe(s + b0, pn, out);
+          const size_t got = out.size() - before;
+          if (got <= 8) {
+            e.len = (uint8_t)pn; e.nids = (uint8_t)got;
+            memcpy(e.bytes, s + b0, pn);
+            memcpy(e.ids, out.data() + before, got * sizeof(uint32_t));
+          }
+        }
+      } else {
+        bpe(s + b0, pn, out);
+      }
       i += len;
     }
   }
 
   void encode(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
+    PieceCache cache;
     size_t start = 0, i = 0;
     while (i < n && !added.empty()) {
+      if (!added_first[s[i]]) { i++; continue; }       // no added token begins with this byte
       // leftmost-longest added token at i
       size_t best_len = 0; uint32_t best_id = 0;
       for (const auto& a : added)
@@ -347,7 +379,7 @@ struct Tokenizer {
           best_len = a.first.size(); best_id = a.second;
         }
       if (best_len) {
-        encode_plain(s + start, i - start, out);
+        encode_plain(s + start, i - start, out, cache);
         out.push_back(best_id);
         i += best_len;
         start = i;
@@ -355,7 +387,7 @@ struct Tokenizer {
         i++;
       }
     }
-    encode_plain(s + start, n - start, out);
+    encode_plain(s + start, n - start, out, cache);
   }
 };
 

@@ -68,6 +68,24 @@ def test_encode_equals_hugging_face(tmp_path, pattern, ignore_merges):
     assert tokenizer.tokenize("Hello", path).tolist() == hf.encode("Hello").ids
 
 
+def test_repeated_pieces_and_the_bounds_of_the_piece_table(tmp_path):
+    """encode keeps the ids of pieces of up to 24 bytes and 8 ids for the rest of the call: pieces at and past both
+    bounds, seen twice in one call and between other pieces that land in the same table, give the Hugging Face ids."""
+    path = str(tmp_path / "tokenizer.json")
+    hf = _train(path, QWEN)
+    t = tokenizer.Tokenizer(path)
+    rng = np.random.default_rng(11)
+    words = []
+    for n in (1, 7, 8, 9, 23, 24, 25, 40):
+        words.append("".join("qzxjkvw"[int(i)] for i in rng.integers(0, 7, n)))            # rare letters: about one id a byte
+        words.append(("tokenizer" * 5)[:n])                                                 # common letters: few ids
+    words += ["日本語한국어日本", "😀🙂😀🙂😀🙂"]                                            # 24 bytes of 3- and 4-byte characters
+    filler = [f"w{i}" for i in range(40000)]                                                 # more pieces than the table has slots
+    text = " ".join(words) + " " + " ".join(filler) + " " + " ".join(reversed(words)) + SPECIAL[0] + " ".join(words)
+    assert t.encode(text).tolist() == hf.encode(text).ids
+    t.close()
+
+
 def test_abi_errors_and_truncation(tmp_path):
     import ctypes as C
     lib = tokenizer.load_library()
