@@ -147,40 +147,61 @@ bool is_space(uint32_t cp) {       // the White_Space property (what \s means in
   return (cp >= 0x09 && cp <= 0x0D) || cp == 0x20 || cp == 0x85 || cp == 0xA0 || cp == 0x1680 || (cp >= 0x2000 && cp <= 0x200A) ||
          cp == 0x2028 || cp == 0x2029 || cp == 0x202F || cp == 0x205F || cp == 0x3000;
 }
-bool is_newline(uint32_t cp) { return cp == '\r' || cp == '\n'; }
 
-struct Cp { uint32_t cp; uint32_t off; };     // code point and its byte offset
-
-// UTF-8 -> code points; a malformed byte becomes one code point 0xFFFD that still covers that byte
-void decode_utf8(const uint8_t* s, size_t n, size_t base, std::vector<Cp>& out) {
-  size_t i = 0;
-  while (i < n) {
-    const uint8_t c = s[i];
-    uint32_t cp = 0xFFFD; size_t len = 1;
-    if (c < 0x80) cp = c;
-    else if ((c & 0xE0) == 0xC0 && i + 1 < n && (s[i + 1] & 0xC0) == 0x80) { cp = ((c & 0x1F) << 6) | (s[i + 1] & 0x3F); len = 2; }
-    else if ((c & 0xF0) == 0xE0 && i + 2 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80) {
-      cp = ((c & 0x0F) << 12) | ((s[i + 1] & 0x3F) << 6) | (s[i + 2] & 0x3F); len = 3;
-    } else if ((c & 0xF8) == 0xF0 && i + 3 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80 && (s[i + 3] & 0xC0) == 0x80) {
-      cp = ((c & 0x07) << 18) | ((s[i + 1] & 0x3F) << 12) | ((s[i + 2] & 0x3F) << 6) | (s[i + 3] & 0x3F); len = 4;
+// Classes of the ASCII range in one table (bit 0 letter, 1 number, 2 space, 3 line break); the rest by range search.
+enum : uint8_t { C_LETTER = 1, C_NUMBER = 2, C_SPACE = 4, C_NEWLINE = 8 };
+struct AsciiClass {
+  uint8_t t[128];
+  constexpr AsciiClass() : t() {
+    for (int c = 0; c < 128; c++) {
+      uint8_t k = 0;
+      if ((c >= 'a' && c <= 'z') || (c >= 'A' && c <= 'Z')) k |= C_LETTER;
+      if (c >= '0' && c <= '9') k |= C_NUMBER;
+      if ((c >= 0x09 && c <= 0x0D) || c == 0x20) k |= C_SPACE;
+      if (c == '\r' || c == '\n') k |= C_NEWLINE;
+      t[c] = k;
     }
-    out.push_back({cp, (uint32_t)(base + i)});
-    i += len;
   }
+};
+constexpr AsciiClass ASCII_CLASS;
+inline uint8_t classes(uint32_t cp) {
+  if (cp < 0x80) return ASCII_CLASS.t[cp];
+  return (is_letter(cp) ? C_LETTER : 0) | (is_number(cp) ? C_NUMBER : 0) | (is_space(cp) ? C_SPACE : 0);
 }
 
 // ------------------------------------------------------------------ the pre-tokenizer's regular expression, by hand
 //   (?i:'s|'t|'re|'ve|'m|'ll|'d) | [^\r\n\p{L}\p{N}]?\p{L}+ | \p{N}{1,D} | ?[^\s\p{L}\p{N}]+[\r\n]* | \s*[\r\n]+ | \s+(?!\S) | \s+
 // Alternatives are tried in this order at every position and the first that matches wins; D = 1 (Qwen) or 3 (cl100k).
+// The scanner walks the UTF-8 bytes themselves: a code point is decoded where it is looked at (one table lookup for
+// ASCII), and a malformed byte counts as one code point U+FFFD that covers that byte.
 struct Scanner {
   int max_digits = 1;
-  // returns the number of code points of the piece that starts at c[i]
-  size_t next(const std::vector<Cp>& c, size_t i) const {
-    const size_t n = c.size();
-    auto at = [&](size_t k) { return k < n ? c[k].cp : 0u; };
-    auto lower = [](uint32_t x) { return x >= 'A' && x <= 'Z' ? x + 32 : x; };
-    if (at(i) == '\'' && i + 1 < n) {
-      const uint32_t a = lower(at(i + 1)), b = i + 2 < n ? lower(at(i + 2)) : 0;
+
+  struct At { uint32_t cp; uint32_t len; uint8_t cls; };      // code point at a byte offset, its length, its classes; len 0 = end
+  __attribute__((always_inline)) static inline At at(const uint8_t* s, size_t n, size_t i) {
+    if (i >= n) return {0, 0, 0};
+    const uint8_t c = s[i];
+    if (c < 0x80) return {c, 1, ASCII_CLASS.t[c]};
+    return at_multibyte(s, n, i);
+  }
+  static At at_multibyte(const uint8_t* s, size_t n, size_t i) {
+    const uint8_t c = s[i];
+    uint32_t cp = 0xFFFD, len = 1;
+    if ((c & 0xE0) == 0xC0 && i + 1 < n && (s[i + 1] & 0xC0) == 0x80) { cp = ((c & 0x1F) << 6) | (s[i + 1] & 0x3F); len = 2; }
+    else if ((c & 0xF0) == 0xE0 && i + 2 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80) {
+      cp = ((c & 0x0F) << 12) | ((s[i + 1] & 0x3F) << 6) | (s[i + 2] & 0x3F); len = 3;
+    } else if ((c & 0xF8) == 0xF0 && i + 3 < n && (s[i + 1] & 0xC0) == 0x80 && (s[i + 2] & 0xC0) == 0x80 && (s[i + 3] & 0xC0) == 0x80) {
+      cp = ((c & 0x07) << 18) | ((s[i + 1] & 0x3F) << 12) | ((s[i + 2] & 0x3F) << 6) | (s[i + 3] & 0x3F); len = 4;
+    }
+    return {cp, len, classes(cp)};
+  }
+
+  // returns the number of bytes of the piece that starts at s[i] (i < n)
+  size_t next(const uint8_t* s, size_t n, size_t i) const {
+    auto lower = [](uint8_t x) -> uint8_t { return x >= 'A' && x <= 'Z' ? x + 32 : x; };
+    const At x = at(s, n, i);
+    if (x.cp == '\'' && i + 1 < n) {
+      const uint8_t a = lower(s[i + 1]), b = i + 2 < n ? lower(s[i + 2]) : 0;     // a byte >= 0x80 matches none of these
       if (a == 's' || a == 't') return 2;
       if ((a == 'r' && b == 'e') || (a == 'v' && b == 'e')) return 3;
       if (a == 'm') return 2;
@@ -189,40 +210,47 @@ struct Scanner {
     }
     {   // [^\r\n\p{L}\p{N}]?\p{L}+
       size_t k = i;
-      const uint32_t x = at(k);
-      if (!is_newline(x) && !is_letter(x) && !is_number(x) && k + 1 < n && is_letter(at(k + 1))) k++;
-      if (k < n && is_letter(at(k))) {
-        while (k < n && is_letter(at(k))) k++;
+      At y = x;
+      if (!(x.cls & (C_NEWLINE | C_LETTER | C_NUMBER))) {
+        const At z = at(s, n, i + x.len);
+        if (z.cls & C_LETTER) { k = i + x.len; y = z; }
+      }
+      if (y.cls & C_LETTER) {
+        do { k += y.len; y = at(s, n, k); } while (y.cls & C_LETTER);
         return k - i;
       }
     }
-    if (is_number(at(i))) {
-      size_t k = i;
-      while (k < n && k - i < (size_t)max_digits && is_number(at(k))) k++;
+    if (x.cls & C_NUMBER) {
+      size_t k = i; int digits = 0;
+      At y = x;
+      while (digits < max_digits && (y.cls & C_NUMBER)) { k += y.len; digits++; y = at(s, n, k); }
       return k - i;
     }
     {   //  ?[^\s\p{L}\p{N}]+[\r\n]*
       size_t k = i;
-      if (at(k) == ' ' && k + 1 < n) k++;
-      auto other = [&](uint32_t x) { return !is_space(x) && !is_letter(x) && !is_number(x); };
-      if (k < n && other(at(k))) {
-        while (k < n && other(at(k))) k++;
-        while (k < n && is_newline(at(k))) k++;
+      At y = x;
+      if (x.cp == ' ' && i + 1 < n) { k = i + 1; y = at(s, n, k); }
+      if (y.len && !(y.cls & (C_SPACE | C_LETTER | C_NUMBER))) {
+        do { k += y.len; y = at(s, n, k); } while (y.len && !(y.cls & (C_SPACE | C_LETTER | C_NUMBER)));
+        while (y.cls & C_NEWLINE) { k += y.len; y = at(s, n, k); }
         return k - i;
       }
     }
-    if (is_space(at(i))) {
-      size_t e = i;
-      while (e < n && is_space(at(e))) e++;
-      // \s*[\r\n]+ : up to and including the last line break of the run
-      for (size_t k = e; k > i; k--)
-        if (is_newline(at(k - 1))) return k - i;
-      // \s+(?!\S) : the whole run at the end of the text, else all but its last character
-      if (e == n) return e - i;
-      if (e - i > 1) return e - i - 1;
-      return 1;                                             // \s+
+    if (x.cls & C_SPACE) {
+      size_t e = i, last_start = i, nl_end = 0;         // end of the run, start of its last character, end of its last line break
+      At y = x;
+      while (y.cls & C_SPACE) {
+        last_start = e;
+        e += y.len;
+        if (y.cls & C_NEWLINE) nl_end = e;
+        y = at(s, n, e);
+      }
+      if (nl_end) return nl_end - i;                      // \s*[\r\n]+ : up to and including the last line break of the run
+      if (e == n) return e - i;                           // \s+(?!\S) : the whole run at the end of the text,
+      if (last_start > i) return last_start - i;          //               else all but its last character
+      return x.len;                                       // \s+
     }
-    return 1;     // not reachable for well-formed input: every code point is a letter, number, space or "other"
+    return x.len;     // not reachable for well-formed input: every code point is a letter, number, space or "other"
   }
 };
 
@@ -310,20 +338,34 @@ struct Tokenizer {
       auto it = vocab.find(whole);
       if (it != vocab.end()) { out.push_back(it->second); return; }
     }
-    std::vector<uint32_t> sym(n);
+    // lowest rank first, leftmost on ties, until no neighbouring pair is a merge.  rank[i] / into[i] describe the pair
+    // (sym[i], sym[i + 1]); a merge changes the two pairs beside it only, so the table is looked up once per new pair
+    uint32_t stack_buf[3 * 64];
+    std::vector<uint32_t> heap_buf;
+    uint32_t* sym = stack_buf;
+    if (n > 64) { heap_buf.resize(3 * n); sym = heap_buf.data(); }
+    uint32_t* rank = sym + n;
+    uint32_t* into = rank + n;
+    auto look = [&](size_t i) {
+      auto it = merges.find(((uint64_t)sym[i] << 32) | sym[i + 1]);
+      if (it == merges.end()) { rank[i] = 0xFFFFFFFFu; into[i] = 0; }
+      else { rank[i] = it->second.first; into[i] = it->second.second; }
+    };
     for (size_t i = 0; i < n; i++) sym[i] = byte_id[s[i]];
-    // lowest rank first, leftmost on ties, until no neighbouring pair is a merge
-    while (sym.size() > 1) {
-      uint32_t best = 0xFFFFFFFFu, merged = 0; size_t at = 0;
-      for (size_t i = 0; i + 1 < sym.size(); i++) {
-        auto it = merges.find(((uint64_t)sym[i] << 32) | sym[i + 1]);
-        if (it != merges.end() && it->second.first < best) { best = it->second.first; merged = it->second.second; at = i; }
-      }
+    size_t len = n;
+    for (size_t i = 0; i + 1 < len; i++) look(i);
+    while (len > 1) {
+      uint32_t best = 0xFFFFFFFFu; size_t at = 0;
+      for (size_t i = 0; i + 1 < len; i++)
+        if (rank[i] < best) { best = rank[i]; at = i; }
       if (best == 0xFFFFFFFFu) break;
-      sym[at] = merged;
-      sym.erase(sym.begin() + at + 1);
+      sym[at] = into[at];
+      for (size_t i = at + 1; i + 1 < len; i++) { sym[i] = sym[i + 1]; rank[i] = rank[i + 1]; into[i] = into[i + 1]; }
+      len--;
+      if (at + 1 < len) look(at);
+      if (at > 0) look(at - 1);
     }
-    out.insert(out.end(), sym.begin(), sym.end());
+    out.insert(out.end(), sym, sym + len);
   }
 
   // Pieces repeat (words, indentation, punctuation runs): the ids of a piece of up to 24 bytes are kept for the rest of
@@ -339,31 +381,27 @@ struct Tokenizer {
   };
 
   void encode_plain(const uint8_t* s, size_t n, std::vector<uint32_t>& out, PieceCache& cache) const {
-    std::vector<Cp> cps;
-    decode_utf8(s, n, 0, cps);
     size_t i = 0;
-    while (i < cps.size()) {
-      const size_t len = scan.next(cps, i);
-      const size_t b0 = cps[i].off, b1 = i + len < cps.size() ? cps[i + len].off : n;
-      const size_t pn = b1 - b0;
+    while (i < n) {
+      const size_t pn = scan.next(s, n, i);
       if (pn <= 24) {
-        PieceCache::Entry& e = cache.slots[PieceCache::hash(s + b0, pn) & (cache.slots.size() - 1)];
-        if (e.len == pn && !memcmp(e.bytes, s + b0, pn)) {
+        PieceCache::Entry& e = cache.slots[PieceCache::hash(s + i, pn) & (cache.slots.size() - 1)];
+        if (e.len == pn && !memcmp(e.bytes, s + i, pn)) {
           out.insert(out.end(), e.ids, e.ids + e.nids);
         } else {
           const size_t before = out.size();
-          bpe(s + b0, pn, out);
+          bpe(s + i, pn, out);
           const size_t got = out.size() - before;
           if (got <= 8) {
             e.len = (uint8_t)pn; e.nids = (uint8_t)got;
-            memcpy(e.bytes, s + b0, pn);
+            memcpy(e.bytes, s + i, pn);
             memcpy(e.ids, out.data() + before, got * sizeof(uint32_t));
           }
         }
       } else {
-        bpe(s + b0, pn, out);
+        bpe(s + i, pn, out);
       }
-      i += len;
+      i += pn;
     }
   }
 
