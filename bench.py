@@ -255,7 +255,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
         floor_us = (weight_bytes + state_bytes) / 8e12 * 1e6
         out[f"bs{B}"] = {"tok_per_s": round(B / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
                          "wall_ms_per_step": round(wall * 1e3 / steps, 4), "steps": steps,
-                         "launch": "hip graph replay" if use_graph else "eager", "launches_per_step": len(loop.launches), "partition": "fused" if fused else "node per kernel", "step_bytes": weight_bytes + state_bytes,
+                         "launch": "hip graph replay" if use_graph else "eager", "ops_per_step": len(loop.launches), "kernel_launches_per_step": loop.graph_exec.node_count() if loop.graph_exec is not None else None, "partition": "fused" if fused else "node per kernel", "step_bytes": weight_bytes + state_bytes,
                          "hbm_floor_us": round(floor_us, 1), "frac_of_floor": round(floor_us / (ms * 1e3), 4),
                          "attention": "double precision (fa2 ops exact=1)",
                          "first_tokens": toks[:4, 0].tolist()}

@@ -295,6 +295,7 @@ int bk_event_destroy(uint64_t ev) {
 }
 
 static bool g_capturing = false;
+static std::map<uint64_t, int> g_graph_nodes;     // executable graph -> kernel nodes it holds
 
 int bk_capture_begin(void) {
   BK_NEED_INIT();
@@ -311,11 +312,22 @@ int bk_capture_end(uint64_t* graph) {
   g_capturing = false;
   hipGraph_t g = nullptr;
   BK_HIP(hipStreamEndCapture(g_stream, &g));
+  size_t n_nodes = 0;
+  (void)hipGraphGetNodes(g, nullptr, &n_nodes);
   hipGraphExec_t exec = nullptr;
   hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
   (void)hipGraphDestroy(g);
   if (e != hipSuccess) return set_error(BK_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
   *graph = (uint64_t)(uintptr_t)exec;
+  g_graph_nodes[*graph] = (int)n_nodes;
+  return BK_OK;
+}
+int bk_graph_node_count(uint64_t graph, int* count) {
+  BK_NEED_INIT();
+  BK_REQUIRE(count, "bk_graph_node_count: null out");
+  const auto it = g_graph_nodes.find(graph);
+  if (it == g_graph_nodes.end()) return set_error(BK_ERR_ARG, "bk_graph_node_count: not a graph of bk_capture_end");
+  *count = it->second;
   return BK_OK;
 }
 int bk_graph_launch(uint64_t graph) {
@@ -327,6 +339,7 @@ int bk_graph_launch(uint64_t graph) {
 int bk_graph_destroy(uint64_t graph) {
   BK_NEED_INIT();
   if (graph) BK_HIP(hipGraphExecDestroy((hipGraphExec_t)(uintptr_t)graph));
+  g_graph_nodes.erase(graph);
   return BK_OK;
 }
 

@@ -45,7 +45,7 @@ _SIGS = {
     "bk_event_elapsed_ms": [u64, u64, C.POINTER(C.c_float)], "bk_event_destroy": [u64],
     "bk_prof_enable": [i32], "bk_prof_reset": [], "bk_prof_report": [C.c_char_p, i32],
     "bk_capture_begin": [], "bk_capture_end": [C.POINTER(u64)], "bk_graph_launch": [u64],
-    "bk_graph_destroy": [u64],
+    "bk_graph_destroy": [u64], "bk_graph_node_count": [u64, C.POINTER(C.c_int)],
     "bk_tune_set": [C.c_char_p, i32],
     "bk_kernel_create": [C.c_char_p], "bk_launch": [i32, C.POINTER(u64), i32], "bk_kernel_destroy": [i32],
     "bk_kernel_describe": [i32, C.c_char_p, i32],
@@ -377,6 +377,11 @@ class Graph:
 
     def launch(self):
         _check(cu().bk_graph_launch(self.h), "bk_graph_launch")
+
+    def node_count(self) -> int:
+        n = C.c_int(0)
+        _check(cu().bk_graph_node_count(self.h, C.byref(n)), "bk_graph_node_count")
+        return n.value
 
     def destroy(self):
         if self.h:

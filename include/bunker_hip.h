@@ -84,6 +84,9 @@ BK_API int bk_capture_begin(void);
 BK_API int bk_capture_end(uint64_t* graph);
 BK_API int bk_graph_launch(uint64_t graph);
 BK_API int bk_graph_destroy(uint64_t graph);
+/* Number of kernel launches the graph replays (one op may be several: a batched matmul is a quantizer launch and a
+ * matrix launch).  For reports; the reference counts launches per step by hand (LOG.md:580). */
+BK_API int bk_graph_node_count(uint64_t graph, int* count);
 
 /* Launch-shape knobs for experiments and tests; the defaults (0, or -1 = chosen from the shape) are the tuned values:
  * "gemv_rpi", "gemv_cap", "gemv_impl", "fused_cap" (GEMV rows per wave step, workgroups per CU, kernel variant),

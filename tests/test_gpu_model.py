@@ -191,6 +191,8 @@ def test_free_running_decode_equals_the_checker_over_seeds(orc, seed):
     rtok, rv = ref.decode(starts, pos0, steps)
     print(f"seed {seed}: min margin {np.min(ref.margins):.5f}", flush=True)
     assert np.array_equal(toks, rtok) and np.array_equal(vals.view(np.uint32), rv.view(np.uint32))
+    # the replayed graph holds at least one kernel per op and not many more (an op is one to three launches)
+    assert len(loop.launches) <= loop.graph_exec.node_count() <= 3 * len(loop.launches)
     loop.close(); env.close()
 
 

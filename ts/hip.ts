@@ -49,6 +49,7 @@ const SYMBOLS = {
   bk_capture_end:           { args: ["ptr"], returns: "i32" },
   bk_graph_launch:          { args: ["u64"], returns: "i32" },
   bk_graph_destroy:         { args: ["u64"], returns: "i32" },
+  bk_graph_node_count:      { args: ["u64", "ptr"], returns: "i32" },
   bk_tune_set:              { args: ["ptr", "i32"], returns: "i32" },
   bk_kernel_create:         { args: ["ptr"], returns: "i32" },
   bk_launch:                { args: ["i32", "ptr", "i32"], returns: "i32" },
@@ -194,6 +195,12 @@ export function captureEnd(): bigint {
 }
 export function graphLaunch(graph: bigint): number { return cu().bk_graph_launch(graph); }
 export function graphDestroy(graph: bigint): void { cu().bk_graph_destroy(graph); }
+/** Kernel launches one replay of the graph stands for. */
+export function graphNodeCount(graph: bigint): number {
+  const out = Buffer.alloc(4);
+  check(cu().bk_graph_node_count(graph, out), "bk_graph_node_count");
+  return out.readInt32LE(0);
+}
 
 /** Quantize a bf16 / f32 weight [rows, K] that is already on the device to Q4_K super-blocks (model load). */
 export function quantizeQ4K(w: bigint, isBf16: boolean, rows: number, K: number): bigint {
