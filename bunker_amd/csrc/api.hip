@@ -506,6 +506,7 @@ int bk_tune_set(const char* key, int value) {
   if (!strcmp(key, "gemv_rpi")) BK_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4, "bk_tune_set: gemv_rpi=%d (0, 1, 2 or 4)", value);
   if (!strcmp(key, "gemv_rpi")) bk::g_tune_rpi = value;
   else if (!strcmp(key, "gemv_cap")) bk::g_tune_cap = value;
+  else if (!strcmp(key, "gemv_steps")) { BK_REQUIRE(value >= 0 && value <= 1024, "bk_tune_set: gemv_steps=%d outside 0..1024", value); bk::g_tune_steps = value; }
   else if (!strcmp(key, "gemv_impl")) bk::g_tune_gemv_impl = value;
   else if (!strcmp(key, "gdn_cs")) bk::g_tune_gdn_cs = value;
   else if (!strcmp(key, "fused_cap")) bk::g_tune_fused_cap = value;

@@ -188,12 +188,20 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q4k_q8_1_subdots_kernel(
 int g_tune_gemv_impl = 2;               // 2: rows staged through LDS when K is a multiple of 2048 (else as 0),
                                         // 0: direct loads in the (block, chunk) mapping
 int g_tune_rpi = 0, g_tune_cap = 16;     // tuning hooks (bk_tune_set): rows per wave step (0: from the shape), workgroups per CU
+int g_tune_steps = 0;                    // > 0: the grid that gives every wave this many row steps (the last one may be short)
 
-static int gemv_grid(int N, int rows_per_wg) {
-  int wgs = (N + rows_per_wg - 1) / rows_per_wg;
+// Workgroups for a launch that needs `wgs` of them at one row step per wave.  Up to the cap (16 per CU) that many; a
+// longer matrix gets the grid in which every wave takes exactly two steps (the second one's rows are in flight while
+// the first is folded).  Measured on the 151936 x 2048 matrix, four rows per step: one step per wave 28.9 us, two 27.4,
+// three 28.7, four 29.4, eight 30.6, and 28.0-29.3 with the grid cut at the cap, where some waves take three steps and
+// the rest two.
+int gemv_grid_for(int wgs) {
+  if (g_tune_steps > 0) return (wgs + g_tune_steps - 1) / g_tune_steps;
   const int cap = num_cus() * g_tune_cap;
-  return wgs < cap ? wgs : cap;
+  return wgs <= cap ? wgs : (wgs + 1) / 2;
 }
+
+static int gemv_grid(int N, int rows_per_wg) { return gemv_grid_for((N + rows_per_wg - 1) / rows_per_wg); }
 
 template <int NR, int EPI>
 static void launch_q8_1_rpi(dim3 block, const uint8_t* w, const uint8_t* x, void* y, const uint16_t* r, int N, int nb, int batch) {

@@ -319,9 +319,13 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
   int wgs = (steps + GEMV_WAVES - 1) / GEMV_WAVES;
   // With a prologue every workgroup repeats the RMSNorm / Q8_1 work of the row, so fewer, longer-lived workgroups win:
   // two per CU measured best (three per CU, one step per wave: 4 % slower over the decode step; one per CU: the rows
-  // in flight no longer cover the memory latency).  Without a prologue the plain GEMV's cap applies.
-  const int cap = num_cus() * (g_tune_fused_cap > 0 ? g_tune_fused_cap : (pro != PRO_Q8 ? 2 : g_tune_cap));
-  if (wgs > cap) wgs = cap;
+  // in flight no longer cover the memory latency).  Without a prologue the plain GEMV's rule applies.
+  if (g_tune_fused_cap > 0 || pro != PRO_Q8) {
+    const int cap = num_cus() * (g_tune_fused_cap > 0 ? g_tune_fused_cap : 2);
+    if (wgs > cap) wgs = cap;
+  } else {
+    wgs = gemv_grid_for(wgs);
+  }
   const dim3 grid(wgs, batch);
   if (swiglu && KB == 4) launch_fused_pro<4, 4, true>(pro, grid, A);
   else if (swiglu) launch_fused_pro<8, 4, true>(pro, grid, A);

@@ -38,6 +38,8 @@ int launch_memread(const void* src, int64_t bytes, void* sink);
 int launch_memcopy(const void* src, void* dst, int64_t bytes);
 
 // gemv.hip
+extern int g_tune_steps;
+int gemv_grid_for(int wgs);
 extern int g_tune_rpi, g_tune_cap, g_tune_mr_unroll, g_tune_mr_cap, g_tune_mr_nt, g_tune_gemv_impl;
 int launch_gemv_q4k_f32(const void* W, const float* x, float* y, int N, int K);
 int launch_gemv_q4k_q8_1(const void* W, const void* xq, void* y, int N, int K, int batch,
