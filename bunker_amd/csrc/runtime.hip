@@ -82,6 +82,12 @@ using namespace bk;
 #define BK_NEED_INIT() \
   do { if (!g_inited) return set_error(BK_ERR_STATE, "bk_init has not been called"); } while (0)
 
+// Between bk_capture_begin and bk_capture_end only launches are recorded; anything else would either end the capture with
+// an error of the runtime's or, for a memset, put a node into the graph that replays wrongly on this platform.
+static bool g_capturing = false;
+#define BK_NOT_CAPTURING(name) \
+  do { if (g_capturing) return set_error(BK_ERR_STATE, name ": not legal between bk_capture_begin and bk_capture_end"); } while (0)
+
 extern "C" {
 
 int bk_init(int device) {
@@ -139,6 +145,7 @@ int bk_device_info(char* buf, int cap) {
 
 int bk_alloc(uint64_t bytes, uint64_t* out) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_alloc");
   BK_REQUIRE(out, "bk_alloc: null out");
   void* p = nullptr;
   hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
@@ -148,6 +155,7 @@ int bk_alloc(uint64_t bytes, uint64_t* out) {
 }
 int bk_free(uint64_t ptr) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_free");
   if (!ptr) return BK_OK;
   if (int rc = sync_all()) return rc;
   BK_HIP(hipFree((void*)(uintptr_t)ptr));
@@ -157,6 +165,7 @@ int bk_free(uint64_t ptr) {
 // the call returns when the copy is complete, as cuMemcpyHtoD/DtoH do.
 int bk_htod(uint64_t dst, const void* src, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_htod");
   BK_REQUIRE(dst && src, "bk_htod: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, src, bytes, hipMemcpyHostToDevice, g_stream));
@@ -165,6 +174,7 @@ int bk_htod(uint64_t dst, const void* src, uint64_t bytes) {
 }
 int bk_dtoh(void* dst, uint64_t src, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_dtoh");
   BK_REQUIRE(dst && src, "bk_dtoh: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemcpyAsync(dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToHost, g_stream));
@@ -173,6 +183,7 @@ int bk_dtoh(void* dst, uint64_t src, uint64_t bytes) {
 }
 int bk_dtod(uint64_t dst, uint64_t src, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_dtod");
   BK_REQUIRE(dst && src, "bk_dtod: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToDevice, g_stream));
@@ -196,6 +207,7 @@ int bk_host_free(uint64_t ptr) {
 }
 int bk_htod_async(uint64_t dst, const void* src, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_htod_async");
   BK_REQUIRE(dst && src, "bk_htod_async: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemcpyAsync((void*)(uintptr_t)dst, src, bytes, hipMemcpyHostToDevice, g_stream));
@@ -203,6 +215,7 @@ int bk_htod_async(uint64_t dst, const void* src, uint64_t bytes) {
 }
 int bk_dtoh_async(void* dst, uint64_t src, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_dtoh_async");
   BK_REQUIRE(dst && src, "bk_dtoh_async: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemcpyAsync(dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToHost, g_stream));
@@ -210,12 +223,14 @@ int bk_dtoh_async(void* dst, uint64_t src, uint64_t bytes) {
 }
 int bk_event_sync(uint64_t ev) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_event_sync");
   BK_REQUIRE(ev, "bk_event_sync: null event");
   BK_HIP(hipEventSynchronize((hipEvent_t)(uintptr_t)ev));
   return BK_OK;
 }
 int bk_memset(uint64_t dst, int value, uint64_t bytes) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_memset");
   BK_REQUIRE(dst, "bk_memset: null pointer");
   if (!bytes) return BK_OK;
   BK_HIP(hipMemsetAsync((void*)(uintptr_t)dst, value, bytes, g_stream));
@@ -223,6 +238,7 @@ int bk_memset(uint64_t dst, int value, uint64_t bytes) {
 }
 int bk_sync(void) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_sync");
   return sync_all();
 }
 
@@ -244,6 +260,7 @@ static int find_stream(uint64_t s) {
 }
 int bk_stream_use(uint64_t s) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_stream_use");
   if (!s) { g_stream = g_main_stream; return BK_OK; }
   const int i = find_stream(s);
   BK_REQUIRE(i >= 0, "bk_stream_use: not a stream of bk_stream_create");
@@ -294,7 +311,6 @@ int bk_event_destroy(uint64_t ev) {
   return BK_OK;
 }
 
-static bool g_capturing = false;
 static std::map<uint64_t, int> g_graph_nodes;     // executable graph -> kernel nodes it holds
 
 int bk_capture_begin(void) {
@@ -332,6 +348,7 @@ int bk_graph_node_count(uint64_t graph, int* count) {
 }
 int bk_graph_launch(uint64_t graph) {
   BK_NEED_INIT();
+  BK_NOT_CAPTURING("bk_graph_launch");
   BK_REQUIRE(graph, "bk_graph_launch: null graph");
   BK_HIP(hipGraphLaunch((hipGraphExec_t)(uintptr_t)graph, g_stream));
   return BK_OK;

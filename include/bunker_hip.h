@@ -78,8 +78,10 @@ BK_API int bk_prof_report(char* buf, int cap);       /* profGpuReport, src/ttir.
  * into a HIP graph (stream capture) and replay it with one call.  The reference
  * tried the same with CUDA graphs through bun:ffi and gave up on struct-pointer
  * crashes (LOG.md:710-738); here the graph lives behind scalar handles.
- * Between begin and end only launches are legal: no alloc, free, copy to or from
- * the host, sync or event call. */
+ * Between begin and end only launches are legal: alloc, free, memset, copies,
+ * sync, event waits, a stream switch and a graph launch return an error (state
+ * -3, "not legal between bk_capture_begin and bk_capture_end") and leave the
+ * capture open. */
 BK_API int bk_capture_begin(void);
 BK_API int bk_capture_end(uint64_t* graph);
 BK_API int bk_graph_launch(uint64_t graph);

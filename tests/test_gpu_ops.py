@@ -416,3 +416,28 @@ def test_streams_order_work_through_events(orc, dev):
     with pytest.raises(rt.BunkerError, match="not a stream"):
         rt._check(rt.cu().bk_stream_use(12345), "bk_stream_use")
     st.destroy(); ev.destroy(); done.destroy()
+
+
+def test_only_launches_are_recorded_between_capture_begin_and_end():
+    """Inside a capture every call that is not a launch is refused with the library's own error and leaves the capture
+    open and usable (a memset node would replay wrongly, a copy or a sync would end the capture with a runtime error);
+    the graph then replays the launches recorded around the refused calls."""
+    import ctypes as C
+    lib = rt.cu()
+    x = np.arange(64, dtype=np.float32)
+    dx = rt.to_device(x); dq = rt.cuAlloc(2 * 36); rt.cuMemset(dq, 0, 72)
+    host = np.zeros(72, np.uint8)
+    p = C.c_uint64(0)
+    with rt.Graph() as gr:
+        rt.quantize_q8_1(dx, dq, 64, 1, rt.F32)
+        for rc in (lib.bk_memset(dq, 0, 72), lib.bk_sync(), lib.bk_alloc(256, C.byref(p)), lib.bk_free(dq),
+                   lib.bk_dtoh(host.ctypes.data_as(C.c_void_p), dq, 72), lib.bk_graph_launch(1)):
+            assert rc != 0 and b"not legal between bk_capture_begin and bk_capture_end" in lib.bk_last_error()
+    assert gr.node_count() == 1
+    for _ in range(2):
+        rt.cuMemset(dq, 0, 72)
+        gr.launch(); rt.cuSync()
+        got = rt.from_device(dq, (72,), np.uint8)
+        assert got[:32].view(np.int8).max() == 127 and got[36:68].view(np.int8).max() == 127
+    gr.destroy()
+    rt.cuFree(dx); rt.cuFree(dq)
