@@ -55,15 +55,16 @@ enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 *
 
 // SWIGLU: the workgroup holds 2 NW waves; waves 0..NW-1 form the tile of 32 gate rows, waves NW..2NW-1 the tile of the
 // same 32 up rows, and the last step writes act = bf16(silu(g) * u) and its Q8_1 block instead of g and u.
-// R16: the tile has 16 weight rows (rows 16..31 of the matrix instruction repeat them and are ignored), for launches with
-// so few tiles that the time is the length of one wave's instruction stream: half the fold per super-block, twice the tiles.
-template <int NW, bool SWIGLU, bool R16 = false>
+// TR: weight rows of the tile.  16 or 8 (the other rows of the matrix instruction repeat them and are ignored) for launches
+// with so few tiles that the time is the length of one wave's instruction stream: a half or a quarter of the fold per
+// super-block, two or four times the tiles.
+template <int NW, bool SWIGLU, int TR = 32>
 __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
-  static_assert(!(SWIGLU && R16), "the SwiGLU form quantizes 32 outputs at a time");
+  static_assert(TR == 32 || TR == 16 || TR == 8, "tiles of 32, 16 or 8 weight rows");
+  static_assert(!(SWIGLU && TR != 32), "the SwiGLU form quantizes 32 outputs at a time");
   constexpr int WAVES = NW * (SWIGLU ? 2 : 1);
-  constexpr int TR = R16 ? 16 : 32;        // weight rows of the tile
-  constexpr int RF = TR / 2;               // of them per lane
-  constexpr int TN = TR / 16;              // 16-row groups (min term)
+  constexpr int RF = TR / 2;               // weight rows per lane
+  constexpr int TN = TR >= 16 ? TR / 16 : 1;   // 16-row groups (min term; a tile of 8 fills half of one, the rest repeats it)
   // Per wave: the activation rows of the current super-block as they lie in memory (288 bytes, rows 292 apart so that
   // the lanes of a read fall into different banks), the weight rows (144 bytes each), and 512 bytes of weight scales
   // in the order the fold reads them (the 6-bit scales as bytes [8 sub-blocks][2 halves][16 rows], then d as doubles
@@ -127,8 +128,8 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
     }                                                                                                                  \
     wr0 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[0]);                                                       \
     wr1 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[1]);                                                       \
-    wr2 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[2]);                                                       \
-    if (!R16) {                                                                                                        \
+    if (TR >= 16) wr2 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[2]);                                         \
+    if (TR == 32) {                                                                                                    \
       wr3 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[3]);                                                     \
       wr4 = *(const uint4*)(wbase + (int64_t)fb_ * 144 + woff[4]);                                                     \
     }                                                                                                                  \
@@ -157,10 +158,13 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
       if (i < 8 || k4 < 2) { p[0] = xr[i].x; p[1] = xr[i].y; p[2] = xr[i].z; p[3] = xr[i].w; }
     }
     *(uint4*)(ldsW + lane * 16) = wr0;
-    *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
-    if (R16) {
+    if (TR == 8) {
+      if (lane < 8) *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
+    } else if (TR == 16) {
+      *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
       if (lane < 16) *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
     } else {
+      *(uint4*)(ldsW + (lane + 64) * 16) = wr1;
       *(uint4*)(ldsW + (lane + 128) * 16) = wr2;
       *(uint4*)(ldsW + (lane + 192) * 16) = wr3;
       if (lane < 32) *(uint4*)(ldsW + (lane + 256) * 16) = wr4;
@@ -258,7 +262,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 #pragma unroll
     for (int t = 0; t < 2; t++) {
       if (t < TN) {
-        const uint4 hm = *(const uint4*)(ldsW + (16 * t + l16) * GW_ROW);
+        const uint4 hm = *(const uint4*)(ldsW + ((16 * t + l16) & (TR - 1)) * GW_ROW);
         const float dmin_neg = -half_to_f32((uint16_t)(hm.x >> 16));
         const uint32_t zb = (hm.z >> (8 * q4)) & 0xffu, wb = (hm.w >> (8 * q4)) & 0xffu;
         am[t][0] = (double)(dmin_neg * (float)(zb & 63u));
@@ -303,9 +307,9 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   __syncthreads();
   const double* all = (const double*)lds_raw;
   // the thread's output row fn of the tile and its batch rows fb0 + FB * (wave R + i): 32 rows -> (lane % 32, lane / 32),
-  // 16 rows -> (lane % 16, lane / 16)
+  // 16 rows -> (lane % 16, lane / 16), 8 rows -> (lane % 8, lane / 8)
   constexpr int R = TR / 2 / WAVES > 0 ? TR / 2 / WAVES : 1, FB = 64 / TR;
-  if (wave * R * FB >= 32) return;         // (eight waves on a 16-row tile: R = 1 and all of them have a batch row)
+  if (wave * R * FB >= 32) return;         // (a 16-row tile gives each of eight waves one batch-row pair; an 8-row tile is finished by four waves)
   const int fn = lane & (TR - 1), fb0 = lane / TR;
   const int rr = 4 * (fn >> 3) + (fn & 3), hh = (fn >> 2) & 1;
   float y[SWIGLU ? 1 : R], u_[SWIGLU ? R : 1], g_[SWIGLU ? R : 1];
@@ -370,7 +374,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 #undef GM_FETCH
 
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
-int g_tune_gemm_r16 = -1;    // tiles of 16 weight rows: 0 off, 1 on (single batch tile only), -1 = from the shape
+int g_tune_gemm_r16 = -1;    // narrow tiles (single batch tile only): 0 off, 1 = 16 weight rows, 2 = 8, -1 = from the shape
 
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi) {
@@ -389,12 +393,17 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
     A.tile_first[i] = tiles;
     tiles += (N[i] + 31) / 32;
   }
-  // One batch tile and so few weight tiles that half the CUs would stay empty: tiles of 16 weight rows (twice as many
-  // workgroups, half the fold per wave).  Measured on the 64-tile shapes at batch 32.
-  const bool r16 = batch <= 32 && (g_tune_gemm_r16 >= 0 ? g_tune_gemm_r16 != 0 : (2 * tiles <= num_cus() && A.nb >= 4));
-  if (r16) {
+  // One batch tile and so few weight tiles that CUs would stay empty: tiles of 16 weight rows (twice as many
+  // workgroups, half the fold per wave) when that still leaves half of them empty... of 8 when a quarter.  Measured on the
+  // 64-tile shapes at batch 32.
+  int tr = 32;
+  if (batch <= 32) {
+    if (g_tune_gemm_r16 >= 0) tr = g_tune_gemm_r16 == 0 ? 32 : (g_tune_gemm_r16 == 1 ? 16 : 8);
+    else if (A.nb >= 4) tr = 4 * tiles <= num_cus() ? 8 : (2 * tiles <= num_cus() ? 16 : 32);
+  }
+  if (tr != 32) {
     tiles = 0;
-    for (int i = 0; i < ngroups; i++) { A.tile_first[i] = tiles; tiles += (N[i] + 15) / 16; }
+    for (int i = 0; i < ngroups; i++) { A.tile_first[i] = tiles; tiles += (N[i] + tr - 1) / tr; }
   }
   for (int i = ngroups; i < 5; i++) A.tile_first[i] = tiles;
   // waves per tile (measured on the decode shapes at batch 32): long rows split eight ways, K = 2048 four ways,
@@ -411,9 +420,12 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
   A.tiles = tiles; A.btiles = btiles;
   const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
-  if (r16 && btiles == 1) {
-    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, true>), grid, dim3(512), 0, stream(), A);
-    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, true>), grid, dim3(256), 0, stream(), A);
+  if (tr == 16) {
+    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 16>), grid, dim3(512), 0, stream(), A);
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 16>), grid, dim3(256), 0, stream(), A);
+  } else if (tr == 8) {
+    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 8>), grid, dim3(512), 0, stream(), A);
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 8>), grid, dim3(256), 0, stream(), A);
   } else if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false>), grid, dim3(512), 0, stream(), A);
   else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false>), grid, dim3(256), 0, stream(), A);
   else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, false>), grid, dim3(128), 0, stream(), A);

@@ -307,7 +307,7 @@ def test_gemm_mfma_every_split_of_k_returns_the_same_bits(orc, dev, N, K, B):
     ref = np.stack([orc.gemv_q4k_q8_1(W, xq[b], N, K) for b in range(B)])
     dW, dxq, dy = dev.up(W), dev.up(xq), dev.empty(B * N * 4)
     try:
-        for r16 in (0, 1):                     # tiles of 32 or of 16 weight rows (the latter for a single batch tile only)
+        for r16 in (0, 1, 2):                  # tiles of 32, 16 or 8 weight rows (the narrow ones for a single batch tile only)
             rt.tune_set("gemm_r16", r16)
             for nw in (1, 2, 4, 8):
                 rt.tune_set("gemm_nw", nw)
