@@ -123,7 +123,19 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   if (gemv_fused_fast_path(K, batch, swiglu)) return launch_gemv_fused(pro, x, nw, K, batch, G, W, out, res, N, epi, swiglu);
   int rc;
   const void* xq = x;
-  if (pro == 2) { if ((rc = launch_rmsnorm(x, nw, nullptr, k.scratch, K, batch))) return rc; xq = k.scratch; }
+  // The GDN layers' projections at hidden size 2048: qkv and z are 256 tiles of the batched matmul, one per CU with eight
+  // waves each, and the 16-row a and b would add two (a second, four-wave form: 11.9 us instead of 8.7 at batch 32).
+  // Those two run inside the norm's launch instead, on CUs it leaves idle.
+  int Gm = G;
+  if (pro == 2 && !swiglu && G == 4 && batch >= GEMM_MFMA_MIN_BATCH && batch <= 32 && K == 2048 && epi[2] == 0 && epi[3] == 0 &&
+      N[2] + N[3] <= 64 && g_tune_small_rows != 0) {
+    const int big = (N[0] + 31) / 32 + (N[1] + 31) / 32, all = big + (N[2] + 31) / 32 + (N[3] + 31) / 32;
+    if (big <= num_cus() && all > num_cus()) Gm = 2;
+  }
+  if (pro == 2 && Gm == 2 && G == 4) {
+    if ((rc = launch_rmsnorm_small_rows(x, nw, k.scratch, K, batch, W[2], W[3], (float*)out[2], (float*)out[3], N[2], N[3]))) return rc;
+    xq = k.scratch;
+  } else if (pro == 2) { if ((rc = launch_rmsnorm(x, nw, nullptr, k.scratch, K, batch))) return rc; xq = k.scratch; }
   else if (pro == 1) { if ((rc = launch_quantize_q8_1(x, DT_BF16, k.scratch, K, batch))) return rc; xq = k.scratch; }
   if (swiglu) {
     // batched and with a Q8_1 result: SwiGLU and the quantization are the matmul kernel's last step
@@ -140,7 +152,7 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
     if (q8out) return launch_swiglu_q8_1(g, u, out[0], q8out, (int64_t)batch * N[0]);
     return launch_elementwise(EW_SWIGLU_OP, g, u, out[0], (int64_t)batch * N[0]);
   }
-  if (batch >= GEMM_MFMA_MIN_BATCH) return matmul_group_mfma(xq, K, batch, G, W, out, res, N, epi);
+  if (batch >= GEMM_MFMA_MIN_BATCH) return matmul_group_mfma(xq, K, batch, Gm, W, out, res, N, epi);
   for (int i = 0; i < G; i++)
     if ((rc = matmul_q8_1(W[i], xq, out[i], N[i], K, batch, epi[i] == 0 ? DT_F32 : DT_BF16, res[i], -1))) return rc;
   return BK_OK;
@@ -513,6 +525,7 @@ int bk_tune_set(const char* key, int value) {
   else if (!strcmp(key, "attn_nt")) bk::g_tune_attn_nt = value;
   else if (!strcmp(key, "attn_bal")) bk::g_tune_attn_bal = value;
   else if (!strcmp(key, "gemm_r16")) bk::g_tune_gemm_r16 = value;
+  else if (!strcmp(key, "small_rows")) bk::g_tune_small_rows = value;
   else if (!strcmp(key, "gdn_nt")) bk::g_tune_gdn_nt = value;
   else if (!strcmp(key, "gemm_nw")) bk::g_tune_gemm_nw = value;
   else if (!strcmp(key, "memread_unroll")) bk::g_tune_mr_unroll = value;

@@ -3,6 +3,7 @@
 // leading batch dimension; all math is f32 with bf16 (round-to-nearest-even) I/O,
 // as in src/fusion.ts:295-330 and src/emitters.ts:31-255.
 #include "ops.h"
+#include "gemv_tile.h"
 
 namespace bk {
 
@@ -35,10 +36,24 @@ int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void*
 // which is what the following matmuls consume.
 // ONE: the row has at most 2048 elements: a thread's 8 values and weights stay in registers between the two passes
 // (one memory round trip instead of two).
-template <bool QUANT, bool ONE>
+// ROWS (with QUANT and ONE): the launch also multiplies a few short matrices (the 16-row a and b projections of a
+// Gated-DeltaNet layer) with the row it has just quantized, so that the batched matmul behind it is left with the
+// tiles of the large matrices only.  Workgroup (row, 0) does the norm's own job; workgroups (row, 1 + j) repeat the norm
+// and the quantization on their own CU, keep the Q8_1 row in LDS and take eight of those rows each, two per wave, with
+// the GEMV's row arithmetic (same int32 dots, same f64 fold, one rounding to f32).
+struct SmallRows {
+  const uint8_t* W[2];    // Q4_K matrices [n[i], N]
+  float* out[2];          // f32 [rows, n[i]]
+  int n[2];
+};
+template <bool QUANT, bool ONE, bool ROWS = false>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                      uint16_t* __restrict__ out, uint8_t* __restrict__ xq, int N) {
+                                                      uint16_t* __restrict__ out, uint8_t* __restrict__ xq, int N,
+                                                      SmallRows sr = SmallRows{}) {
+  static_assert(!ROWS || (QUANT && ONE), "the small rows need the quantized row of a single pass");
   __shared__ double lds[4];
+  __shared__ __align__(16) uint8_t xq_l[ROWS ? 2048 / 32 * 36 : 16];
+  const bool own = !ROWS || blockIdx.y == 0;      // this workgroup writes the norm's results
   const int row = blockIdx.x;
   const uint16_t* xr = x + (int64_t)row * N;
   double ss = 0.0;     // squares of bf16 values are exact in f32; their sum is carried in double
@@ -52,6 +67,19 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     for (int j = 0; j < 4; j++) {
       const float a = __uint_as_float(u[j] << 16), b = __uint_as_float(u[j] & 0xffff0000u);
       ss += (double)(a * a) + (double)(b * b);
+    }
+  }
+  // the weight rows of the small matrices do not depend on the norm: requested behind the row itself (loads return in
+  // issue order), they arrive while the sum is reduced and the row scaled and quantized
+  uint4 sr_hdr[2] = {}, sr_q[2] = {};
+  if (ROWS && !own) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nb = N / 256, blk = min(lane >> 3, nb - 1), c = lane & 7;
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      const int r = min(((int)blockIdx.y - 1) * 8 + wave * 2 + k, sr.n[0] + sr.n[1] - 1);      // past the end: the last row again
+      const bool second = r >= sr.n[0];
+      const uint8_t* rp = (second ? sr.W[1] : sr.W[0]) + (int64_t)(second ? r - sr.n[0] : r) * nb * 144 + blk * 144;
+      sr_hdr[k] = load_w16(rp); sr_q[k] = load_w16(rp + 16 + 16 * c);
     }
   }
   ss = block_sum_f64<4>(ss, lds);
@@ -71,17 +99,61 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
       o[j] = (uint32_t)ha | ((uint32_t)hb << 16);
       f[2 * j] = bf16_to_f32(ha); f[2 * j + 1] = bf16_to_f32(hb);
     }
-    if (out) *(uint4*)(out + (int64_t)row * N + i) = make_uint4(o[0], o[1], o[2], o[3]);
+    if (out && own) *(uint4*)(out + (int64_t)row * N + i) = make_uint4(o[0], o[1], o[2], o[3]);
     if (QUANT) {
       // Q8_1 of the bf16-rounded values: block = 4 consecutive lanes x 8 elements
       uint32_t pk[2];
       const uint32_t ds = quad_q8_1(f, pk);
-      uint8_t* ob = xq + ((int64_t)row * (N / 32) + i / 32) * 36;
-      uint32_t* oq = (uint32_t*)(ob + (i & 31));
-      oq[0] = pk[0]; oq[1] = pk[1];
-      if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+      if (own) {
+        uint8_t* ob = xq + ((int64_t)row * (N / 32) + i / 32) * 36;
+        uint32_t* oq = (uint32_t*)(ob + (i & 31));
+        oq[0] = pk[0]; oq[1] = pk[1];
+        if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+      } else if (ROWS) {
+        uint8_t* ob = xq_l + (i / 32) * 36;
+        uint32_t* oq = (uint32_t*)(ob + (i & 31));
+        oq[0] = pk[0]; oq[1] = pk[1];
+        if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+      }
     }
   }
+  if (ROWS) {
+    if (own) return;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = N / 256, blk = lane >> 3, c = lane & 7;
+    const bool active = blk < nb;                       // lanes past the row add exact zeros
+    const ScaleSel sel = make_scale_sel(c);
+    XQ xs;
+    load_xq(xs, xq_l, min(blk, nb - 1), c, active);
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      const int r = ((int)blockIdx.y - 1) * 8 + wave * 2 + k;
+      if (r >= sr.n[0] + sr.n[1]) break;                // wave-uniform
+      const bool second = r >= sr.n[0];
+      const int rr = second ? r - sr.n[0] : r;
+      int I0, I1;
+      const double tot = wave_sum_f64(slot_dot(sr_hdr[k], sr_q[k], xs, sel, I0, I1, (c & 1) != 0));
+      if (lane == 0) (second ? sr.out[1] : sr.out[0])[(int64_t)row * (second ? sr.n[1] : sr.n[0]) + rr] = (float)tot;
+    }
+  }
+}
+
+int g_tune_small_rows = 1;     // 0: the short matrices of a projection group stay in the batched matmul
+
+// rmsnorm -> Q8_1 (into xq) together with the products of two short matrices with the quantized rows (see SmallRows)
+int launch_rmsnorm_small_rows(const void* x, const void* w, void* xq, int N, int rows, const void* Wa, const void* Wb, float* out_a,
+                              float* out_b, int na, int nb_rows) {
+  BK_REQUIRE(x && w && xq && Wa && Wb && out_a && out_b, "rmsnorm_small_rows: null pointer");
+  BK_REQUIRE(N > 0 && N % 256 == 0 && N <= 2048 && rows > 0 && rows <= 65535, "rmsnorm_small_rows: N=%d must be a multiple of 256 up to 2048 (rows=%d)", N, rows);
+  BK_REQUIRE(na > 0 && nb_rows > 0 && na + nb_rows <= 64, "rmsnorm_small_rows: %d + %d rows (at most 64 together)", na, nb_rows);
+  BK_REQUIRE(((uintptr_t)Wa & 15) == 0 && ((uintptr_t)Wb & 15) == 0, "rmsnorm_small_rows: misaligned matrix");
+  SmallRows sr;
+  sr.W[0] = (const uint8_t*)Wa; sr.W[1] = (const uint8_t*)Wb; sr.out[0] = out_a; sr.out[1] = out_b; sr.n[0] = na; sr.n[1] = nb_rows;
+  hipLaunchKernelGGL((rmsnorm_kernel<true, true, true>), dim3(rows, 1 + (na + nb_rows + 7) / 8), dim3(256), 0, stream(),
+                     (const uint16_t*)x, (const uint16_t*)w, (uint16_t*)nullptr, (uint8_t*)xq, N, sr);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
 }
 
 int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows) {

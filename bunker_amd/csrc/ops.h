@@ -53,6 +53,7 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
                       void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
 
 // gemm_mfma.hip
+extern int g_tune_small_rows;
 extern int g_tune_gemm_nw, g_tune_gemm_r16, g_tune_gdn_nt, g_tune_attn_nt, g_tune_attn_bal;
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi);
@@ -64,6 +65,8 @@ int launch_gemm_q4k_q8_1_mfma(const void* W, const void* xq, void* y, int N, int
 enum : int { EW_CAST_OP = 0, EW_ADD_OP = 1, EW_SWIGLU_OP = 2 };
 int launch_embed(const void* E, const int32_t* ids_dev, int32_t id_scalar, void* out, int H, int vocab, int batch);
 int launch_rmsnorm(const void* x, const void* w, void* out, void* xq, int N, int rows);
+int launch_rmsnorm_small_rows(const void* x, const void* w, void* xq, int N, int rows, const void* Wa, const void* Wb, float* out_a,
+                              float* out_b, int na, int nb_rows);
 int launch_elementwise(int op, const void* a, const void* b, void* out, int64_t n);
 int launch_swiglu_q8_1(const float* g, const float* u, void* out, void* out_q8, int64_t n);
 int launch_conv1d_decode(const void* x, const void* st, const void* w, void* out, void* st_new, int C, int batch);

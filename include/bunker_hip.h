@@ -93,7 +93,8 @@ BK_API int bk_graph_node_count(uint64_t graph, int* count);
 /* Launch-shape knobs for experiments and tests; the defaults (0, or -1 = chosen from the shape) are the tuned values:
  * "gemv_rpi", "gemv_cap", "gemv_steps", "gemv_impl", "fused_cap" (GEMV rows per wave step, workgroups per CU up to
  * which a wave takes one step, row steps per wave, kernel variant),
- * "gemm_nw" (waves per matmul tile: 1, 2, 4, 8), "gemm_r16" (narrow matmul tiles: 1 = 16 weight rows, 2 = 8), "gdn_cs" (column slabs of the
+ * "gemm_nw" (waves per matmul tile: 1, 2, 4, 8), "gemm_r16" (narrow matmul tiles: 1 = 16 weight rows, 2 = 8), "small_rows" (0: the two 16-row
+ * matrices of a batched projection group stay in the matmul instead of the norm's launch), "gdn_cs" (column slabs of the
  * GDN core op), "gdn_nt" / "attn_nt" (state / cache pages through nontemporal accesses), "attn_bal" (attention splits
  * under lengths in device memory: 0 = equal ranges of max_ctx, 2 = of each sequence's own length, 1 = the batch's
  * workgroups shared out by length, -1 = 1 for long ranges, else 2).  No counterpart in the reference. */

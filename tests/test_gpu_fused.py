@@ -199,3 +199,41 @@ def test_fa2_fused_is_norm_rope_append_attend(orc, dev, batch):
     ro, _ = orc.attn_decode_paged(qn, kc, vc, bt, ctx, batch, NH, NKV, HD, 16, gate=qgate.ravel()[HD:],
                                   gate_bstride=NH * 2 * HD, gate_hstride=2 * HD)
     assert np.abs(f32(out).astype(np.float64) - f32(ro)).max() <= 2e-2
+
+
+@pytest.mark.parametrize("batch", [8, 32])
+def test_gemv_fused_short_matrices_inside_the_norm_launch(orc, dev, batch):
+    """A batched projection group whose two large matrices alone fill the CUs with matmul tiles (6144 + 2048 rows = 256
+    tiles) and whose two short ones (16 rows each) would add two more: the short ones are multiplied inside the
+    RMSNorm -> Q8_1 launch.  Same bits as the checker's row loop for all four, and as the same op with the short
+    matrices left in the matmul."""
+    print(f"gemv_fused short matrices batch={batch}", flush=True)
+    K, Ns, epis = 2048, [6144, 2048, 16, 16], [1, 1, 0, 0]
+    g = synth.rng(4100 + batch)
+    Ws = [synth.q4k_centered(g, n, K, 0.02) for n in Ns]
+    x = bf(g.standard_normal((batch, K)).astype(np.float32))
+    x[batch - 1] = 0                                         # an all-zero row: every Q8_1 scale is 0
+    w = bf((g.standard_normal(K) * 0.1).astype(np.float32))
+    xq_rows = ref_activation(orc, 2, x, w)
+    spec = f"gemv_fused K={K} pro=2 G=4 batch={batch} " + " ".join(f"N{i}={n} epi{i}={e}" for i, (n, e) in enumerate(zip(Ns, epis)))
+    got = {}
+    try:
+        for small in (1, 0):
+            rt.tune_set("small_rows", small)
+            args, outs = [dev.up(x), dev.up(w)], []
+            for i, n in enumerate(Ns):
+                o = dev.empty(batch * n * (4 if epis[i] == 0 else 2))
+                rt.cuMemset(o, 0xff, batch * n * (4 if epis[i] == 0 else 2))
+                outs.append(o); args += [dev.up(Ws[i]), o]
+            launch(spec, args)
+            got[small] = [rt.from_device(o, (batch, n), np.float32 if e == 0 else np.uint16) for o, n, e in zip(outs, Ns, epis)]
+    finally:
+        rt.tune_set("small_rows", 1)
+    for i, n in enumerate(Ns):
+        assert np.array_equal(got[1][i].view(np.uint32 if epis[i] == 0 else np.uint16), got[0][i].view(np.uint32 if epis[i] == 0 else np.uint16)), i
+        for b in range(batch) if n <= 16 else (0, batch - 1):
+            y = orc.gemv_q4k_q8_1(Ws[i], xq_rows[b], n, K)
+            if epis[i] == 0:
+                assert np.array_equal(got[1][i][b].view(np.uint32), y.view(np.uint32)), (i, b)
+            else:
+                assert np.array_equal(got[1][i][b], orc.cast_bf16(y)), (i, b)
