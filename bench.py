@@ -201,7 +201,6 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     # matrix-instruction attention (within 2e-2 per attention output; tokens then follow the checker only while the
     # top-1 / top-2 margin clears the noise)
     for B, steps, exact in ((1, steps_bs1, True), (32, steps_bs32, True), (1, steps_bs1, False), (32, steps_bs32, False)):
-        runner.ATTN_EXACT = exact
         if not exact:
             S = synth_model.device_state(synth_model.synth_state(D, batch=B, seed=7, share_kv_across_batch=True))
             g = model.buildModelGraph(D, B)
@@ -209,8 +208,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
             starts = [(9419 + 4099 * i) % D.VOCAB for i in range(B)]
             warm = 8 if B == 1 else 4
             loop = runner.DeviceLoop(g, env, B, starts, 4096, max_steps=warm + steps, use_graph=use_graph,
-                                     partition=runner.fusedPartition(g) if fused else None)
-            runner.ATTN_EXACT = True
+                                     partition=runner.fusedPartition(g) if fused else None, attn_exact=False)
             loop.step(warm)
             rt.cuSync()
             e0, e1 = rt.Event().record(), rt.Event()
@@ -272,9 +270,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     pf.close()
     out["prefill"] = {"prompt_tokens": n_prompt, "chunk": chunk, "chunks_in_flight": 2, "tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
                       "first_generated_token": tok, "attention": "double precision (the state T decode steps leave, bit for bit)"}
-    runner.ATTN_EXACT = False
-    pf = prefill.Prefill(D, envs[0], chunk=chunk)
-    runner.ATTN_EXACT = True
+    pf = prefill.Prefill(D, envs[0], chunk=chunk, attn_exact=False)
     pf.run(prompt, 0, 0)
     rt.cuSync()
     t0 = time.perf_counter()
@@ -284,9 +280,7 @@ def bench_decode(rt, synth, use_graph=True, steps_bs1=240, steps_bs32=48, fused=
     out["prefill"]["with_bf16_mfma_attention"] = {"tok_per_s": round(n_prompt / wall, 1), "ms": round(wall * 1e3, 2),
                                                   "attention": "query tile x K/V tile on the bf16 matrix cores (fa2_prefill exact=0)"}
     # the reference's prefill forms on both ops that couple tokens: tiled bf16 attention and the chunked GDN recurrence
-    runner.ATTN_EXACT = False
-    pf = prefill.Prefill(D, envs[0], chunk=chunk, gdn_chunked=True)
-    runner.ATTN_EXACT = True
+    pf = prefill.Prefill(D, envs[0], chunk=chunk, gdn_chunked=True, attn_exact=False)
     pf.run(prompt, 0, 0)
     rt.cuSync()
     t0 = time.perf_counter()

@@ -45,18 +45,19 @@ class _Slot:
 
 class Prefill:
     def __init__(self, D: Dims, env: DecodeEnv, chunk: int = 1024, on_attention: Callable | None = None, overlap: bool | int = True,
-                 gdn_chunked: bool = False):
+                 gdn_chunked: bool = False, attn_exact: bool = True):
         """``env`` supplies the weights and the state buffers (those of sequence ``seq`` are updated in place).
         ``on_attention(layer, first_token_index, rows)`` receives each full-attention layer's output
         (uint16 bf16 bits ``[T, NH*HD]``) as it is produced — for tests.  ``overlap``: chunks in flight (True = 2,
         False = 1: everything on the library's first stream).  ``gdn_chunked``: the Gated-DeltaNet recurrence in chunks of
         64 tokens on the f32 matrix instruction (the form of the reference's prefill prototypes) instead of the scan;
-        state and outputs then agree with T decode steps to ~1e-6 relative, not to the bit."""
+        state and outputs then agree with T decode steps to ~1e-6 relative, not to the bit.  ``attn_exact=False``: the
+        causal attention of a chunk on the bf16 matrix cores (within 2e-2) instead of the double-precision decode kernel."""
         if chunk < 1 or chunk > 4096:
             raise ValueError("Prefill: chunk must be 1..4096 tokens")
         self.D, self.env, self.chunk, self.on_attention = D, env, int(chunk), on_attention
         self.gdn_chunked = bool(gdn_chunked)
-        self.attn_exact = bool(_runner.ATTN_EXACT)       # double-precision attention, or the matrix-instruction form (runner.ATTN_EXACT)
+        self.attn_exact = bool(attn_exact)       # double-precision attention (the bits of T decode steps), or the tiled matrix-instruction form
         self._owned: list[int] = []
         in_flight = 2 if overlap is True else max(int(overlap), 1)
         self._streams = [rt.Stream() for _ in range(in_flight)] if in_flight > 1 else []

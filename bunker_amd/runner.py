@@ -190,7 +190,7 @@ _SPEC_KEYS = {
 }
 
 
-def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str:
+def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False, attn_exact: bool = True) -> str:
     """Op name plus the constants the reference baked into the kernel text."""
     parts = [n.op] + [f"{k}={int(n.params[k])}" for k in _SPEC_KEYS[n.op]]
     if n.op == "gemm" and n.params.get("cast"):
@@ -202,20 +202,20 @@ def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False) -> str
             parts.append("ids_dev=1")
         if n.op in ("rope", "ropek", "fa2_attn"):
             parts.append("pos_dev=1")
-    if n.op == "fa2_attn" and not ATTN_EXACT:
+    if n.op == "fa2_attn" and not attn_exact:
         parts.append("exact=0")
     return " ".join(parts)
 
 
-# Attention ops run their double-precision form by default (the checker's bits, so a decode reproduces the host
-# evaluation token for token); False selects the bf16 matrix-instruction form (within 2e-2, 1.5 to 1.8 times faster on
-# the attention launches themselves) for every plan built afterwards.
-ATTN_EXACT = True
+# attn_exact (an argument of node_spec, compilePartition, compileStep, DeviceLoop and prefill.Prefill): attention ops
+# run their double-precision form by default (the checker's bits, so a decode reproduces the host evaluation token for
+# token); False selects the bf16 matrix-instruction form (within 2e-2, 1.5 to 1.8 times faster on the attention
+# launches themselves) for the plans of that call only.
 
 Q8OUT_MIN_BATCH = 8      # from this batch on producers also emit their output as Q8_1 (gemv_fused then runs its batched path)
 
 
-def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict) -> KernelPlan:
+def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict, attn_exact: bool = True) -> KernelPlan:
     """The fused op spec and slot list for a multi-node group (see fusedPartition)."""
     ops = tuple(n.op for n in grp)
     bpart = f" batch={batch}" if batch != 1 else ""
@@ -270,7 +270,7 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         P = fa.params
         spec = (f"fa2_fused HD={int(P['HD'])} NH={int(P['NH'])} NKV={int(P['NKV'])} MAX_LEN={int(P['MAX_LEN'])} "
                 f"ROT_HALF={int(rp.params['ROT_HALF'])}") + bpart + (" pos_dev=1" if device_scalars else "") + \
-            ("" if ATTN_EXACT else " exact=0")
+            ("" if attn_exact else " exact=0")
         args = [qn.inputs[0].tensorName, kn.inputs[0].tensorName, fa.inputs[2].tensorName, qn.inputs[1].tensorName,
                 kn.inputs[1].tensorName, rp.inputs[1].tensorName, rp.inputs[2].tensorName, rp.inputs[3].tensorName,
                 fa.inputs[4].tensorName, fa.inputs[5].tensorName, fa.outputs[0].tensorName]
@@ -283,7 +283,7 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
     raise NotImplementedError(f"no fused kernel for the group {ops}")
 
 
-def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_scalars: bool = False) -> list:
+def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_scalars: bool = False, attn_exact: bool = True) -> list:
     """One KernelPlan per group.  Single nodes keep the reference's op and slot order; in a partition that has
     fused groups, a stand-alone rmsnorm whose readers are all matmuls also leaves its result as Q8_1 in an
     auxiliary buffer, and those matmuls read that instead of quantizing again."""
@@ -292,7 +292,7 @@ def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_sc
     plans = []
     for grp in ordered:
         if len(grp) != 1:
-            plans.append(_group_plan(graph, grp, batch, device_scalars, q8_of))
+            plans.append(_group_plan(graph, grp, batch, device_scalars, q8_of, attn_exact))
             continue
         n = grp[0]
         args = [i.tensorName for i in n.inputs] + [o.tensorName for o in n.outputs]
@@ -312,13 +312,13 @@ def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_sc
             spec = f"gemv_fused K={K} pro=0 G=1 N0={N} epi0={1 if n.params.get('cast') else 0}" + bpart
             plans.append(KernelPlan(spec, f"gemv_{n.id}", [q8_of[n.inputs[0].tensorName], args[1], args[2]], n.grid, grp))
             continue
-        plans.append(KernelPlan(node_spec(n, batch, device_scalars), f"{n.op}_{n.id}", args, n.grid, grp))
+        plans.append(KernelPlan(node_spec(n, batch, device_scalars, attn_exact), f"{n.op}_{n.id}", args, n.grid, grp))
     return plans
 
 
-def compileStep(graph: Graph, partition: Partition, batch: int = 1, device_scalars: bool = False) -> CompiledStep:
+def compileStep(graph: Graph, partition: Partition, batch: int = 1, device_scalars: bool = False, attn_exact: bool = True) -> CompiledStep:
     ordered = topoOrder(graph, partition)
-    plans = compilePartition(graph, ordered, batch, device_scalars)
+    plans = compilePartition(graph, ordered, batch, device_scalars, attn_exact)
     cache: dict[str, rt.LoadedKernel] = {}
     schedule = []
     for p in plans:
@@ -500,7 +500,7 @@ class DeviceLoop:
     """
 
     def __init__(self, graph: Graph, env: DecodeEnv, batch: int, start_tokens, start_pos, max_steps: int,
-                 partition: Partition | None = None, use_graph: bool = True, feed: bool = True):
+                 partition: Partition | None = None, use_graph: bool = True, feed: bool = True, attn_exact: bool = True):
         if not env.inplace:
             raise ValueError("DeviceLoop needs DecodeEnv(inplace_state=True)")
         ids = np.asarray(start_tokens, np.int32).reshape(batch)
@@ -516,7 +516,7 @@ class DeviceLoop:
             raise ValueError(f"DeviceLoop: start position {int(pos.max())} + {max_steps} steps exceeds the KV capacity "
                              f"MAX_LEN={max_len}")
         self.graph, self.env, self.batch, self.max_steps = graph, env, batch, max_steps
-        self.compiled = compileStep(graph, partition or choosePartition(graph), batch, device_scalars=True)
+        self.compiled = compileStep(graph, partition or choosePartition(graph), batch, device_scalars=True, attn_exact=attn_exact)
         env.bind(self.compiled)
         self.d_ids = rt.to_device(ids)
         self.d_pos = rt.to_device(pos)

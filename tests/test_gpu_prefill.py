@@ -101,6 +101,77 @@ def test_gdn_prefill_chunked_form_against_the_scan(Hg, T):
     assert np.all(np.abs(o1 - o0) <= 2.0 ** -7 * np.abs(o0) + 1e-4), np.abs(o1 - o0).max()
 
 
+def _gdn_inputs(g, Hg, T, decay_mix):
+    C = 3 * Hg * 128
+    conv = bf(g.standard_normal((T, C)).astype(np.float32))
+    z = bf(g.standard_normal((T, Hg * 128)).astype(np.float32))
+    A_log = g.uniform(-2, 1, Hg).astype(np.float32)
+    dt_bias = bf(g.standard_normal(Hg).astype(np.float32))
+    a_p = (g.standard_normal((T, Hg)) * 2).astype(np.float32); b_p = g.standard_normal((T, Hg)).astype(np.float32)
+    if decay_mix:
+        # strong and weak decays in the same run: head 0 barely decays (decay ~ 1 - 1e-4), head 1 loses most of its
+        # state at every token (decay ~ e^-8), the others alternate between the two by token
+        A_log[0] = -4.0; a_p[:, 0] = -4.0
+        if Hg > 1:
+            A_log[1] = 1.0; a_p[:, 1] = 3.0
+        for h in range(2, Hg):
+            a_p[::2, h] = -5.0; a_p[1::2, h] = 3.0
+    norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    S = (g.standard_normal((Hg, 128, 128)) * 0.02).astype(np.float32)
+    return conv, z, A_log, dt_bias, a_p, b_p, norm_w, S
+
+
+def _gdn_prefill_gpu(inputs, Hg, T, chunked):
+    ptrs = [rt.to_device(a) for a in inputs]
+    dout = rt.cuAlloc(T * Hg * 128 * 2)
+    rt.cuMemset(dout, 0xff, T * Hg * 128 * 2)
+    _launch(f"gdn_prefill LVH={Hg} T={T} chunked={chunked}", ptrs + [dout, ptrs[7]])
+    out = rt.from_device(dout, (T, Hg * 128), np.uint16)
+    S = rt.from_device(ptrs[7], inputs[7].shape, np.float32)
+    for p in ptrs + [dout]:
+        rt.cuFree(p)
+    return out, S
+
+
+@pytest.mark.parametrize("Hg,T,decay_mix", [(3, 200, False), (16, 1024, False), (4, 300, True)])
+def test_gdn_prefill_both_forms_against_the_checker_chained_over_T(orc, Hg, T, decay_mix):
+    """Scan and chunked form against the checker's single-token step chained over T tokens (the multi-token host loop of
+    prototypes/gdn_gated.ts:67-88 refGDN, one token at a time).  Yardstick: the checker with both k-reductions
+    accumulated in double (rows_per_chain=0).  Both GPU forms: state within 1e-4 of the largest state element per
+    head, bf16 outputs within 2e-2 max-abs (plus one bf16 step for the large ones).  At T = 200 the scan must also
+    return the bytes of the checker in the canonical f32 order (rows_per_chain=16) — past the 16-token lookahead of
+    its LDS staging and past a 64-token chunk boundary."""
+    print(f"gdn_prefill vs checker Hg={Hg} T={T} decay_mix={decay_mix}", flush=True)
+    g = synth.rng(8300 + Hg + T)
+    inp = _gdn_inputs(g, Hg, T, decay_mix)
+    conv, z, A_log, dt_bias, a_p, b_p, norm_w, S = inp
+    ref_o = np.empty((T, Hg * 128), np.uint16)
+    s = S
+    for t in range(T):
+        ref_o[t], s = orc.gdn_step(conv[t], z[t], A_log, dt_bias, a_p[t], b_p[t], norm_w, s, Hg, rows_per_chain=0)
+    ref_S = s.astype(np.float64); ro = f32(ref_o).astype(np.float64)
+    canon = None
+    if T <= 300:
+        canon_o = np.empty_like(ref_o); s = S
+        for t in range(T):
+            canon_o[t], s = orc.gdn_step(conv[t], z[t], A_log, dt_bias, a_p[t], b_p[t], norm_w, s, Hg, rows_per_chain=16)
+        canon = (canon_o, s)
+    for chunked in (0, 1):
+        out, gS = _gdn_prefill_gpu(inp, Hg, T, chunked)
+        assert not (out == 0xffff).any(), "an output row was left unwritten"
+        o = f32(out).astype(np.float64)
+        assert np.isfinite(o).all() and np.isfinite(gS).all()
+        for h in range(Hg):
+            scale = np.abs(ref_S[h]).max()
+            err = np.abs(gS[h].astype(np.float64) - ref_S[h]).max()
+            assert err <= 1e-4 * scale, (chunked, h, err, scale)
+        d = np.abs(o - ro)
+        assert np.all(d <= 2e-2 + 2.0 ** -7 * np.abs(ro)), (chunked, d.max(), np.unravel_index(d.argmax(), d.shape))
+        if chunked == 0 and canon is not None:
+            assert np.array_equal(out, canon[0]), "scan output bytes differ from the checker's canonical order"
+            assert np.array_equal(gS.view(np.uint32), canon[1].view(np.uint32)), "scan state bits differ"
+
+
 @pytest.mark.parametrize("T,pos0,splits", [(6, 0, 0), (37, 12, 0), (37, 60, 3), (2, 15, 2)])
 def test_fa2_prefill_token_pairs_return_the_single_row_bits(orc, T, pos0, splits):
     """The matrix-instruction form (exact=0): two consecutive tokens per workgroup (their heads side by side in the 16 columns of the products, each column
@@ -379,11 +450,7 @@ def test_prefill_in_the_chunked_and_tiled_forms_stays_close_to_the_exact_one():
     results = []
     for fast in (False, True):
         env = runner.DecodeEnv(g, W, synth_model.device_state(S), inplace_state=True)
-        runner.ATTN_EXACT = not fast
-        try:
-            pf = prefill.Prefill(D, env, chunk=chunk, gdn_chunked=fast)
-        finally:
-            runner.ATTN_EXACT = True
+        pf = prefill.Prefill(D, env, chunk=chunk, gdn_chunked=fast, attn_exact=not fast)
         tok, val = pf.run(prompt, seq=seq, pos0=0)
         state = {"logits": rt.from_device(pf.d_logits, (D.VOCAB,), np.float32).astype(np.float64), "tok": tok}
         for l in range(D.NL):

@@ -15,8 +15,9 @@ f32 = synth.bf16_to_f32
 NH, NKV, HD = 16, 2, 256
 
 
-def _both(g, B, L, splits_req=0):
-    """One problem through both entry points; returns (out, lse) of each and the inputs."""
+def _both(g, B, L, splits_req=0, own_choice=False):
+    """One problem through both entry points; returns (out, lse) of each and the inputs.  own_choice: the no-alloc
+    entry point is handed splits = 0 and picks the count itself, the workspace form gets what bk_attn_plan returns."""
     kc, vc, bt, ctx = synth.paged_kv_random(g, B, L)
     q = bf(g.standard_normal((B, NH, HD)).astype(np.float32))
     splits, ws = rt.attn_plan(B, NKV, L, splits_req)
@@ -34,7 +35,7 @@ def _both(g, B, L, splits_req=0):
     for p in (o1, o2):
         rt.cuMemset(p, 0xFF, B * NH * HD * 2)
     print(f"attn_decode_noalloc B={B} L={L} splits={splits}", flush=True)
-    rt.attn_decode_noalloc(dq, dkc, dvc, dbt, bt.shape[1], dctx, L, o1, l1, B, NH, NKV, HD, 16, splits)
+    rt.attn_decode_noalloc(dq, dkc, dvc, dbt, bt.shape[1], dctx, L, o1, l1, B, NH, NKV, HD, 16, 0 if own_choice else splits)
     rt.attn_decode(dq, dkc, dvc, dbt, bt.shape[1], dctx, L, o2, l2, B, NH, NKV, HD, 16, splits, dws, ws)
     rt.cuSync()
     res = (rt.from_device(o1, (B, NH, HD), np.uint16), rt.from_device(l1, (B, NH), np.float32),
@@ -57,9 +58,14 @@ def test_noalloc_attention_equals_the_workspace_form(orc):
     ro, rl = orc.attn_decode_paged(q, kc, vc, bt, ctx, 2, NH, NKV, HD, 16)
     assert np.abs(f32(o1).astype(np.float64) - f32(ro)).max() <= 2e-2
     assert np.all(np.abs(l1 - rl) <= 1e-4 * np.maximum(1, np.abs(rl)))
-    # a third, with the library's own split count asked for through splits = 0 on both sides
-    (o1, l1, o2, l2), _, _ = _both(g, 3, 4096, 0)
+    # a third: the no-alloc entry point itself is handed splits = 0 (its own choice, held to what the array takes) and
+    # must cut the pages like bk_attn_decode at the count bk_attn_plan returns; also against the checker
+    (o1, l1, o2, l2), (q, kc, vc, bt, ctx), s_own = _both(g, 3, 4096, 0, own_choice=True)
+    assert s_own > 1
     assert np.array_equal(o1, o2) and np.array_equal(l1.view(np.uint32), l2.view(np.uint32))
+    ro, rl = orc.attn_decode_paged(q, kc, vc, bt, ctx, 3, NH, NKV, HD, 16)
+    assert np.abs(f32(o1).astype(np.float64) - f32(ro)).max() <= 2e-2
+    assert np.all(np.abs(l1 - rl) <= 1e-4 * np.maximum(1, np.abs(rl)))
 
 
 def test_noalloc_attention_refuses_more_partials_than_the_array_holds():
