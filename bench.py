@@ -55,6 +55,7 @@ def measured_traffic(kernel: str, shape: str):
     return None
 SHAPES = [("qkv", 6144, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144), ("lm_head", 151936, 2048)]
 ROTATION_BYTES = 600e6  # every shape rotates through copies of its matrix that add up to at least this much
+PREWARM_S = 0.4         # untimed GEMV launches in front of the timed region (clock warm-up; reported as prewarm_ms)
 
 
 def gemv_bytes(N, K, batch=1):
@@ -569,8 +570,9 @@ def bench_prefill_ops(rt, synth, iters=5):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # 2000 timed steps after 500 warm-up steps: the clocks of an idle GPU take a few thousand launches to settle
-    # (the same kernels measure 8 % slower in a 200-step run); the whole GEMV section still lasts 0.2 s
+    # 2000 timed steps after 500 warm-up steps by default; a fixed, untimed clock warm-up (PREWARM_S) runs in front of
+    # them whatever --steps says, because the clocks of an idle GPU take a few thousand launches to settle (without it
+    # the same kernels measured 8 % slower in a 20- or 200-step run)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -642,6 +644,11 @@ def main():
         e0, e1 = rt.Event(), rt.Event()
         for w in range(args.warmup):
             launch(name, N, K, w)
+        if args.mode == "graph":
+            # one untimed replay directly in front of the timed one: the timed replay is then queued while the device
+            # is still busy, so its K launches are measured at the device's own rate even when K is small (a lone
+            # 20-launch replay also pays the host's submission latency, +0.5 us per launch)
+            graphs[name].launch()
         e0.record()
         if args.mode == "graph":
             graphs[name].launch()
@@ -655,7 +662,7 @@ def main():
     # duration of the shortest possible launch in the same mode (16-byte read by one workgroup): the floor under every
     # kernel here, and the reason the three small shapes cannot come near the HBM roofline
     sink = rt.cuAlloc(256)
-    n_floor = min(args.steps, 500)
+    n_floor = 500
     for _ in range(20):
         rt.memread(sink, 16, sink + 128)
     rt.cuSync()
@@ -664,16 +671,31 @@ def main():
             for _ in range(n_floor):
                 rt.memread(sink, 16, sink + 128)
         rt.cuSync()
-    f0, f1 = rt.Event(), rt.Event()
-    f0.record()
-    if args.mode == "graph":
-        gfl.launch()
-    else:
-        for _ in range(n_floor):
-            rt.memread(sink, 16, sink + 128)
-    f1.record()
-    rt.cuSync()
-    launch_floor_us = f0.elapsed_ms(f1) * 1e3 / n_floor
+
+    def measure_floor():
+        f0, f1 = rt.Event(), rt.Event()
+        f0.record()
+        if args.mode == "graph":
+            gfl.launch()
+        else:
+            for _ in range(n_floor):
+                rt.memread(sink, 16, sink + 128)
+        f1.record()
+        rt.cuSync()
+        return f0.elapsed_ms(f1) * 1e3 / n_floor
+
+    # Untimed clock warm-up of fixed length, so that a short run (--steps 20) is measured at the clocks a long one
+    # settles at: the clocks of an idle GPU take a few thousand launches to come up.  The same GEMV launches as the timed
+    # region, all four shapes in turn, for PREWARM_S seconds of wall time; --steps / --warmup keep their meaning.
+    launch_floor_cold_us = measure_floor()
+    t_pw = time.perf_counter()
+    while time.perf_counter() - t_pw < PREWARM_S:
+        for name, N, K in SHAPES:
+            for i in range(100 if N < 100000 else 25):
+                launch(name, N, K, i)
+        rt.cuSync()
+    prewarm_ms = (time.perf_counter() - t_pw) * 1e3
+    launch_floor_us = measure_floor()
     rt.cuFree(sink)
 
     t0 = time.perf_counter()
@@ -725,6 +747,8 @@ def main():
                    "launch_mode": args.mode, "device": info["name"], "cus": info["cus"]},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "launch_floor_us": round(launch_floor_us, 3),
+        "launch_floor_before_prewarm_us": round(launch_floor_cold_us, 3),
+        "prewarm_ms": round(prewarm_ms, 1),
         "wall_ms_per_step_incl_warmup": round(wall * 1e3 / args.steps, 5),
         "per_shape": per_shape,
         "roofline": roofline,
