@@ -31,6 +31,7 @@ struct Kernel {
   int nslots = 0;
   void* scratch = nullptr;     // per-handle device workspace, allocated at create time
   size_t scratch_bytes = 0;
+  int generation = 0;          // how often the slot has been reused
   int64_t get(const char* k, int64_t def) const {
     auto it = p.find(k);
     return it == p.end() ? def : it->second;
@@ -39,17 +40,28 @@ struct Kernel {
 };
 
 static std::vector<Kernel> g_kernels;
+static std::vector<int> g_free_slots;          // destroyed handles' slots, taken again by bk_kernel_create
+// handle = slot | generation << 20: a handle kept past its bk_kernel_destroy does not name the slot's next kernel
+enum : int { HANDLE_SLOTS = 1 << 20, HANDLE_GENS = 1 << 10 };
+static int handle_of(int slot) { return slot | ((g_kernels[slot].generation & (HANDLE_GENS - 1)) << 20); }
+static Kernel* kernel_of(int handle) {
+  const int slot = handle & (HANDLE_SLOTS - 1);
+  if (handle < 0 || slot >= (int)g_kernels.size()) return nullptr;
+  Kernel& k = g_kernels[slot];
+  return (k.run && handle_of(slot) == handle) ? &k : nullptr;
+}
 
 // bk_shutdown: every handle's workspace goes back to the device and the handles become invalid
 void kernels_release_all() {
   for (Kernel& k : g_kernels)
     if (k.scratch) (void)hipFree(k.scratch);
   g_kernels.clear();
+  g_free_slots.clear();
 }
 
 std::string kernel_label(int kernel) {
-  if (kernel < 0 || kernel >= (int)g_kernels.size()) return "?";
-  return g_kernels[kernel].spec;
+  const Kernel* k = kernel_of(kernel);
+  return k ? k->spec : "?";
 }
 
 static int need(Kernel& k, const char* key) {
@@ -537,6 +549,7 @@ int bk_tune_set(const char* key, int value) {
 
 int bk_kernel_create(const char* spec) {
   BK_NEED_INIT();
+  if (capturing()) return set_error(BK_ERR_STATE, "bk_kernel_create: not legal between bk_capture_begin and bk_capture_end");
   BK_REQUIRE(spec && *spec, "bk_kernel_create: empty spec");
   Kernel k;
   k.spec = spec;
@@ -557,15 +570,25 @@ int bk_kernel_create(const char* spec) {
     if (k.scratch) (void)hipFree(k.scratch);
     return rc;
   }
+  // a destroyed handle's slot is taken again (a server that builds a loop per request would otherwise grow the table
+  // without bound); the generation in the upper bits makes a stale handle number an error instead of another kernel
+  if (!g_free_slots.empty()) {
+    const int slot = g_free_slots.back();
+    g_free_slots.pop_back();
+    k.generation = g_kernels[slot].generation + 1;
+    g_kernels[slot] = k;
+    return handle_of(slot);
+  }
+  BK_REQUIRE(g_kernels.size() < (size_t)HANDLE_SLOTS, "bk_kernel_create: more than %d live handles", HANDLE_SLOTS);
   g_kernels.push_back(k);
-  return (int)g_kernels.size() - 1;
+  return handle_of((int)g_kernels.size() - 1);
 }
 
 int bk_launch(int kernel, const uint64_t* slots, int nslots) {
   BK_NEED_INIT();
-  if (kernel < 0 || kernel >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "bk_launch: unknown kernel handle %d", kernel);
-  Kernel& k = g_kernels[kernel];
-  if (!k.run) return set_error(BK_ERR_STATE, "bk_launch: kernel handle %d has been destroyed", kernel);
+  Kernel* kp = kernel_of(kernel);
+  if (!kp) return set_error(BK_ERR_STATE, "bk_launch: unknown or destroyed kernel handle %d", kernel);
+  Kernel& k = *kp;
   BK_REQUIRE(slots, "bk_launch: null slots");
   BK_REQUIRE(nslots >= k.nslots, "bk_launch: '%s' takes %d argument slots, got %d", k.op.c_str(), k.nslots, nslots);
   if (prof_on()) {
@@ -580,22 +603,28 @@ int bk_launch(int kernel, const uint64_t* slots, int nslots) {
 
 int bk_kernel_destroy(int kernel) {
   BK_NEED_INIT();
-  if (kernel < 0 || kernel >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "bk_kernel_destroy: unknown kernel handle %d", kernel);
-  Kernel& k = g_kernels[kernel];
-  if (!k.run) return BK_OK;                       // destroyed before
+  if (capturing()) return set_error(BK_ERR_STATE, "bk_kernel_destroy: not legal between bk_capture_begin and bk_capture_end");
+  const int slot = kernel & (HANDLE_SLOTS - 1);
+  if (kernel < 0 || slot >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "bk_kernel_destroy: unknown kernel handle %d", kernel);
+  Kernel& k = g_kernels[slot];
+  if (!k.run || handle_of(slot) != kernel) return BK_OK;      // destroyed before
   if (k.scratch) {
     BK_HIP(hipDeviceSynchronize());               // launches that still use the workspace finish first
     BK_HIP(hipFree(k.scratch));
   }
-  k.scratch = nullptr; k.scratch_bytes = 0; k.run = nullptr;     // the slot stays, so later handles keep their numbers
-  k.spec += " [destroyed]";
+  k.scratch = nullptr; k.scratch_bytes = 0; k.run = nullptr;
+  k.p.clear();
+  k.spec = k.op + " [destroyed]";
+  g_free_slots.push_back(slot);
   return BK_OK;
 }
 
 int bk_kernel_describe(int kernel, char* buf, int cap) {
-  if (kernel < 0 || kernel >= (int)g_kernels.size()) return set_error(BK_ERR_STATE, "unknown kernel handle %d", kernel);
   BK_REQUIRE(buf && cap > 0, "bk_kernel_describe: bad buffer");
-  snprintf(buf, cap, "%s [%d slots]", g_kernels[kernel].spec.c_str(), g_kernels[kernel].nslots);
+  const int slot = kernel & (HANDLE_SLOTS - 1);
+  if (kernel < 0 || slot >= (int)g_kernels.size() || handle_of(slot) != kernel)
+    return set_error(BK_ERR_STATE, "unknown kernel handle %d", kernel);
+  snprintf(buf, cap, "%s [%d slots]", g_kernels[slot].spec.c_str(), g_kernels[slot].nslots);
   return BK_OK;
 }
 

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void attn_decode_kernel(AttnArgs A)
   const int tk_n = n / A.G;
   const bool col_valid = tk_n < ntk;
   const int row_n = row0 + (col_valid ? tk_n : 0);
-  const int len = (A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add;       // of this lane's column
+  const int len = min((A.ctx_len ? A.ctx_len[row_n] : A.ctx_scalar) + A.ctx_add, A.max_ctx);       // of this lane's column
   int len_wg = len;                             // the longest column: what the cache holds behind it need not be a number
 #pragma unroll
   for (int off = 1; off < 16; off <<= 1) len_wg = max(len_wg, __shfl_xor(len_wg, off));
@@ -364,7 +364,7 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
   // start-up and merge decide the time and the plan's own cost of about a microsecond is not won back), else relative
   // splits; the rows of a prompt keep the plain form (paired and single rows must cut alike).
   // balanced: the batch shares batch * splits slots; a slot's page budget is largest when rows - 1 slots are held back
-  A.slots = 0; A.rel = 0; A.max_pages = pages;
+  A.slots = 0; A.rel = 0; A.max_pages = pages; A.max_ctx = ctx_len ? max_ctx : ctx_scalar + ctx_add;
   const bool prompt_rows = block_table && bt_stride == 0;
   if (ctx_len && tpw == 1 && !prompt_rows && splits > 1 && g_tune_attn_bal != 0) {
     const bool can_balance = batch <= 64 && batch * splits <= ATT_MAX_SPLITS && (int64_t)batch * pages < (1 << 24) &&

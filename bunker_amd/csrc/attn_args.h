@@ -38,6 +38,7 @@ struct AttnArgs {
   int bt_stride, ctx_scalar, ctx_add, NH, NKV, G, splits, pages_per_split;
   int tpw, rows;              // query rows per workgroup (1, or 2 consecutive rows of one sequence: prompt tokens), rows in all
   int max_pages;              // pages of the longest context the caller allows
+  int max_ctx;                // that context in tokens: a length above it is read as max_ctx (also inside the last page)
   int rel;                    // 1: lengths in device memory, every sequence cuts its own pages into `splits` equal ranges
   int slots;                  // > 0: balanced form, this many workgroup slots per KV head shared by the rows (rows <= 64)
   float scale;

@@ -146,7 +146,8 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   if (!attn_wg_range(A, lane, b, split, p_begin, p_end)) return;
   const int row = __builtin_amdgcn_readfirstlane(b);          // one query row per workgroup (tpw = 1)
   const int kvh = blockIdx.y;
-  const int len = (A.ctx_len ? A.ctx_len[row] : A.ctx_scalar) + A.ctx_add;
+  const int len_raw = (A.ctx_len ? A.ctx_len[row] : A.ctx_scalar) + A.ctx_add;
+  const int len = min(len_raw, A.max_ctx);                     // a length above the bound is read as the bound
   const int lim = min(len, p_end * ATT_PAGE);                  // tokens of this split end here
   const int npg = max(p_end - p_begin, 0);
   const int ntiles = (npg + EX_TILE_PAGES - 1) / EX_TILE_PAGES;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
   if (PREP) {
     uint32_t* lds_q = (uint32_t*)xch;
     uint16_t* sh = (uint16_t*)(lds_q + ATT_HD * EX_COLS) + wave * ATT_HD;
-    const int pos_raw = len - 1;
+    const int pos_raw = len_raw - 1;
     const int pos = min(max(pos_raw, 0), A.pmax_len - 1);
     const int ppage = pos / ATT_PAGE - p_begin, slot = pos % ATT_PAGE;
     const bool holds = pos == pos_raw && ppage >= 0 && ppage < npg;

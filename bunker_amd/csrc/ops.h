@@ -10,6 +10,7 @@ enum : int { DT_F32 = 0, DT_BF16 = 1 };
 
 // runtime.hip
 bool inited();
+bool capturing();        // between bk_capture_begin and bk_capture_end: nothing may allocate, free, copy or wait
 int current_device();
 bool prof_on();
 int prof_begin(int kernel);

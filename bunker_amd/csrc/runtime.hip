@@ -61,6 +61,11 @@ int prof_end() {
 }
 std::string kernel_label(int kernel);   // api.hip
 void kernels_release_all();             // api.hip
+static std::map<uint64_t, int> g_graph_nodes;     // executable graph (bk_capture_end) -> kernel nodes it holds
+static void graphs_release_all() {
+  for (auto& kv : g_graph_nodes) (void)hipGraphExecDestroy((hipGraphExec_t)(uintptr_t)kv.first);
+  g_graph_nodes.clear();
+}
 static int prof_collect() {
   if (int rc = sync_all()) return rc;
   for (auto& p : g_pending) {
@@ -85,6 +90,7 @@ using namespace bk;
 // Between bk_capture_begin and bk_capture_end only launches are recorded; anything else would either end the capture with
 // an error of the runtime's or, for a memset, put a node into the graph that replays wrongly on this platform.
 static bool g_capturing = false;
+bool bk::capturing() { return g_capturing; }
 #define BK_NOT_CAPTURING(name) \
   do { if (g_capturing) return set_error(BK_ERR_STATE, name ": not legal between bk_capture_begin and bk_capture_end"); } while (0)
 
@@ -118,6 +124,7 @@ int bk_init(int device) {
 int bk_shutdown(void) {
   if (!g_inited) return BK_OK;
   (void)sync_all();
+  graphs_release_all();                   // executable graphs of bk_capture_end that were never destroyed
   kernels_release_all();
   for (auto& p : g_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto& ev : g_pool) (void)hipEventDestroy(ev);
@@ -311,7 +318,6 @@ int bk_event_destroy(uint64_t ev) {
   return BK_OK;
 }
 
-static std::map<uint64_t, int> g_graph_nodes;     // executable graph -> kernel nodes it holds
 
 int bk_capture_begin(void) {
   BK_NEED_INIT();

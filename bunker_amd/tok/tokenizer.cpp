@@ -372,7 +372,13 @@ struct Tokenizer {
   // the call.  The table belongs to the call, not to the tokenizer, so calls on several threads share nothing.
   struct PieceCache {
     struct Entry { uint8_t len = 0xFF, nids = 0; uint8_t bytes[24]; uint32_t ids[8]; };
-    std::vector<Entry> slots = std::vector<Entry>(1 << 14);
+    std::vector<Entry> slots;
+    // sized from the input (a slot per 8 bytes, 256 to 16384 slots): a chat-sized call does not pay for a megabyte
+    explicit PieceCache(size_t input_bytes) {
+      size_t want = 256;
+      while (want < (1u << 14) && want < input_bytes / 8) want <<= 1;
+      slots.resize(want);
+    }
     static size_t hash(const uint8_t* s, size_t n) {
       uint64_t h = 0xcbf29ce484222325ull ^ n;
       for (size_t i = 0; i < n; i++) h = (h ^ s[i]) * 0x100000001b3ull;
@@ -406,7 +412,7 @@ struct Tokenizer {
   }
 
   void encode(const uint8_t* s, size_t n, std::vector<uint32_t>& out) const {
-    PieceCache cache;
+    PieceCache cache(n);
     size_t start = 0, i = 0;
     while (i < n && !added.empty()) {
       if (!added_first[s[i]]) { i++; continue; }       // no added token begins with this byte

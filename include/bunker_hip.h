@@ -79,9 +79,10 @@ BK_API int bk_prof_report(char* buf, int cap);       /* profGpuReport, src/ttir.
  * tried the same with CUDA graphs through bun:ffi and gave up on struct-pointer
  * crashes (LOG.md:710-738); here the graph lives behind scalar handles.
  * Between begin and end only launches are legal: alloc, free, memset, copies,
- * sync, event waits, a stream switch and a graph launch return an error (state
- * -3, "not legal between bk_capture_begin and bk_capture_end") and leave the
- * capture open. */
+ * sync, event waits, a stream switch, a graph launch, bk_kernel_create and
+ * bk_kernel_destroy (they allocate, clear and free a handle's workspace) return
+ * an error (state -3, "not legal between bk_capture_begin and bk_capture_end")
+ * and leave the capture open. */
 BK_API int bk_capture_begin(void);
 BK_API int bk_capture_end(uint64_t* graph);
 BK_API int bk_graph_launch(uint64_t graph);
@@ -111,8 +112,11 @@ BK_API int bk_kernel_create(const char* spec);
 BK_API int bk_launch(int kernel, const uint64_t* slots, int nslots);
 /* Handles of ops with intermediate results (gemm, gemv_fused, fa2_*, argmax, gdn_prefill) own a device workspace,
  * allocated by bk_kernel_create.  bk_kernel_destroy waits for the device, returns the workspace and makes the handle
- * invalid (later handles keep their numbers); bk_shutdown does the same for every handle.  cuModuleUnload is the
- * reference's nearest counterpart (its kernels own no device memory, src/ttir.ts:488-491). */
+ * invalid: its slot is taken again by a later bk_kernel_create under a new handle number (slot | generation << 20), so
+ * a process that builds and destroys handles per request does not grow the table, and a handle kept past its destroy
+ * is refused instead of naming another kernel; bk_shutdown releases every handle and every graph of bk_capture_end
+ * that was not destroyed.  cuModuleUnload is the reference's nearest counterpart (its kernels own no device memory,
+ * src/ttir.ts:488-491). */
 BK_API int bk_kernel_destroy(int kernel);
 BK_API int bk_kernel_describe(int kernel, char* buf, int cap);
 

@@ -144,22 +144,32 @@ def test_advance_stops_at_the_capacity(dev):
 
 @pytest.mark.parametrize("splits", [1, 3])
 def test_attention_lengths_outside_the_bound(orc, dev, splits):
-    """ctx_len <= 0: zeros and lse = -inf; ctx_len > max_ctx: read as max_ctx (no page beyond the block-table row)."""
+    """ctx_len <= 0: zeros and lse = -inf; ctx_len > max_ctx: read as max_ctx, to the token (max_ctx = 60 ends inside a
+    page).  The over-long length sits on a middle row, and every block-table row has four spare columns with valid page
+    ids behind the four the bound allows (the caches hold those pages): a missing clamp would read memory of this test."""
     print(f"attn bounds splits={splits}", flush=True)
     g = synth.rng(904)
-    B, L = 3, 64
-    kc, vc, bt, ctx = synth.paged_kv_random(g, B, L)
-    ctx[:] = [0, 40, 100]
+    B, L, L_alloc = 4, 60, 128
+    kc, vc, bt, ctx = synth.paged_kv_random(g, B, L_alloc)          # 8 pages per table row, 32 pages in the caches
+    ctx[:] = [40, 100, 0, 57]
     q = bf(g.standard_normal((B, NH, HD)).astype(np.float32))
     s, ws = rt.attn_plan(B, NKV, L, splits)
     assert s == splits
-    dws = dev.empty(ws) if ws else 0
-    dout, dlse = dev.empty(B * NH * HD * 2), dev.empty(B * NH * 4)
-    rt.attn_decode(dev.up(q), dev.up(kc), dev.up(rt.v_pages_to_device_layout(vc)), dev.up(bt), bt.shape[1], dev.up(ctx), L,
-                   dout, dlse, B, NH, NKV, HD, 16, s, dws, ws)
-    out = rt.from_device(dout, (B, NH, HD), np.uint16); lse = rt.from_device(dlse, (B, NH), np.float32)
-    assert not out[0].any() and np.all(np.isneginf(lse[0]))
-    ref_ctx = np.array([1, 40, 64], np.int32)
+    dq, dkc, dvc, dbt, dctx = dev.up(q), dev.up(kc), dev.up(rt.v_pages_to_device_layout(vc)), dev.up(bt), dev.up(ctx)
+    ref_ctx = np.array([40, 60, 1, 57], np.int32)
     ro, rl = orc.attn_decode_paged(q, kc, vc, bt, ref_ctx, B, NH, NKV, HD, 16)
-    assert np.abs(f32(out[1:]).astype(np.float64) - f32(ro[1:])).max() <= 2e-2
-    assert np.all(np.abs(lse[1:] - rl[1:]) <= 1e-4 * np.maximum(1, np.abs(rl[1:])))
+    keep = [0, 1, 3]
+    for exact in (False, True):
+        if exact:
+            s2, ws2 = rt.attn_plan_exact(B, NKV, L, splits)
+        else:
+            s2, ws2 = s, ws
+        dws = dev.empty(ws2) if ws2 else 0
+        dout, dlse = dev.empty(B * NH * HD * 2), dev.empty(B * NH * 4)
+        (rt.attn_decode_exact if exact else rt.attn_decode)(dq, dkc, dvc, dbt, bt.shape[1], dctx, L, dout, dlse, B, NH, NKV, HD, 16, s2, dws, ws2)
+        out = rt.from_device(dout, (B, NH, HD), np.uint16); lse = rt.from_device(dlse, (B, NH), np.float32)
+        assert not out[2].any() and np.all(np.isneginf(lse[2])), exact
+        if exact:
+            assert np.array_equal(out[keep], ro[keep])
+        assert np.abs(f32(out[keep]).astype(np.float64) - f32(ro[keep])).max() <= 2e-2, exact
+        assert np.all(np.abs(lse[keep] - rl[keep]) <= 1e-4 * np.maximum(1, np.abs(rl[keep]))), exact

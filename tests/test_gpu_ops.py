@@ -428,12 +428,22 @@ def test_only_launches_are_recorded_between_capture_begin_and_end():
     dx = rt.to_device(x); dq = rt.cuAlloc(2 * 36); rt.cuMemset(dq, 0, 72)
     host = np.zeros(72, np.uint8)
     p = C.c_uint64(0)
+    k_spare = rt.compileAndLoad("gemm N=64 K=256")            # owns a workspace
     with rt.Graph() as gr:
         rt.quantize_q8_1(dx, dq, 64, 1, rt.F32)
         for rc in (lib.bk_memset(dq, 0, 72), lib.bk_sync(), lib.bk_alloc(256, C.byref(p)), lib.bk_free(dq),
-                   lib.bk_dtoh(host.ctypes.data_as(C.c_void_p), dq, 72), lib.bk_graph_launch(1)):
+                   lib.bk_dtoh(host.ctypes.data_as(C.c_void_p), dq, 72), lib.bk_graph_launch(1),
+                   lib.bk_kernel_create(b"gemm N=64 K=256"), lib.bk_kernel_destroy(k_spare.fn)):
             assert rc != 0 and b"not legal between bk_capture_begin and bk_capture_end" in lib.bk_last_error()
     assert gr.node_count() == 1
+    # the handle the capture refused to destroy is still alive; once destroyed its slot is reused under another number
+    # and the old number is refused
+    slots = (C.c_uint64 * 3)(0, 0, 0)
+    rt.unloadKernel(k_spare)
+    k_new = rt.compileAndLoad("gemm N=64 K=256")
+    assert k_new.fn != k_spare.fn and (k_new.fn & 0xfffff) == (k_spare.fn & 0xfffff)
+    assert lib.bk_launch(k_spare.fn, slots, 3) != 0 and b"destroyed" in lib.bk_last_error()
+    rt.unloadKernel(k_new)
     for _ in range(2):
         rt.cuMemset(dq, 0, 72)
         gr.launch(); rt.cuSync()
