@@ -505,6 +505,103 @@ def bench_kernels(rt, synth, use_graph=True, iters=50):
     return res
 
 
+def bench_fused_ops(rt, synth, use_graph=True, iters=48, batches=(1, 32)):
+    """The fused ops the decode step is made of, each on its own (one stream, weights and state rotated through 24
+    copies like the 24 layers of the step): microseconds per launch and algorithmic GB/s.  The same launches a decode
+    step makes, without the device loop, the prompt pass or a second stream around them."""
+    g = synth.rng(21)
+    bf = synth.f32_to_bf16
+    H, I, Hg, NH, NKV, HD, MAXL, POS = 2048, 6144, 16, 16, 2, 256, 4352, 4096
+    ROT = 24
+    res = {}
+
+    def q4k(N, K):
+        h = synth.q4k_random(g, N, K)
+        first = rt.to_device(h)
+        out = [first]
+        for _ in range(ROT - 1):
+            p = rt.cuAlloc(h.nbytes); rt.cuDtoD(p, first, h.nbytes); out.append(p)
+        return out, h.nbytes
+
+    def time_op(key, spec, args_of, nbytes, owned):
+        k = rt.compileAndLoad(spec)
+        def launch(i):
+            rc = rt.cuLaunch(k, [1, 1, 1], [128, 1, 1], args_of(i))
+            if rc != 0:
+                raise rt.BunkerError(f"{spec}: {rt.last_error()}")
+        for i in range(3):
+            launch(i)
+        us = _time_launches(rt, lambda: [launch(i) for i in range(iters)], use_graph) / iters
+        res[key] = {"spec": spec, "us": round(us, 3), "bytes": int(nbytes), "GBps": round(nbytes / us / 1e3, 1),
+                    "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        rt.unloadKernel(k)
+        for p in owned:
+            rt.cuFree(p)
+
+    for B in batches:
+        bp = f" batch={B}" if B != 1 else ""
+        q8 = B >= 8
+        x = rt.to_device(bf(g.standard_normal((B, H), dtype=np.float32)))
+        nw = rt.to_device(bf((g.standard_normal(H) * 0.1).astype(np.float32)))
+        resid = rt.to_device(bf(g.standard_normal((B, H), dtype=np.float32)))
+        # GDN layer projections: rmsnorm + qkv, z, a, b
+        (Wqkv, b0), (Wz, b1), (Wa, b2), (Wb, b3) = q4k(3 * Hg * 128, H), q4k(Hg * 128, H), q4k(Hg, H), q4k(Hg, H)
+        oq, oz, oa, ob = rt.cuAlloc(B * 3 * Hg * 128 * 2), rt.cuAlloc(B * Hg * 128 * 2), rt.cuAlloc(B * Hg * 4), rt.cuAlloc(B * Hg * 4)
+        time_op(f"gdn_projections_b{B}", f"gemv_fused K={H} pro=2 G=4 N0={3 * Hg * 128} epi0=1 N1={Hg * 128} epi1=1 N2={Hg} epi2=0 N3={Hg} epi3=0" + bp,
+                lambda i: [x, nw, Wqkv[i % ROT], oq, Wz[i % ROT], oz, Wa[i % ROT], oa, Wb[i % ROT], ob],
+                b0 + b1 + b2 + b3 + B * H * 2 + B * (4 * Hg * 128) * 2, Wqkv + Wz + Wa + Wb + [oa, ob])
+        # conv1d + GDN step (reads the projections' outputs)
+        C = 3 * Hg * 128
+        st = [rt.to_device(bf(g.standard_normal((B, 3, C), dtype=np.float32))) for _ in range(ROT)]
+        cw = rt.to_device(bf((g.standard_normal((C, 4)) * 0.5).astype(np.float32)))
+        A_log = rt.to_device(g.uniform(-2, 1, Hg).astype(np.float32)); dtb = rt.to_device(bf(g.standard_normal(Hg).astype(np.float32)))
+        ap = rt.to_device(g.standard_normal((B, Hg)).astype(np.float32)); bpp = rt.to_device(g.standard_normal((B, Hg)).astype(np.float32))
+        gw = rt.to_device((1 + 0.1 * g.standard_normal(128)).astype(np.float32))
+        S0 = (g.standard_normal((B, Hg, 128, 128), dtype=np.float32) * np.float32(0.02))
+        dS = [rt.to_device(S0) for _ in range(ROT)]
+        rt.cuHtoD(oq, bf(g.standard_normal((B, C), dtype=np.float32))); rt.cuHtoD(oz, bf(g.standard_normal((B, Hg * 128), dtype=np.float32)))
+        gout = rt.cuAlloc(B * Hg * 128 * 2); gq8 = rt.cuAlloc(B * Hg * 4 * 36)
+        time_op(f"gdn_conv_b{B}", f"gdn_conv LVH={Hg} LKD=128 LVD=128" + bp + (" q8out=1" if q8 else ""),
+                lambda i: [oq, st[i % ROT], cw, oz, A_log, dtb, ap, bpp, gw, dS[i % ROT], gout, st[i % ROT], dS[i % ROT]] + ([gq8] if q8 else []),
+                B * Hg * (2 * 128 * 128 * 4) + B * C * 2 * 7 + B * Hg * 128 * 4, st + dS + [cw, A_log, dtb, ap, bpp, gw, oq, oz])
+        # out_proj + residual add (reads the GDN output; batched: its Q8_1 copy)
+        Wo, bo = q4k(H, Hg * 128)
+        hout = rt.cuAlloc(B * H * 2)
+        time_op(f"out_proj_add_b{B}", f"gemv_fused K={Hg * 128} pro={0 if q8 else 1} G=1 N0={H} epi0=2" + bp,
+                lambda i: [gq8 if q8 else gout, Wo[i % ROT], resid, hout], bo + B * (Hg * 128 * 2 + 2 * H * 2), Wo + [gout, gq8])
+        # MLP: rmsnorm + gate, up + SwiGLU, then down + residual add
+        (Wg, bg), (Wu, bu), (Wd, bd) = q4k(I, H), q4k(I, H), q4k(H, I)
+        act = rt.cuAlloc(B * I * 2); aq8 = rt.cuAlloc(B * (I // 32) * 36)
+        time_op(f"gate_up_swiglu_b{B}", f"gemv_fused K={H} pro=2 G=2 swiglu=1 N0={I} N1={I}" + bp + (" q8out=1" if q8 else ""),
+                lambda i: [x, nw, Wg[i % ROT], Wu[i % ROT], act] + ([aq8] if q8 else []), bg + bu + B * (H + I) * 2, Wg + Wu)
+        time_op(f"down_add_b{B}", f"gemv_fused K={I} pro={0 if q8 else 1} G=1 N0={H} epi0=2" + bp,
+                lambda i: [aq8 if q8 else act, Wd[i % ROT], resid, hout], bd + B * (I * 2 + 2 * H * 2), Wd + [act, aq8])
+        # attention layer: rmsnorm + q|gate, k, v; norms + rope + append + attention over 4096 cached tokens; o_proj + add
+        (Wq, bq), (Wk, bk), (Wv, bv), (Wop, bop) = q4k(2 * NH * HD, H), q4k(NKV * HD, H), q4k(NKV * HD, H), q4k(H, NH * HD)
+        qg, kk, vv = rt.cuAlloc(B * 2 * NH * HD * 2), rt.cuAlloc(B * NKV * HD * 2), rt.cuAlloc(B * NKV * HD * 2)
+        time_op(f"attn_projections_b{B}", f"gemv_fused K={H} pro=2 G=3 N0={2 * NH * HD} epi0=1 N1={NKV * HD} epi1=1 N2={NKV * HD} epi2=1" + bp,
+                lambda i: [x, nw, Wq[i % ROT], qg, Wk[i % ROT], kk, Wv[i % ROT], vv], bq + bk + bv + B * H * 2 + B * (2 * NH + 2 * NKV) * HD * 2,
+                Wq + Wk + Wv)
+        for buf, n in ((qg, B * 2 * NH * HD), (kk, B * NKV * HD), (vv, B * NKV * HD)):
+            rt.cuHtoD(buf, bf(g.standard_normal(n, dtype=np.float32)))
+        page = bf(g.standard_normal((64, NKV, 16, HD), dtype=np.float32))
+        cache = np.tile(page, ((B * (MAXL // 16) + 63) // 64, 1, 1, 1))[: B * (MAXL // 16)]
+        NR = 6 if B == 1 else 3
+        kcs = [rt.to_device(cache) for _ in range(NR)]; vcs = [rt.to_device(cache) for _ in range(NR)]
+        cos_t = rt.to_device(g.uniform(-1, 1, (MAXL, 32)).astype(np.float32)); sin_t = rt.to_device(g.uniform(-1, 1, (MAXL, 32)).astype(np.float32))
+        qw = rt.to_device(bf((g.standard_normal(HD) * 0.1).astype(np.float32))); kw = rt.to_device(bf((g.standard_normal(HD) * 0.1).astype(np.float32)))
+        dpos = rt.to_device(np.full(B, POS, np.int32))
+        aout = rt.cuAlloc(B * NH * HD * 2); attq8 = rt.cuAlloc(B * (NH * HD // 32) * 36)
+        time_op(f"fa2_fused_b{B}_ctx{POS}", f"fa2_fused HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF=32 pos_dev=1" + bp + (" q8out=1" if q8 else ""),
+                lambda i: [qg, kk, vv, qw, kw, cos_t, sin_t, dpos, kcs[i % NR], vcs[i % NR], aout] + ([attq8] if q8 else []),
+                B * (2 * NKV * (POS + 1) * HD * 2 + (2 * NH + 2 * NKV + NH) * HD * 2), kcs + vcs + [cos_t, sin_t, qw, kw, dpos, qg, kk, vv])
+        time_op(f"o_proj_add_b{B}", f"gemv_fused K={NH * HD} pro={0 if q8 else 1} G=1 N0={H} epi0=2" + bp,
+                lambda i: [attq8 if q8 else aout, Wop[i % ROT], resid, hout], bop + B * (NH * HD * 2 + 2 * H * 2), Wop + [aout, attq8, hout])
+        for p in (x, nw, resid):
+            rt.cuFree(p)
+    return res
+
+
 MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 MFMA_F32_PEAK_TFLOPS = 157.3       # MI355X f32 matrix
 
@@ -576,9 +673,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sections", default="gemv,decode,kernels,gemm,load,tok",
-                    help="comma list of gemv (headline, always on), decode (with prefill), kernels, gemm, calib, load (weights path), "
-                         "tok (tokenizer, host only)")
+    ap.add_argument("--sections", default="gemv,decode,kernels,gemm,fused,load,tok",
+                    help="comma list of gemv (headline, always on), decode (with prefill), kernels, gemm, fused (the decode step's "
+                         "fused ops one by one), calib, load (weights path), tok (tokenizer, host only)")
     ap.add_argument("--mode", choices=["graph", "stream"], default="graph",
                     help="GEMV section. graph: the K launches of a shape replayed from one HIP graph (the device's own launch "
                          "rate); stream: K individual launches per shape queued from the host (used under rocprofv3)")
@@ -776,6 +873,8 @@ def main():
         out["kernels"] = bench_kernels(rt, synth, use_graph=not args.no_graph)
     if "gemm" in sections:
         out["gemm_bs32"] = bench_gemm(rt, synth, use_graph=not args.no_graph)
+    if "fused" in sections:
+        out["fused_ops"] = bench_fused_ops(rt, synth, use_graph=not args.no_graph)
     if "load" in sections:
         out["weights_path"] = bench_load(rt, synth)
     if "tok" in sections:
