@@ -544,31 +544,48 @@ def bench_fused_ops(rt, synth, use_graph=True, iters=48, batches=(1, 32)):
         x = rt.to_device(bf(g.standard_normal((B, H), dtype=np.float32)))
         nw = rt.to_device(bf((g.standard_normal(H) * 0.1).astype(np.float32)))
         resid = rt.to_device(bf(g.standard_normal((B, H), dtype=np.float32)))
-        # GDN layer projections: rmsnorm + qkv, z, a, b
-        (Wqkv, b0), (Wz, b1), (Wa, b2), (Wb, b3) = q4k(3 * Hg * 128, H), q4k(Hg * 128, H), q4k(Hg, H), q4k(Hg, H)
-        oq, oz, oa, ob = rt.cuAlloc(B * 3 * Hg * 128 * 2), rt.cuAlloc(B * Hg * 128 * 2), rt.cuAlloc(B * Hg * 4), rt.cuAlloc(B * Hg * 4)
-        time_op(f"gdn_projections_b{B}", f"gemv_fused K={H} pro=2 G=4 N0={3 * Hg * 128} epi0=1 N1={Hg * 128} epi1=1 N2={Hg} epi2=0 N3={Hg} epi3=0" + bp,
-                lambda i: [x, nw, Wqkv[i % ROT], oq, Wz[i % ROT], oz, Wa[i % ROT], oa, Wb[i % ROT], ob],
-                b0 + b1 + b2 + b3 + B * H * 2 + B * (4 * Hg * 128) * 2, Wqkv + Wz + Wa + Wb + [oa, ob])
-        # conv1d + GDN step (reads the projections' outputs)
+        # GDN layer.  Batch < 8 (slab form): rmsnorm + qkv (+ conv1d), z, a, b | recurrence in four column slabs per head,
+        # raw outputs | gated norm + out_proj + residual add.  Batched: rmsnorm + qkv, z, a, b | conv1d + recurrence |
+        # out_proj + add reading the recurrence's Q8_1 copy.
+        slab = not q8
         C = 3 * Hg * 128
+        (Wqkv, b0), (Wz, b1), (Wa, b2), (Wb, b3) = q4k(C, H), q4k(Hg * 128, H), q4k(Hg, H), q4k(Hg, H)
+        oq, oz, oa, ob = rt.cuAlloc(B * C * 2), rt.cuAlloc(B * Hg * 128 * 2), rt.cuAlloc(B * Hg * 4), rt.cuAlloc(B * Hg * 4)
         st = [rt.to_device(bf(g.standard_normal((B, 3, C), dtype=np.float32))) for _ in range(ROT)]
         cw = rt.to_device(bf((g.standard_normal((C, 4)) * 0.5).astype(np.float32)))
+        conv_bytes = B * C * 2 * 6 + C * 8         # three state rows in and out, the taps
+        if slab:
+            time_op(f"gdn_projections_conv_b{B}", f"gemv_fused K={H} pro=2 G=4 N0={C} epi0=3 N1={Hg * 128} epi1=1 N2={Hg} epi2=0 N3={Hg} epi3=0" + bp,
+                    lambda i: [x, nw, Wqkv[i % ROT], st[i % ROT], cw, oq, st[i % ROT], Wz[i % ROT], oz, Wa[i % ROT], oa, Wb[i % ROT], ob],
+                    b0 + b1 + b2 + b3 + B * H * 2 + B * (4 * Hg * 128) * 2 + conv_bytes, Wqkv + Wz + Wa + Wb + [oa, ob])
+        else:
+            time_op(f"gdn_projections_b{B}", f"gemv_fused K={H} pro=2 G=4 N0={C} epi0=1 N1={Hg * 128} epi1=1 N2={Hg} epi2=0 N3={Hg} epi3=0" + bp,
+                    lambda i: [x, nw, Wqkv[i % ROT], oq, Wz[i % ROT], oz, Wa[i % ROT], oa, Wb[i % ROT], ob],
+                    b0 + b1 + b2 + b3 + B * H * 2 + B * (4 * Hg * 128) * 2, Wqkv + Wz + Wa + Wb + [oa, ob])
         A_log = rt.to_device(g.uniform(-2, 1, Hg).astype(np.float32)); dtb = rt.to_device(bf(g.standard_normal(Hg).astype(np.float32)))
         ap = rt.to_device(g.standard_normal((B, Hg)).astype(np.float32)); bpp = rt.to_device(g.standard_normal((B, Hg)).astype(np.float32))
         gw = rt.to_device((1 + 0.1 * g.standard_normal(128)).astype(np.float32))
         S0 = (g.standard_normal((B, Hg, 128, 128), dtype=np.float32) * np.float32(0.02))
         dS = [rt.to_device(S0) for _ in range(ROT)]
         rt.cuHtoD(oq, bf(g.standard_normal((B, C), dtype=np.float32))); rt.cuHtoD(oz, bf(g.standard_normal((B, Hg * 128), dtype=np.float32)))
-        gout = rt.cuAlloc(B * Hg * 128 * 2); gq8 = rt.cuAlloc(B * Hg * 4 * 36)
-        time_op(f"gdn_conv_b{B}", f"gdn_conv LVH={Hg} LKD=128 LVD=128" + bp + (" q8out=1" if q8 else ""),
-                lambda i: [oq, st[i % ROT], cw, oz, A_log, dtb, ap, bpp, gw, dS[i % ROT], gout, st[i % ROT], dS[i % ROT]] + ([gq8] if q8 else []),
-                B * Hg * (2 * 128 * 128 * 4) + B * C * 2 * 7 + B * Hg * 128 * 4, st + dS + [cw, A_log, dtb, ap, bpp, gw, oq, oz])
-        # out_proj + residual add (reads the GDN output; batched: its Q8_1 copy)
+        gout = rt.cuAlloc(B * Hg * 128 * 2); gq8 = rt.cuAlloc(B * Hg * 4 * 36); graw = rt.cuAlloc(B * (Hg * 128 * 8 + Hg * 32))
+        state_bytes = B * Hg * (2 * 128 * 128 * 4)
+        if slab:
+            time_op(f"gdn_slabs_b{B}", f"gdn_slabs LVH={Hg} LKD=128 LVD=128" + bp,
+                    lambda i: [oq, oz, A_log, dtb, ap, bpp, dS[i % ROT], graw, dS[i % ROT]],
+                    state_bytes + B * (C * 2 + Hg * 128 * 2 + Hg * 128 * 8 + Hg * 32), dS + st + [cw, A_log, dtb, ap, bpp, oq, oz])
+        else:
+            time_op(f"gdn_conv_b{B}", f"gdn_conv LVH={Hg} LKD=128 LVD=128" + bp + " q8out=1",
+                    lambda i: [oq, st[i % ROT], cw, oz, A_log, dtb, ap, bpp, gw, dS[i % ROT], gout, st[i % ROT], dS[i % ROT], gq8],
+                    state_bytes + B * C * 2 + conv_bytes + B * Hg * 128 * 4, st + dS + [cw, A_log, dtb, ap, bpp, oq, oz])
         Wo, bo = q4k(H, Hg * 128)
         hout = rt.cuAlloc(B * H * 2)
-        time_op(f"out_proj_add_b{B}", f"gemv_fused K={Hg * 128} pro={0 if q8 else 1} G=1 N0={H} epi0=2" + bp,
-                lambda i: [gq8 if q8 else gout, Wo[i % ROT], resid, hout], bo + B * (Hg * 128 * 2 + 2 * H * 2), Wo + [gout, gq8])
+        if slab:
+            time_op(f"out_proj_gated_norm_add_b{B}", f"gemv_fused K={Hg * 128} pro=3 G=1 N0={H} epi0=2" + bp,
+                    lambda i: [graw, gw, Wo[i % ROT], resid, hout], bo + B * (Hg * 128 * 8 + 2 * H * 2), Wo + [gout, gq8, graw, gw])
+        else:
+            time_op(f"out_proj_add_b{B}", f"gemv_fused K={Hg * 128} pro=0 G=1 N0={H} epi0=2" + bp,
+                    lambda i: [gq8, Wo[i % ROT], resid, hout], bo + B * (Hg * 128 * 2 + 2 * H * 2), Wo + [gout, gq8, graw, gw])
         # MLP: rmsnorm + gate, up + SwiGLU, then down + residual add
         (Wg, bg), (Wu, bu), (Wd, bd) = q4k(I, H), q4k(I, H), q4k(H, I)
         act = rt.cuAlloc(B * I * 2); aq8 = rt.cuAlloc(B * (I // 32) * 36)

@@ -108,10 +108,12 @@ static int run_gemm(Kernel& k, const uint64_t* s) {
 
 // ---- op: gemv_fused — rmsnorm / quantize + up to four matmuls over one activation + their cast / add / swiglu
 // consumers (src/model.ts:65-73, 161-191 as one launch; the node-by-node result to the bit).
-// params: K, pro (0: x is Q8_1, 1: x is bf16, 2: x is bf16 and goes through rmsnorm with norm_w first),
-//         G matrices with N<i>, epi<i> (0: f32, 1: bf16, 2: bf16(bf16(y) + residual)), swiglu=0|1 (G=2: gate, up), batch=1
-// slots:  x, [norm_w if pro=2], then per matrix: W, [residual if epi=2], out      (swiglu: x, [norm_w], Wg, Wu, out
-//         [, out as Q8_1 blocks when q8out=1: batch >= 8 only])
+// params: K, pro (0: x is Q8_1, 1: x is bf16, 2: x is bf16 and goes through rmsnorm with norm_w first, 3: x is the raw
+//         block of a gdn_slabs op and goes through that op's gated RMS norm with norm_w (f32 [128]) first: K = 2048, batch < 8),
+//         G matrices with N<i>, epi<i> (0: f32, 1: bf16, 2: bf16(bf16(y) + residual), 3 (matrix 0, pro=2, K = 1024 or
+//         2048, batch < 8): bf16, then conv1d_decode over the N0 channels), swiglu=0|1 (G=2: gate, up), batch=1
+// slots:  x, [norm_w if pro=2|3], then per matrix: W, [residual if epi=2 | conv_state_in, conv_w if epi=3], out,
+//         [conv_state_new if epi=3]      (swiglu: x, [norm_w], Wg, Wu, out [, out as Q8_1 blocks when q8out=1: batch >= 8 only])
 // Shapes outside the fused kernel (K other than 1024, 2048, 3584, 4096, 6144, or batch >= 8) run as rmsnorm/quantize,
 // matmuls, swiglu.
 static int run_gemv_fused(Kernel& k, const uint64_t* s) {
@@ -119,8 +121,9 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
   const bool swiglu = k.get("swiglu", 0) != 0;
   int si = 0;
   const void* x = P<void>(s[si++]);
-  const void* nw = pro == 2 ? P<void>(s[si++]) : nullptr;
+  const void* nw = (pro == 2 || pro == 3) ? P<void>(s[si++]) : nullptr;
   const void* W[4] = {}; void* out[4] = {}; const void* res[4] = {}; int N[4] = {}, epi[4] = {};
+  FusedConv conv{};
   char key[16];
   for (int i = 0; i < G; i++) {
     snprintf(key, sizeof key, "N%d", i); N[i] = (int)k.get(key, 0);
@@ -128,11 +131,13 @@ static int run_gemv_fused(Kernel& k, const uint64_t* s) {
     W[i] = P<void>(s[si++]);
     if (swiglu) continue;
     if (epi[i] == 2) res[i] = P<void>(s[si++]);
+    if (epi[i] == 3) { conv.st = P<void>(s[si]); conv.w = P<void>(s[si + 1]); si += 2; }
     out[i] = P<void>(s[si++]);
+    if (epi[i] == 3) conv.st_new = P<void>(s[si++]);
   }
   if (swiglu) out[0] = P<void>(s[si++]);
   void* q8out = swiglu && k.get("q8out", 0) ? P<void>(s[si++]) : nullptr;      // composed path only (build_gemv_fused checks)
-  if (gemv_fused_fast_path(K, batch, swiglu)) return launch_gemv_fused(pro, x, nw, K, batch, G, W, out, res, N, epi, swiglu);
+  if (gemv_fused_fast_path(K, batch, swiglu)) return launch_gemv_fused(pro, x, nw, K, batch, G, W, out, res, N, epi, swiglu, conv.st ? &conv : nullptr);
   int rc;
   const void* xq = x;
   // The GDN layers' projections at hidden size 2048: qkv and z are 256 tiles of the batched matmul, one per CU with eight
@@ -175,9 +180,11 @@ static int build_gemv_fused(Kernel& k) {
   const int64_t K = k.get("K", 0), pro = k.get("pro", 0), G = k.get("G", 1), batch = k.get("batch", 1);
   const bool swiglu = k.get("swiglu", 0) != 0;
   BK_REQUIRE(K > 0 && K % 256 == 0, "gemv_fused: K=%lld must be a positive multiple of 256", (long long)K);
-  BK_REQUIRE(pro >= 0 && pro <= 2 && G >= 1 && G <= 4 && batch >= 1 && batch <= 4096, "gemv_fused: bad pro/G/batch");
+  BK_REQUIRE(pro >= 0 && pro <= 3 && G >= 1 && G <= 4 && batch >= 1 && batch <= 4096, "gemv_fused: bad pro/G/batch");
+  BK_REQUIRE(pro != 3 || (K == 2048 && !swiglu && gemv_fused_fast_path((int)K, (int)batch, false)),
+             "gemv_fused: pro=3 (gated norm of a gdn_slabs block) serves K = 2048 at batch < 8");
   BK_REQUIRE(!swiglu || G == 2, "gemv_fused: swiglu needs G=2 (gate, up)");
-  int nslots = 1 + (pro == 2 ? 1 : 0);
+  int nslots = 1 + (pro >= 2 ? 1 : 0);
   char key[16];
   for (int i = 0; i < G; i++) {
     snprintf(key, sizeof key, "N%d", i);
@@ -186,8 +193,9 @@ static int build_gemv_fused(Kernel& k) {
     BK_REQUIRE(!swiglu || k.get(key, 0) % 4 == 0, "gemv_fused: swiglu needs N to be a multiple of 4");
     snprintf(key, sizeof key, "epi%d", i);
     const int64_t e = k.get(key, 0);
-    BK_REQUIRE(e >= 0 && e <= 2, "gemv_fused: bad %s", key);
-    nslots += swiglu ? 1 : (e == 2 ? 3 : 2);
+    BK_REQUIRE((e >= 0 && e <= 2) || (e == 3 && i == 0 && pro == 2 && !swiglu && (K == 2048 || K == 1024) && gemv_fused_fast_path((int)K, (int)batch, false)),
+               "gemv_fused: bad %s (3 = conv1d behind matrix 0 of an rmsnorm group with K = 1024 or 2048 at batch < 8)", key);
+    nslots += swiglu ? 1 : (e == 2 ? 3 : (e == 3 ? 5 : 2));
   }
   if (swiglu) nslots += 1;
   if (k.get("q8out", 0)) {
@@ -245,6 +253,14 @@ static int run_gdn_conv(Kernel& k, const uint64_t* s) {
                                P<float>(s[6]), P<float>(s[7]), P<float>(s[8]), P<float>(s[9]), P<void>(s[10]), P<void>(s[11]),
                                P<float>(s[12]), k.get("q8out", 0) ? P<void>(s[13]) : nullptr, (int)k.get("LVH", 0),
                                (int)k.get("batch", 1));
+}
+// ---- op: gdn_slabs = gdn_delta_rule without its gated norm, four column slabs per head (few sequences: every slab on
+// a CU of its own).  The raw outputs go to `raw` (per sequence: f32 o[LVH*128] | f32 z*sigmoid(z)[LVH*128] | f64 sum of
+// o^2 per (head, slab)), which the out_proj matmul's prologue turns into the op's output (gemv_fused pro=3).
+// slots: conv_out, z, A_log, dt_bias, a_p, b_p, s_state_in, raw, s_state_new      params: LVH, batch=1
+static int run_gdn_slabs(Kernel& k, const uint64_t* s) {
+  return launch_gdn_slabs(P<void>(s[0]), P<void>(s[1]), P<float>(s[2]), P<void>(s[3]), P<float>(s[4]), P<float>(s[5]), P<float>(s[6]),
+                          P<void>(s[7]), P<float>(s[8]), (int)k.get("LVH", 0), (int)k.get("batch", 1));
 }
 // ---- ops: qnorm (q-gate buffer, w, out; NH heads, input rows 2*HD apart), knorm (k, w, out; NKV heads)
 static int run_qnorm(Kernel& k, const uint64_t* s) {
@@ -393,7 +409,7 @@ static int build_kernel(Kernel& k) {
       {"rmsnorm_q8_1", run_rmsnorm_q8, 4, "N", nullptr}, {"cast", run_cast, 2, "N", nullptr},
       {"add", run_add, 3, "N", nullptr},            {"swiglu", run_swiglu, 3, "N", nullptr},
       {"conv1d_decode", run_conv1d, 5, "QKVD", nullptr}, {"gdn_delta_rule", run_gdn, 10, "LVH", nullptr},
-      {"gdn_conv", run_gdn_conv, 13, "LVH", nullptr},
+      {"gdn_conv", run_gdn_conv, 13, "LVH", nullptr},   {"gdn_slabs", run_gdn_slabs, 9, "LVH", nullptr},
       {"qnorm", run_qnorm, 3, "HD", "NH"},          {"knorm", run_knorm, 3, "HD", "NKV"},
       {"rope", run_rope, 4, "HD", "NH"},            {"ropek", run_rope, 4, "HD", "NKV"},
       {"advance", run_advance, 6, "batch", "max_steps"},
@@ -406,7 +422,7 @@ static int build_kernel(Kernel& k) {
       if ((rc = need(k, "ROT_HALF")) || (rc = need(k, "MAX_LEN"))) return rc;
     }
     if (k.op == "advance" && (rc = need(k, "max_pos"))) return rc;
-    if (k.op == "gdn_delta_rule" || k.op == "gdn_conv")
+    if (k.op == "gdn_delta_rule" || k.op == "gdn_conv" || k.op == "gdn_slabs")
       BK_REQUIRE(k.get("LKD", 128) == 128 && k.get("LVD", 128) == 128, "gdn_delta_rule: dk = dv = 128 only");
     k.run = sp.run; k.nslots = sp.nslots + (k.op == "gdn_conv" && k.get("q8out", 0) ? 1 : 0);
     return BK_OK;

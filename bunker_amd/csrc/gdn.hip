@@ -229,6 +229,117 @@ __global__ __launch_bounds__(GDN_THREADS) void gdn_step_kernel(GdnArgs A) {
   }
 }
 
+// Column-slab form of the fused step for few (sequence, head) pairs, where one 256-thread workgroup per head leaves most
+// of the chip idle and its one CU fetches all 64 KiB of the head's state: a head is cut into four slabs of 32 columns,
+// one wavefront each.  Lane (kg = lane / 8, vq = lane % 8) owns rows 16 kg .. 16 kg + 15 and four columns of the slab,
+// so both k-reductions keep the canonical order (fmaf chains over 16 consecutive rows, then the 8 chain results in
+// order) and S' and o have the bits of the one-workgroup form.  Every slab works out the head's norms and gates itself
+// (the inputs are convolved already: the projection in front of this launch applies conv1d in its last step).  What needs
+// the whole head - the gated RMS norm - moves into the matmul behind it: a slab leaves its 32 raw outputs o (f32), the
+// output gate z * sigmoid(z) (f32) and the sum of o^2 over its columns (f64) in `raw`:
+//   raw, per sequence: f32 o[Hg * 128] | f32 zs[Hg * 128] | f64 ssq[Hg][4]
+struct GdnRawLayout {
+  int Hg;
+  __host__ __device__ size_t floats() const { return (size_t)Hg * GDN_D * 2; }
+  __host__ __device__ size_t bytes() const { return floats() * 4 + (size_t)Hg * 4 * 8; }
+};
+template <bool NT>
+__global__ __launch_bounds__(64) void gdn_slab_kernel(GdnArgs A, uint8_t* __restrict__ raw_base) {
+  constexpr int CS = 4, COLS = GDN_D / CS, KG = 8, ROWS = 16;
+  __shared__ float kn[GDN_D], qn[GDN_D];
+  __shared__ float part[KG][COLS];
+  const int h = blockIdx.x, slab = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+  const int vq = lane & 7, kg = lane >> 3;
+  const int col0 = slab * COLS + vq * 4;
+  const int64_t bh = (int64_t)b * A.Hg + h;
+  const uint16_t* qp = A.q + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* kp = A.k + (int64_t)b * A.qkv_bstride + h * GDN_D;
+  const uint16_t* vp = A.v + (int64_t)b * A.qkv_bstride + h * GDN_D;
+
+  // small operands first, the 16 KiB of S right behind them (loads return in order)
+  const uint32_t q2 = *(const uint32_t*)(qp + 2 * lane), k2 = *(const uint32_t*)(kp + 2 * lane);
+  const uint2 vv = *(const uint2*)(vp + col0);
+  const float ap = A.a_p[bh], bp = A.b_p[bh], alog = A.A_log[h], dtb = bf16_to_f32(A.dt_bias[h]);
+  const float zin = bf16_to_f32(A.z[bh * GDN_D + slab * COLS + (lane & 31)]);
+  const float* Sp = A.S_in + bh * GDN_D * GDN_D;
+  float4 S[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    const f32x4_nt* sp = (const f32x4_nt*)(Sp + (int64_t)(kg * ROWS + r) * GDN_D + col0);
+    const f32x4_nt t = NT ? __builtin_nontemporal_load(sp) : *sp;
+    S[r] = make_float4(t[0], t[1], t[2], t[3]);
+  }
+
+  const float q0 = __uint_as_float(q2 << 16), q1 = __uint_as_float(q2 & 0xffff0000u);
+  const float k0 = __uint_as_float(k2 << 16), k1 = __uint_as_float(k2 & 0xffff0000u);
+  const double ssq = wave_sum_f64((double)(q0 * q0) + (double)(q1 * q1));      // squares of bf16 values: exact in f32
+  const double ssk = wave_sum_f64((double)(k0 * k0) + (double)(k1 * k1));
+  const float rq = rsqrt_f64(ssq + 1e-6) * 0.08838834764831845f, rk = rsqrt_f64(ssk + 1e-6);
+  qn[2 * lane] = q0 * rq; qn[2 * lane + 1] = q1 * rq;
+  kn[2 * lane] = k0 * rk; kn[2 * lane + 1] = k1 * rk;
+  const float sp_in = ap + dtb;
+  const float softplus = (float)log1p(exp((double)sp_in));
+  const float decay = (float)exp(-(double)((float)exp((double)alog) * softplus));
+  const float beta = sigmoid_f64(bp);
+  const float zs = zin * sigmoid_f64(zin);
+  __syncthreads();
+
+  float kr[ROWS], qr[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) { kr[r] = kn[kg * ROWS + r]; qr[r] = qn[kg * ROWS + r]; }
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    S[r].x *= decay; S[r].y *= decay; S[r].z *= decay; S[r].w *= decay;
+    acc.x = fmaf(kr[r], S[r].x, acc.x); acc.y = fmaf(kr[r], S[r].y, acc.y);
+    acc.z = fmaf(kr[r], S[r].z, acc.z); acc.w = fmaf(kr[r], S[r].w, acc.w);
+  }
+  *(float4*)&part[kg][vq * 4] = acc;
+  __syncthreads();
+  float4 pk[KG];
+#pragma unroll
+  for (int j = 0; j < KG; j++) pk[j] = *(const float4*)&part[j][vq * 4];
+  __builtin_amdgcn_sched_barrier(0);
+  float4 kS = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int j = 0; j < KG; j++) { kS.x += pk[j].x; kS.y += pk[j].y; kS.z += pk[j].z; kS.w += pk[j].w; }
+  __syncthreads();   // part is reused for o below
+  float4 d;
+  d.x = (__uint_as_float(vv.x << 16) - kS.x) * beta;
+  d.y = (__uint_as_float(vv.x & 0xffff0000u) - kS.y) * beta;
+  d.z = (__uint_as_float(vv.y << 16) - kS.z) * beta;
+  d.w = (__uint_as_float(vv.y & 0xffff0000u) - kS.w) * beta;
+
+  float* So = A.S_out + bh * GDN_D * GDN_D;
+  acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    S[r].x = fmaf(kr[r], d.x, S[r].x); S[r].y = fmaf(kr[r], d.y, S[r].y);
+    S[r].z = fmaf(kr[r], d.z, S[r].z); S[r].w = fmaf(kr[r], d.w, S[r].w);
+    {
+      f32x4_nt* sp = (f32x4_nt*)(So + (int64_t)(kg * ROWS + r) * GDN_D + col0);
+      const f32x4_nt t = {S[r].x, S[r].y, S[r].z, S[r].w};
+      if (NT) __builtin_nontemporal_store(t, sp); else *sp = t;
+    }
+    acc.x = fmaf(qr[r], S[r].x, acc.x); acc.y = fmaf(qr[r], S[r].y, acc.y);
+    acc.z = fmaf(qr[r], S[r].z, acc.z); acc.w = fmaf(qr[r], S[r].w, acc.w);
+  }
+  *(float4*)&part[kg][vq * 4] = acc;
+  __syncthreads();
+  // lanes 0..31 and 32..63 both sum column lane % 32 (the same bits); the sum of squares then covers each column twice
+  float o = 0.0f;
+#pragma unroll
+  for (int j = 0; j < KG; j++) o += part[j][lane & 31];
+  const double oss = wave_sum_f64(lane < 32 ? (double)o * (double)o : 0.0);
+  const GdnRawLayout L{A.Hg};
+  float* rawf = (float*)(raw_base + (size_t)b * L.bytes());
+  if (lane < 32) {
+    rawf[h * GDN_D + slab * COLS + lane] = o;
+    rawf[A.Hg * GDN_D + h * GDN_D + slab * COLS + lane] = zs;
+  }
+  if (lane == 0) ((double*)(rawf + L.floats()))[h * 4 + slab] = oss;
+}
+
 int g_tune_gdn_cs = 0;    // column slabs per head for the core entry point (0 = from the shape)
 int g_tune_gdn_nt = -1;   // state through nontemporal loads and stores: 0 off, 1 on, -1 = from the shape
 
@@ -277,6 +388,28 @@ int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv
   const bool nt = g_tune_gdn_nt >= 0 ? g_tune_gdn_nt != 0 : (int64_t)Hg * batch >= 128;
   if (nt) hipLaunchKernelGGL((gdn_step_kernel<1, true, true, true>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
   else hipLaunchKernelGGL((gdn_step_kernel<1, true, true, false>), dim3(Hg, 1, batch), dim3(GDN_THREADS), 0, stream(), A);
+  BK_LAUNCH_CHECK();
+  return BK_OK;
+}
+
+size_t gdn_raw_bytes(int Hg, int batch) { return GdnRawLayout{Hg}.bytes() * (size_t)batch; }
+
+// gdn_delta_rule without its gated norm, in column slabs (see gdn_slab_kernel): conv_out is [q | k | v] bf16 after conv1d
+int launch_gdn_slabs(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
+                     const float* b_p, const float* S_in, void* raw, float* S_out, int Hg, int batch) {
+  GdnArgs A{};
+  const int KEYDIM = Hg * GDN_D;
+  A.q = (const uint16_t*)conv_out; A.k = A.q + KEYDIM; A.v = A.q + 2 * KEYDIM;
+  A.qkv_bstride = 3 * (int64_t)KEYDIM;
+  A.z = (const uint16_t*)z; A.A_log = A_log; A.dt_bias = (const uint16_t*)dt_bias; A.a_p = a_p; A.b_p = b_p;
+  A.S_in = S_in; A.S_out = S_out; A.out = (uint16_t*)raw; A.Hg = Hg;
+  BK_REQUIRE(conv_out && z && A_log && dt_bias && a_p && b_p && raw, "gdn_slabs: null pointer");
+  BK_REQUIRE(((uintptr_t)raw & 15) == 0 && ((uintptr_t)conv_out & 3) == 0, "gdn_slabs: raw must be 16-byte aligned, conv_out 4-byte aligned");
+  int rc = check_common(A, batch);
+  if (rc) return rc;
+  const bool nt = g_tune_gdn_nt >= 0 ? g_tune_gdn_nt != 0 : (int64_t)Hg * batch >= 128;
+  if (nt) hipLaunchKernelGGL((gdn_slab_kernel<true>), dim3(Hg, 4, batch), dim3(64), 0, stream(), A, (uint8_t*)raw);
+  else hipLaunchKernelGGL((gdn_slab_kernel<false>), dim3(Hg, 4, batch), dim3(64), 0, stream(), A, (uint8_t*)raw);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

@@ -21,7 +21,16 @@
 
 namespace bk {
 
-enum : int { PRO_Q8 = 0, PRO_BF16 = 1, PRO_RMSNORM = 2 };
+// PRO_GNORM: the activation is the raw output of the column-slab GDN step (gdn.hip gdn_slab_kernel) and goes through
+// that op's gated RMS norm first (src/emitters.ts:110-118): per head of 128, o * rsqrt(mean(o^2) + 1e-6) * norm_w * (z *
+// sigmoid(z)) -> bf16, with the sum of squares taken from the four slab sums the step left (added as (s0 + s1) + (s2 +
+// s3): the association of the one-workgroup form's block reduction, so the bits agree).
+enum : int { PRO_Q8 = 0, PRO_BF16 = 1, PRO_RMSNORM = 2, PRO_GNORM = 3 };
+// EPI_CONV (matrix 0 only): the row's bf16 output is channel `row` of conv1d_decode's input and goes through the 4-tap
+// causal convolution + SiLU at once (src/emitters.ts:48-72): out = bf16(r * sigmoid(r)), r = (w0 s0 + w1 s1) + (w2 s2 +
+// w3 x), and the channel's state rows become (s1, s2, x).  The lane that read a channel's rows rewrites them, so the
+// state may be updated in place.
+enum : int { EPI_CONV = 3 };
 
 struct FusedGroup {
   const uint8_t* W;
@@ -33,9 +42,95 @@ struct FusedArgs {
   FusedGroup g[4];
   int step_first[5];     // first step of each matrix; step_first[i >= ngroups] = total steps
   int ngroups;
-  const void* x;         // PRO_Q8: Q8_1 [batch, K/32 blocks]; else bf16 [batch, K]
-  const uint16_t* norm_w;
+  const void* x;         // PRO_Q8: Q8_1 [batch, K/32 blocks]; PRO_GNORM: the GDN step's raw block per sequence; else bf16 [batch, K]
+  const uint16_t* norm_w; // PRO_RMSNORM: bf16 [K]; PRO_GNORM: f32 [128]
 };
+// What only the conv-epilogue and gated-norm forms read.  Kept out of FusedArgs: with these 32 bytes in every kernel's
+// argument block the other forms measured 0.2-0.4 us slower per launch (19 us over a decode step).
+struct FusedArgsX : FusedArgs {
+  // EPI_CONV: conv state bf16 [batch, 3, C] (in, new; may alias), taps bf16 [C, 4]; C = rows of matrix 0
+  const uint16_t* conv_st;
+  uint16_t* conv_st_new;
+  const uint16_t* conv_w;
+  int64_t x_bstride;     // PRO_GNORM: bytes between two sequences' raw blocks
+};
+
+// A launch with one matrix (out_proj, o_proj, down, lm_head: half of the decode step's launches) gets its arguments in
+// 64 bytes instead of 168: the kernel's first instructions wait for the argument block, and a block that spans fewer
+// cache lines arrives sooner.  The kernel works on the full form, rebuilt in registers.
+struct FusedArgs1 {
+  FusedGroup g0;
+  const void* x;
+  const uint16_t* norm_w;
+  int64_t x_bstride;
+  int steps, pad;
+};
+__device__ __forceinline__ const FusedArgs& fused_args_full(const FusedArgs& A) { return A; }
+__device__ __forceinline__ const FusedArgsX& fused_args_full(const FusedArgsX& A) { return A; }
+__device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs1& P) {
+  FusedArgsX A;
+  A.g[0] = P.g0; A.g[1] = P.g0; A.g[2] = P.g0; A.g[3] = P.g0;
+  A.step_first[0] = 0; A.step_first[1] = P.steps; A.step_first[2] = P.steps; A.step_first[3] = P.steps; A.step_first[4] = P.steps;
+  A.ngroups = 1; A.x = P.x; A.norm_w = P.norm_w;
+  A.conv_st = nullptr; A.conv_st_new = nullptr; A.conv_w = nullptr; A.x_bstride = P.x_bstride;
+  return A;
+}
+
+// The operands of one channel of the convolution, requested ahead of the step's arithmetic
+struct ConvRegs {
+  uint16_t s0, s1, s2;
+  uint2 w;
+};
+__device__ __forceinline__ void conv_regs_load(ConvRegs& c, const FusedArgsX& A, int bidx, int C, int ch) {
+  ch = min(ch, C - 1);
+  const uint16_t* sb = A.conv_st + (int64_t)bidx * 3 * C;
+  c.s0 = sb[ch]; c.s1 = sb[C + ch]; c.s2 = sb[2 * C + ch];
+  c.w = *(const uint2*)(A.conv_w + 4 * (int64_t)ch);
+}
+__device__ __forceinline__ uint16_t conv_regs_apply(const ConvRegs& c, const FusedArgsX& A, int bidx, int C, int ch, uint16_t x) {
+  const float w0 = __uint_as_float(c.w.x << 16), w1 = __uint_as_float(c.w.x & 0xffff0000u);
+  const float w2 = __uint_as_float(c.w.y << 16), w3 = __uint_as_float(c.w.y & 0xffff0000u);
+  // products of two bf16 values are exact in f32
+  const float r = __fadd_rn(__fadd_rn(w0 * bf16_to_f32(c.s0), w1 * bf16_to_f32(c.s1)),
+                            __fadd_rn(w2 * bf16_to_f32(c.s2), w3 * bf16_to_f32(x)));
+  uint16_t* nb = A.conv_st_new + (int64_t)bidx * 3 * C;
+  nb[ch] = c.s1; nb[C + ch] = c.s2; nb[2 * C + ch] = x;
+  return f32_to_bf16(__fmul_rn(r, sigmoid_f64(r)));
+}
+
+// PRO_GNORM: what a thread holds of the raw block: 8 outputs, their gates, the norm weights, the head's four slab sums
+struct GnormRegs {
+  float4 o[2], zs[2], nw[2];
+  double2 ss[2];
+};
+__device__ __forceinline__ void gnorm_load(GnormRegs& r, const uint8_t* __restrict__ raw, const float* __restrict__ norm_w, int K) {
+  const int i = threadIdx.x * 8;                       // K = 2048: one pass of 256 threads x 8 elements
+  const float* o = (const float*)raw;
+  const float* zs = o + K;
+  const double* ss = (const double*)(zs + K);
+  r.o[0] = *(const float4*)(o + i); r.o[1] = *(const float4*)(o + i + 4);
+  r.zs[0] = *(const float4*)(zs + i); r.zs[1] = *(const float4*)(zs + i + 4);
+  r.nw[0] = *(const float4*)(norm_w + (i & 127)); r.nw[1] = *(const float4*)(norm_w + (i & 127) + 4);
+  r.ss[0] = *(const double2*)(ss + (i >> 7) * 4); r.ss[1] = *(const double2*)(ss + (i >> 7) * 4 + 2);
+}
+__device__ __forceinline__ void stage_gnorm(const GnormRegs& g, uint8_t* lds_xq) {
+  const double tot = (g.ss[0].x + g.ss[0].y) + (g.ss[1].x + g.ss[1].y);
+  const float orstd = rsqrt_f64(tot / 128.0 + 1e-6);
+  const float o[8] = {g.o[0].x, g.o[0].y, g.o[0].z, g.o[0].w, g.o[1].x, g.o[1].y, g.o[1].z, g.o[1].w};
+  const float z[8] = {g.zs[0].x, g.zs[0].y, g.zs[0].z, g.zs[0].w, g.zs[1].x, g.zs[1].y, g.zs[1].z, g.zs[1].w};
+  const float w[8] = {g.nw[0].x, g.nw[0].y, g.nw[0].z, g.nw[0].w, g.nw[1].x, g.nw[1].y, g.nw[1].z, g.nw[1].w};
+  float f[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) f[j] = bf16_to_f32(f32_to_bf16(__fmul_rn(__fmul_rn(__fmul_rn(o[j], orstd), w[j]), z[j])));
+  uint32_t pk[2];
+  const uint32_t ds = quad_q8_1(f, pk);
+  const int i = threadIdx.x * 8;
+  uint8_t* ob = lds_xq + (i / 32) * 36;
+  uint32_t* oq = (uint32_t*)(ob + (i & 31));
+  oq[0] = pk[0]; oq[1] = pk[1];
+  if ((i & 31) == 0) *(uint32_t*)(ob + 32) = ds;
+  __syncthreads();
+}
 
 // What a step needs to know about its matrix (all wave-uniform).
 struct StepSel {
@@ -175,14 +270,17 @@ __device__ __forceinline__ void fused_stage_park(const FusedStage<KB, RPI>& g, u
 
 // KB = super-blocks per row (K = 256 * KB).  Lane (b, c) folds super-block 8r + b in pass r; when KB is not a multiple of 8
 // the lanes past the row in the last pass read a clamped block and an all-zero activation slice, which adds exact zeros.
-template <int KB, int RPI, int PRO, bool SWIGLU>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A) {
+template <int KB, int RPI, int PRO, bool SWIGLU, bool CONV = false, typename ARGS = FusedArgs>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) {
+  const auto& A = fused_args_full(A_in);
+  static_assert(!CONV || (!SWIGLU && RPI == 4 && PRO == PRO_RMSNORM), "the conv epilogue exists for the form the decode step asks for");
   constexpr int NR = (KB + 7) / 8;
   constexpr int RP = KB * 9;                 // 16-byte pieces per row
   constexpr int PIECES = RPI * RP;
   constexpr int K = KB * 256;
   constexpr int ROWS_PER_STEP = SWIGLU ? RPI / 2 : RPI;
   __shared__ uint4 tiles[GEMV_WAVES][PIECES];
+  static_assert(PRO != PRO_GNORM || KB == 8, "the gated-norm prologue is written for rows of 2048 (16 heads of 128)");
   __shared__ __align__(16) uint8_t lds_xq[PRO == PRO_Q8 ? 16 : (K / 32) * 36];
   __shared__ double lds_red[4];
 
@@ -196,14 +294,21 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
   const int total = A.step_first[4];
   uint4* tile = tiles[wv];
 
-  ActRegs<KB> act;
-  if (PRO != PRO_Q8) act_load<PRO, KB>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
+  [[maybe_unused]] ActRegs<KB> act;
+  [[maybe_unused]] GnormRegs gn;
+  if constexpr (PRO == PRO_GNORM) gnorm_load(gn, (const uint8_t*)A.x + (int64_t)bidx * A.x_bstride, (const float*)A.norm_w, K);
+  else if constexpr (PRO != PRO_Q8) act_load<PRO, KB>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
 
   int s = blockIdx.x * GEMV_WAVES + wv;
   StepSel cur = select_step<ROWS_PER_STEP>(A, s < total ? s : 0);
   FusedStage<KB, RPI> g;
   // unconditional (a wave without a step of its own requests step 0): with a branch around these loads the
   // prologue's first wait could not be counted and would drain the weight rows as well
+  // EPI_CONV: the channel's state rows and taps, requested ahead of the weight rows (they come from L2 and are back
+  // long before the step's dots are folded); lanes 0..RPI-1 hold the step's rows
+  const int rl_conv = 2 * (lane & 1) + ((lane >> 1) & 1);
+  [[maybe_unused]] ConvRegs cr, crn;       // touched only by the CONV form (unused, they would end up as LDS-backed arrays)
+  if constexpr (CONV) conv_regs_load(cr, A, bidx, A.g[0].N, cur.row0 + rl_conv);      // unconditional: rows of the other matrices read a clamped channel
   fused_stage_load<KB, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
 
   XQ x[NR];
@@ -212,7 +317,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
 #pragma unroll
     for (int r = 0; r < NR; r++) load_xq(x[r], xq, r * 8 + b, c, (r + 1) * 8 <= KB || r * 8 + b < KB);
   } else {
-    stage_activation<PRO, KB>(act, lds_xq, lds_red);
+    if constexpr (PRO == PRO_GNORM) stage_gnorm(gn, lds_xq);
+    else stage_activation<PRO, KB>(act, lds_xq, lds_red);
 #pragma unroll
     for (int r = 0; r < NR; r++) load_xq(x[r], lds_xq, r * 8 + b, c, (r + 1) * 8 <= KB || r * 8 + b < KB);
   }
@@ -221,8 +327,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
     fused_stage_park<KB, RPI>(g, tile, lane);
     const int sn = s + nwaves;
     StepSel nxt = cur;
+    if constexpr (CONV) crn = cr;
     if (sn < total) {
       nxt = select_step<ROWS_PER_STEP>(A, sn);
+      if constexpr (CONV) conv_regs_load(crn, A, bidx, A.g[0].N, nxt.row0 + rl_conv);
       fused_stage_load<KB, RPI, SWIGLU>(g, nxt.W, A.g[1].W, nxt.row0, nxt.N, lane);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -258,11 +366,14 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(FusedArgs A
         const int64_t o = (int64_t)bidx * cur.N + row;
         if (cur.epi == EPI_F32) store_out<EPI_F32>(cur.out, cur.res, o, v);
         else if (cur.epi == EPI_BF16) store_out<EPI_BF16>(cur.out, cur.res, o, v);
-        else store_out<EPI_BF16_ADD>(cur.out, cur.res, o, v);
+        else if (CONV && cur.epi == EPI_CONV) {
+          if constexpr (CONV) ((uint16_t*)cur.out)[o] = conv_regs_apply(cr, A, bidx, cur.N, row, f32_to_bf16(v));
+        } else store_out<EPI_BF16_ADD>(cur.out, cur.res, o, v);
       }
     }
     s = sn;
     cur = nxt;
+    if constexpr (CONV) cr = crn;
   }
 }
 
@@ -273,8 +384,26 @@ bool gemv_fused_fast_path(int K, int batch, bool swiglu) {
 }
 
 template <int KB, int RPI, bool SWIGLU>
-static void launch_fused_pro(int pro, dim3 grid, const FusedArgs& A) {
+static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
   const dim3 block(GEMV_WAVES * 64);
+  if constexpr (KB == 8 && !SWIGLU) {
+    if (pro == PRO_GNORM && AX.ngroups > 1) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_GNORM, SWIGLU, false, FusedArgsX>), grid, block, 0, stream(), AX); return; }
+  }
+  if constexpr ((KB == 8 || KB == 4) && !SWIGLU) {
+    if (pro == PRO_RMSNORM && AX.conv_st) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU, true, FusedArgsX>), grid, block, 0, stream(), AX); return; }
+  }
+  if constexpr (!SWIGLU) {
+    if (AX.ngroups == 1) {         // one matrix: the 64-byte argument block
+      FusedArgs1 P{};
+      P.g0 = AX.g[0]; P.x = AX.x; P.norm_w = AX.norm_w; P.x_bstride = AX.x_bstride; P.steps = AX.step_first[4];
+      if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, false, false, FusedArgs1>), grid, block, 0, stream(), P);
+      else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, false, false, FusedArgs1>), grid, block, 0, stream(), P);
+      else if (pro == PRO_RMSNORM) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, false, FusedArgs1>), grid, block, 0, stream(), P);
+      else if constexpr (KB == 8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_GNORM, false, false, FusedArgs1>), grid, block, 0, stream(), P);
+      return;
+    }
+  }
+  const FusedArgs& A = AX;
   if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, SWIGLU>), grid, block, 0, stream(), A);
   else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, SWIGLU>), grid, block, 0, stream(), A);
   else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
@@ -285,16 +414,23 @@ int g_tune_fused_cap = 0;     // workgroups per CU of the fused GEMV (0: chosen 
 // Fast path only (gemv_fused_fast_path says whether it applies); the caller composes the same
 // result from separate kernels otherwise.
 int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
-                      void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu) {
-  BK_REQUIRE(pro == PRO_Q8 || pro == PRO_BF16 || pro == PRO_RMSNORM, "gemv_fused: bad prologue %d", pro);
-  BK_REQUIRE(x && (pro != PRO_RMSNORM || norm_w), "gemv_fused: null activation or norm weight");
+                      void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu, const FusedConv* conv) {
+  BK_REQUIRE(pro == PRO_Q8 || pro == PRO_BF16 || pro == PRO_RMSNORM || pro == PRO_GNORM, "gemv_fused: bad prologue %d", pro);
+  BK_REQUIRE(x && ((pro != PRO_RMSNORM && pro != PRO_GNORM) || norm_w), "gemv_fused: null activation or norm weight");
+  BK_REQUIRE(pro != PRO_GNORM || (K == 2048 && !swiglu), "gemv_fused: the gated-norm prologue serves K = 2048 (16 heads of 128), got K=%d", K);
   BK_REQUIRE(gemv_fused_fast_path(K, batch, swiglu), "gemv_fused: K=%d batch=%d is outside the fused kernel's shapes", K, batch);
   BK_REQUIRE(ngroups >= 1 && ngroups <= 4 && (!swiglu || ngroups == 2), "gemv_fused: bad number of matrices %d", ngroups);
   BK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemv_fused: activation and norm weight must be 16-byte aligned");
   const int KB = K / 256, RPI = KB <= 8 ? 4 : 2;
   const int rows_per_step = swiglu ? RPI / 2 : RPI;
-  FusedArgs A{};
+  FusedArgsX A{};
   A.ngroups = ngroups; A.x = x; A.norm_w = (const uint16_t*)norm_w;
+  A.x_bstride = pro == PRO_GNORM ? (int64_t)gdn_raw_bytes(K / 128, 1) : 0;
+  if (conv) {
+    BK_REQUIRE(!swiglu && pro == PRO_RMSNORM && (KB == 8 || KB == 4) && epi[0] == EPI_CONV && conv->st && conv->st_new && conv->w && ((uintptr_t)conv->w & 7) == 0,
+               "gemv_fused: the conv epilogue serves matrix 0 of an rmsnorm group with K = 1024 or 2048 (state, new state and 8-byte aligned taps given)");
+    A.conv_st = (const uint16_t*)conv->st; A.conv_st_new = (uint16_t*)conv->st_new; A.conv_w = (const uint16_t*)conv->w;
+  }
   int steps = 0;
   for (int i = 0; i < ngroups; i++) {
     BK_REQUIRE(W[i] && N[i] > 0 && ((uintptr_t)W[i] & 15) == 0, "gemv_fused: matrix %d: null, misaligned or N <= 0", i);
@@ -307,7 +443,8 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
       if (i == 0) { BK_REQUIRE(out[0], "gemv_fused: null output"); steps = (N[0] + rows_per_step - 1) / rows_per_step; }
     } else {
       BK_REQUIRE(out[i], "gemv_fused: matrix %d: null output", i);
-      BK_REQUIRE(epi[i] == EPI_F32 || epi[i] == EPI_BF16 || epi[i] == EPI_BF16_ADD, "gemv_fused: bad epilogue %d", epi[i]);
+      BK_REQUIRE(epi[i] == EPI_F32 || epi[i] == EPI_BF16 || epi[i] == EPI_BF16_ADD || (epi[i] == EPI_CONV && i == 0 && conv),
+                 "gemv_fused: bad epilogue %d", epi[i]);
       BK_REQUIRE(epi[i] != EPI_BF16_ADD || res[i], "gemv_fused: the add epilogue needs a residual");
       A.g[i].out = out[i]; A.g[i].res = (const uint16_t*)res[i]; A.g[i].epi = epi[i];
       A.step_first[i] = steps;

@@ -50,8 +50,10 @@ int launch_q4k_q8_1_subdots(const void* W, const void* xq, int32_t* I, int N, in
 // gemv_fused.hip   pro: 0 = x is Q8_1, 1 = x is bf16 (quantized in the kernel), 2 = rmsnorm(x, norm_w) then quantized
 extern int g_tune_fused_cap;
 bool gemv_fused_fast_path(int K, int batch, bool swiglu);
+struct FusedConv { const void* st; void* st_new; const void* w; };   // epi 3 of matrix 0: conv1d_decode's state, new state, taps
 int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int batch, int ngroups, const void* const* W,
-                      void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu);
+                      void* const* out, const void* const* res, const int* N, const int* epi, bool swiglu,
+                      const FusedConv* conv = nullptr);
 
 // gemm_mfma.hip
 extern int g_tune_small_rows;
@@ -94,6 +96,10 @@ int launch_gdn_conv_fused(const void* qkv, const void* conv_st, const void* conv
                           void* out, void* conv_st_new, float* S_out, void* out_q8, int Hg, int batch);
 int launch_gdn_core(const void* q, const void* k, const void* v, const float* g, const float* beta, const float* S_in,
                     void* out, float* S_out, int Hg, int batch);
+// column-slab form without the gated norm: raw = per sequence f32 o[Hg*128] | f32 z*sigmoid(z)[Hg*128] | f64 sum o^2 [Hg][4]
+size_t gdn_raw_bytes(int Hg, int batch);
+int launch_gdn_slabs(const void* conv_out, const void* z, const float* A_log, const void* dt_bias, const float* a_p,
+                     const float* b_p, const float* S_in, void* raw, float* S_out, int Hg, int batch);
 
 // attn.hip
 // what launch_attn_decode needs to fold the step's preparation (head norms, rotation, cache append) into the

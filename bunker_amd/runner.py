@@ -55,7 +55,22 @@ def choosePartition(graph: Graph, env=None, opts: dict | None = None) -> Partiti
 LM_HEAD_ROWS = 32768     # matmuls with more rows keep the stand-alone norm + quantizer (its cost is paid once, not per workgroup)
 
 
-def fusedPartition(graph: Graph) -> Partition:
+SLAB_MAX_BATCH = 7       # up to this batch the GDN step runs in column slabs (64 workgroups for 16 heads instead of 16)
+
+
+def graph_batch(graph: Graph) -> int:
+    """Sequences per step of a graph built by buildModelGraph (the leading dimension of its activations)."""
+    return int(graph.nodes[0].outputs[0].type.shape[0])
+
+
+def gdn_slab_form(gd: GraphNode, proj_K: int, batch: int) -> bool:
+    """Whether a GDN layer runs as [norm + projections + conv1d] [gdn_slabs] [gated norm + out_proj + add]: the kernels
+    exist for heads of 128 x 128, ZD = 2048 and projection rows of 1024 or 2048 at batch < 8."""
+    return (batch <= SLAB_MAX_BATCH and int(gd.params["ZD"]) == 2048 and int(gd.params["LKD"]) == 128 and int(gd.params["LVD"]) == 128
+            and proj_K in (1024, 2048))
+
+
+def fusedPartition(graph: Graph, slabs: bool | None = None) -> Partition:
     """Groups of nodes that one fused kernel (or one short kernel sequence) serves.
 
     The counterpart of src/fusion.ts's partitioning, with the fusions that pay on this hardware:
@@ -65,9 +80,14 @@ def fusedPartition(graph: Graph) -> Partition:
       conv1d_decode + gdn_delta_rule                          (the conv output stays on chip)
       qnorm + rope + knorm + ropek + fa2_attn                 (norm, rotation and cache append in one launch)
     A group is formed only when no tensor produced inside it (other than its declared result) is read outside.
+    At small batch (``slabs``; None = decided from the graph by gdn_slab_form) a GDN layer is cut differently, so that
+    its recurrence can run in column slabs on four times as many CUs: conv1d_decode joins the projections in front of it
+    (the convolution is the last step of the qkv rows), gdn_delta_rule stands alone and leaves its gated norm to the
+    out_proj group behind it (compilePartition: gdn_slabs, gemv_fused pro=3).
     """
     taken: set = set()
     groups: dict[int, list] = {}          # first node id -> group
+    batch = graph_batch(graph)
 
     def consumers(t):
         return graph.tensors[t].consumers
@@ -103,6 +123,15 @@ def fusedPartition(graph: Graph) -> Partition:
                         sw = c0[0]
                 nodes = [n] + list(cons) + ([sw] if sw else [])
                 results = {sw.outputs[0].tensorName} if sw else {c.outputs[0].tensorName for c in cons}
+                # slab form of a GDN layer: the convolution that reads the first matmul's rows joins the group
+                cv = consumers(cons[0].outputs[0].tensorName)
+                if not sw and len(cons) == 4 and len(cv) == 1 and cv[0].op == "conv1d_decode" and cons[0].params.get("cast"):
+                    gd = consumers(cv[0].outputs[0].tensorName)
+                    use = slabs if slabs is not None else (len(gd) == 1 and gd[0].op == "gdn_delta_rule" and
+                                                          gdn_slab_form(gd[0], int(cons[0].params["K"]), batch))
+                    if use and len(gd) == 1 and gd[0].op == "gdn_delta_rule":
+                        nodes.append(cv[0])
+                        results = (results - {cons[0].outputs[0].tensorName}) | {cv[0].outputs[0].tensorName}
                 if only_inside(nodes, results):
                     take(nodes)
         elif n.op == "gemm" and not n.params.get("cast"):
@@ -215,11 +244,24 @@ def node_spec(n: GraphNode, batch: int = 1, device_scalars: bool = False, attn_e
 Q8OUT_MIN_BATCH = 8      # from this batch on producers also emit their output as Q8_1 (gemv_fused then runs its batched path)
 
 
-def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict, attn_exact: bool = True) -> KernelPlan:
+def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of: dict, attn_exact: bool = True,
+                raw_of: dict | None = None) -> KernelPlan:
     """The fused op spec and slot list for a multi-node group (see fusedPartition)."""
     ops = tuple(n.op for n in grp)
     bpart = f" batch={batch}" if batch != 1 else ""
     name = "+".join(ops) + f"_{grp[0].id}"
+    raw_of = raw_of if raw_of is not None else {}
+    if ops[0] == "rmsnorm" and sorted(ops[1:]) == ["conv1d_decode", "gemm", "gemm", "gemm", "gemm"]:
+        norm, gemms, cv = grp[0], [n for n in grp if n.op == "gemm"], next(n for n in grp if n.op == "conv1d_decode")
+        K = int(gemms[0].params["K"])
+        spec = f"gemv_fused K={K} pro=2 G=4 " + " ".join(
+            f"N{i}={int(m.params['N'])} epi{i}={3 if i == 0 else (1 if m.params.get('cast') else 0)}" for i, m in enumerate(gemms)) + bpart
+        # x, norm_w, then W, conv_state_in, conv_w, conv out, conv_state_new for the qkv rows and W, out for the others
+        args = [norm.inputs[0].tensorName, norm.inputs[1].tensorName, gemms[0].inputs[1].tensorName, cv.inputs[1].tensorName,
+                cv.inputs[2].tensorName, cv.outputs[0].tensorName, cv.outputs[1].tensorName]
+        for m in gemms[1:]:
+            args += [m.inputs[1].tensorName, m.outputs[0].tensorName]
+        return KernelPlan(spec, name, args, [1, 1, 1], grp)
     if ops[0] == "rmsnorm" and ops[-1] == "swiglu":
         norm, gate, up, sw = grp
         N, K = int(gate.params["N"]), int(gate.params["K"])
@@ -247,6 +289,10 @@ def _group_plan(graph: Graph, grp: list, batch: int, device_scalars: bool, q8_of
         res = next(i.tensorName for i in a.inputs if i.tensorName != cast_out)
         N, K = int(m.params["N"]), int(m.params["K"])
         src = m.inputs[0].tensorName
+        if src in raw_of:     # the activation is the raw block of a gdn_slabs op: its gated norm is this kernel's prologue
+            aux, norm_w = raw_of[src]
+            return KernelPlan(f"gemv_fused K={K} pro=3 G=1 N0={N} epi0=2" + bpart, name,
+                              [aux, norm_w, m.inputs[1].tensorName, res, a.outputs[0].tensorName], [1, 1, 1], grp)
         if src in q8_of:      # the activation already exists as Q8_1 (written by a stand-alone rmsnorm_q8_1)
             spec, first = f"gemv_fused K={K} pro=0 G=1 N0={N} epi0=2" + bpart, q8_of[src]
         else:
@@ -289,14 +335,30 @@ def compilePartition(graph: Graph, ordered: Partition, batch: int = 1, device_sc
     auxiliary buffer, and those matmuls read that instead of quantizing again."""
     fused = any(len(grp) > 1 for grp in ordered)
     q8_of: dict[str, str] = {}
+    raw_of: dict[str, tuple] = {}       # output of a gdn_delta_rule node in slab form -> (its raw block, its norm weight)
+    in_conv_group = {n.outputs[0].tensorName for grp in ordered if len(grp) == 6 for n in grp if n.op == "conv1d_decode"}
     plans = []
     for grp in ordered:
         if len(grp) != 1:
-            plans.append(_group_plan(graph, grp, batch, device_scalars, q8_of, attn_exact))
+            plans.append(_group_plan(graph, grp, batch, device_scalars, q8_of, attn_exact, raw_of))
             continue
         n = grp[0]
         args = [i.tensorName for i in n.inputs] + [o.tensorName for o in n.outputs]
         bpart = f" batch={batch}" if batch != 1 else ""
+        if fused and n.op == "gdn_delta_rule" and n.inputs[0].tensorName in in_conv_group:
+            # slab form (fusedPartition put the convolution into the projections' group): the op leaves raw outputs, and
+            # the one matmul that reads its output runs the gated norm in its prologue
+            out = n.outputs[0].tensorName
+            cons = graph.tensors[out].consumers
+            if len(cons) == 1 and cons[0].op == "gemm" and cons[0].inputs[0].tensorName == out and int(cons[0].params["K"]) == 2048:
+                aux = out + ".raw"
+                raw_of[out] = (aux, n.inputs[6].tensorName)
+                LVH = int(n.params["LVH"])
+                spec = f"gdn_slabs LVH={LVH} LKD={int(n.params['LKD'])} LVD={int(n.params['LVD'])}" + bpart
+                a = [i.tensorName for i in n.inputs]
+                plans.append(KernelPlan(spec, f"gdn_slabs_{n.id}", a[:6] + [a[7], aux, n.outputs[1].tensorName], n.grid, grp,
+                                        {aux: batch * (LVH * 128 * 8 + LVH * 32)}))
+                continue
         if fused and n.op == "rmsnorm":
             out = n.outputs[0].tensorName
             cons = graph.tensors[out].consumers

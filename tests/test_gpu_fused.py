@@ -237,3 +237,87 @@ def test_gemv_fused_short_matrices_inside_the_norm_launch(orc, dev, batch):
                 assert np.array_equal(got[1][i][b].view(np.uint32), y.view(np.uint32)), (i, b)
             else:
                 assert np.array_equal(got[1][i][b], orc.cast_bf16(y)), (i, b)
+
+
+@pytest.mark.parametrize("K,batch,C", [(2048, 1, 6144), (2048, 3, 390), (1024, 2, 6144), (1024, 1, 262)])
+def test_gemv_fused_conv_epilogue_is_gemm_cast_conv1d(orc, dev, K, batch, C):
+    """gemv_fused epi0=3: the rows of matrix 0 go through conv1d_decode in the kernel's last step (the slab form of a GDN
+    layer).  Output, the shifted state (in place) and the other matrices of the group against the node sequence
+    rmsnorm -> gemm (cast) -> conv1d_decode, to the bit; two steps in a row, the second on the state the first left.
+    C = 390 / 262 are not multiples of the four rows of a wave step."""
+    print(f"gemv_fused conv epilogue K={K} batch={batch} C={C}", flush=True)
+    g = synth.rng(1300 + K + batch + C)
+    Ns, epis = [C, 130, 16, 18], [3, 1, 0, 0]
+    Ws = [synth.q4k_centered(g, n, K, 0.02) for n in Ns]
+    w = bf((g.standard_normal(K) * 0.1).astype(np.float32))
+    st = bf(g.standard_normal((batch, 3, C)).astype(np.float32))
+    cw = bf((g.standard_normal((C, 4)) * 0.5).astype(np.float32))
+    dst, dcw, dw = dev.up(st), dev.up(cw), dev.up(w)
+    dWs = [dev.up(W) for W in Ws]
+    outs = [dev.empty(batch * n * (4 if e == 0 else 2)) for n, e in zip(Ns, epis)]
+    spec = f"gemv_fused K={K} pro=2 G=4 batch={batch} " + " ".join(f"N{i}={n} epi{i}={e}" for i, (n, e) in enumerate(zip(Ns, epis)))
+    k = rt.compileAndLoad(spec)
+    ref_st = [st[b] for b in range(batch)]
+    for step in range(2):
+        x = bf(g.standard_normal((batch, K)).astype(np.float32))
+        args = [dev.up(x), dw, dWs[0], dst, dcw, outs[0], dst, dWs[1], outs[1], dWs[2], outs[2], dWs[3], outs[3]]
+        assert rt.cuLaunch(k, [1, 1, 1], [128, 1, 1], args) == 0, rt.last_error()
+        rt.cuSync()
+        xq_rows = ref_activation(orc, 2, x, w)
+        got_conv = rt.from_device(outs[0], (batch, C), np.uint16)
+        got_st = rt.from_device(dst, (batch, 3, C), np.uint16)
+        for b in range(batch):
+            qkv = orc.cast_bf16(orc.gemv_q4k_q8_1(Ws[0], xq_rows[b], C, K))
+            conv, ref_st[b] = orc.conv1d_decode(qkv, ref_st[b], cw)
+            assert np.array_equal(got_conv[b], conv), (step, b)
+            assert np.array_equal(got_st[b], ref_st[b]), (step, b)
+            assert np.array_equal(rt.from_device(outs[1], (batch, Ns[1]), np.uint16)[b], orc.cast_bf16(orc.gemv_q4k_q8_1(Ws[1], xq_rows[b], Ns[1], K)))
+            for i in (2, 3):
+                y = orc.gemv_q4k_q8_1(Ws[i], xq_rows[b], Ns[i], K)
+                assert np.array_equal(rt.from_device(outs[i], (batch, Ns[i]), np.float32)[b].view(np.uint32), y.view(np.uint32))
+    rt.unloadKernel(k)
+    with pytest.raises(rt.BunkerError, match="epi"):
+        rt.compileAndLoad("gemv_fused K=2048 pro=2 G=2 N0=64 epi0=1 N1=64 epi1=3")          # only matrix 0
+    with pytest.raises(rt.BunkerError, match="epi"):
+        rt.compileAndLoad("gemv_fused K=2048 pro=2 G=1 N0=64 epi0=3 batch=8")               # the batched path has no such step
+
+
+@pytest.mark.parametrize("B", [1, 3])
+def test_gdn_slabs_then_gated_norm_prologue_is_gdn_delta_rule_then_matmul(orc, dev, B):
+    """gdn_slabs (four column slabs per head, raw outputs) followed by gemv_fused pro=3 (the gated RMS norm in the
+    matmul's prologue) against gdn_delta_rule -> gemm -> cast -> add of the checker: state and the matmul's output to the
+    bit, and the raw block's pieces against the checker's gated norm."""
+    print(f"gdn_slabs + pro=3 B={B}", flush=True)
+    g = synth.rng(1400 + B)
+    Hg, H = 16, 520
+    C = 3 * Hg * 128
+    conv = bf(g.standard_normal((B, C)).astype(np.float32))
+    z = bf(g.standard_normal((B, Hg * 128)).astype(np.float32))
+    A_log = g.uniform(-2, 1, Hg).astype(np.float32)
+    dt_bias = bf(g.standard_normal(Hg).astype(np.float32))
+    a_p = g.standard_normal((B, Hg)).astype(np.float32); b_p = g.standard_normal((B, Hg)).astype(np.float32)
+    norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    S = (g.standard_normal((B, Hg, 128, 128)) * 0.02).astype(np.float32)
+    Wo = synth.q4k_centered(g, H, Hg * 128, 0.02)
+    res = bf(g.standard_normal((B, H)).astype(np.float32))
+    raw_bytes = Hg * 128 * 8 + Hg * 32
+    draw, dS, dnw = dev.empty(B * raw_bytes), dev.up(S), dev.up(norm_w)
+    bp = f" batch={B}" if B != 1 else ""
+    launch(f"gdn_slabs LVH={Hg} LKD=128 LVD=128" + bp,
+           [dev.up(conv), dev.up(z), dev.up(A_log), dev.up(dt_bias), dev.up(a_p), dev.up(b_p), dS, draw, dS])      # S updated in place
+    dout = dev.empty(B * H * 2)
+    launch(f"gemv_fused K={Hg * 128} pro=3 G=1 N0={H} epi0=2" + bp, [draw, dnw, dev.up(Wo), dev.up(res), dout])
+    Sn = rt.from_device(dS, S.shape, np.float32)
+    out = rt.from_device(dout, (B, H), np.uint16)
+    raw = rt.from_device(draw, (B, raw_bytes), np.uint8)
+    for b in range(B):
+        ro, rS = orc.gdn_step(conv[b], z[b], A_log, dt_bias, a_p[b], b_p[b], norm_w, S[b], Hg, rows_per_chain=16)
+        assert np.array_equal(Sn[b].view(np.uint32), rS.view(np.uint32)), b
+        y = orc.gemv_q4k_q8_1(Wo, orc.pack_q8_1(f32(ro)), H, Hg * 128)
+        assert np.array_equal(out[b], orc.add_bf16(orc.cast_bf16(y), res[b])), b
+        # the raw block: o and z * sigmoid(z) per column, the sum of o^2 per (head, slab)
+        o = raw[b, :Hg * 128 * 4].view(np.float32).astype(np.float64).reshape(Hg, 4, 32)
+        ss = raw[b, Hg * 128 * 8:].view(np.float64).reshape(Hg, 4)
+        assert np.allclose(ss, (o ** 2).sum(axis=2), rtol=1e-14, atol=0)
+    with pytest.raises(rt.BunkerError, match="pro=3"):
+        rt.compileAndLoad("gemv_fused K=4096 pro=3 G=1 N0=64 epi0=2")

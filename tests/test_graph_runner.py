@@ -100,7 +100,7 @@ def test_fused_partition_groups_and_specs():
     still orders by dependencies; the fused specs carry shapes and epilogues."""
     import collections
     g = model.buildModelGraph(SYNTH)
-    part = runner.fusedPartition(g)
+    part = runner.fusedPartition(g, slabs=False)
     ids = [n.id for grp in part for n in grp]
     assert sorted(ids) == [n.id for n in g.nodes]
     kinds = collections.Counter(tuple(n.op for n in grp) for grp in part)
@@ -126,6 +126,27 @@ def test_fused_partition_groups_and_specs():
     assert "gemv_fused K=2048 pro=2 G=2 swiglu=1 N0=6144 N1=6144" in specs
     assert "gemv_fused K=6144 pro=1 G=1 N0=2048 epi0=2" in specs
     assert "fa2_fused HD=256 NH=16 NKV=2 MAX_LEN=4352 ROT_HALF=32 pos_dev=1" in specs
+    # At batch 1 (the default choice up to batch 7 for layers with ZD = 2048) a GDN layer is cut the other way: the
+    # convolution joins the projections, the recurrence stands alone in its slab form and leaves raw outputs, and the
+    # out_proj group reads those through its gated-norm prologue
+    part_s = runner.fusedPartition(g)
+    assert sorted(n.id for grp in part_s for n in grp) == [n.id for n in g.nodes] and len(part_s) == 124
+    kinds_s = collections.Counter(tuple(sorted(n.op for n in grp)) for grp in part_s)
+    assert kinds_s[("conv1d_decode", "gemm", "gemm", "gemm", "gemm", "rmsnorm")] == 18 and kinds_s[("gdn_delta_rule",)] == 18
+    assert kinds_s[("conv1d_decode", "gdn_delta_rule")] == 0
+    plans_s = runner.compilePartition(g, runner.topoOrder(g, part_s), 1, True)
+    conv_plan = next(p for p in plans_s if "epi0=3" in p.spec)
+    assert conv_plan.spec == "gemv_fused K=2048 pro=2 G=4 N0=6144 epi0=3 N1=2048 epi1=1 N2=16 epi2=0 N3=16 epi3=0" and len(conv_plan.args) == 13
+    assert conv_plan.args[3] == "model.layers.0.conv_state_in" and conv_plan.args[6].endswith("conv_state_new")
+    slab = next(p for p in plans_s if p.spec.startswith("gdn_slabs"))
+    assert slab.spec == "gdn_slabs LVH=16 LKD=128 LVD=128" and list(slab.aux.values()) == [16 * 128 * 8 + 16 * 32]
+    assert slab.args[0] == conv_plan.args[5] and slab.args[6] == "model.layers.0.s_state_in"
+    outp = next(p for p in plans_s if p.args[0] == slab.args[7])
+    assert outp.spec == "gemv_fused K=2048 pro=3 G=1 N0=2048 epi0=2" and outp.args[1] == "model.layers.0.linear_attn.norm.weight"
+    assert sum(p.spec.startswith("gdn_slabs") for p in plans_s) == 18 and not any(p.spec.startswith("gdn_conv") for p in plans_s)
+    # the small test model (ZD = 256) and batches from 8 on keep conv1d + recurrence in one launch
+    gt = model.buildModelGraph(model.TINY)
+    assert all(not p.spec.startswith("gdn_slabs") for p in runner.compilePartition(gt, runner.topoOrder(gt, runner.fusedPartition(gt)), 1, True))
     # from batch 8 on gdn_conv, fa2_fused and the SwiGLU group leave their output as Q8_1 too, and the projection behind
     # them reads that (pro=0) instead of quantizing
     g32 = model.buildModelGraph(SYNTH, 32)

@@ -48,6 +48,8 @@ def expand(plan, batch, attn_exact, q8_in):
     q8out = SUFFIX["q8out"] if batch >= ts_const("Q8OUT_MIN_BATCH") else ""
     if len(ops) == 1:
         op, p = ops[0], P[0]
+        if plan["spec"].startswith("gdn_slabs"):
+            return fill(FUSED["gdn_slabs"], LVH=p["LVH"], LKD=p["LKD"], LVD=p["LVD"]) + bpart
         if plan["spec"].startswith("rmsnorm_q8_1"):
             return fill(FUSED["rmsnorm_q8_1"], N=p["N"]) + bpart
         if op == "gemm" and q8_in:
@@ -65,10 +67,16 @@ def expand(plan, batch, attn_exact, q8_in):
         return s
     if key == "rmsnorm+gemm+gemm+swiglu":
         return fill(FUSED[key], K=P[1]["K"], N=P[1]["N"]) + bpart + (q8out if P[1]["N"] % 32 == 0 else "")
+    if ops[0] == "rmsnorm" and "conv1d_decode" in ops:
+        gem = [p for o, p in zip(ops, P) if o == "gemm"]
+        mats = "".join(fill(FUSED["mat"], i=i, N=p["N"], EPI=3 if i == 0 else (1 if p.get("cast") else 0)) for i, p in enumerate(gem))
+        return fill(FUSED["rmsnorm+gemm*+conv1d_decode"], K=gem[0]["K"], MATS=mats) + bpart
     if ops[0] == "rmsnorm" and all(o == "gemm" for o in ops[1:]):
         mats = "".join(fill(FUSED["mat"], i=i, N=p["N"], EPI=1 if p.get("cast") else 0) for i, p in enumerate(P[1:]))
         return fill(FUSED["rmsnorm+gemm*"], K=P[1]["K"], G=len(ops) - 1, MATS=mats) + bpart
     if key == "gemm+cast+add":
+        if " pro=3 " in plan["spec"]:        # reads the raw block of a gdn_slabs op (rawOf in specs.ts)
+            return fill(FUSED["gemm+cast+add@raw"], K=P[0]["K"], N=P[0]["N"]) + bpart
         return fill(FUSED[key], K=P[0]["K"], N=P[0]["N"], PRO=0 if q8_in else 1) + bpart
     if key == "conv1d_decode+gdn_delta_rule":
         return fill(FUSED[key], LVH=P[1]["LVH"], LKD=P[1]["LKD"], LVD=P[1]["LVD"]) + bpart + q8out
@@ -110,13 +118,14 @@ def test_fixture_is_what_the_host_layer_builds_today():
 def test_ts_constants_and_exports():
     assert SPEC_KEYS == runner._SPEC_KEYS                      # the same 14 ops, the same constants in the same order
     assert ts_const("Q8OUT_MIN_BATCH") == runner.Q8OUT_MIN_BATCH and ts_const("LM_HEAD_ROWS") == runner.LM_HEAD_ROWS
+    assert ts_const("SLAB_MAX_BATCH") == runner.SLAB_MAX_BATCH
     assert ts_const("PAGE_TOKENS") == 16
     for fn in ("nodeSpec", "groupPlan", "compilePartition", "loadPartition", "stateBytes", "ropeTables"):
         assert re.search(r"^export function %s\(" % fn, TS, flags=re.M), fn
     # every fused group the Python partition forms has a template, and the templates name only variables groupPlan fills
     keys = {"+".join(p["ops"]) for b in ("batch1", "batch32") for p in GOLD[b]["fused"]["distinct"] if len(p["ops"]) > 1}
     for k in keys:
-        assert k in FUSED or (k.startswith("rmsnorm+gemm") and "rmsnorm+gemm*" in FUSED), k
+        assert k in FUSED or (k.startswith("rmsnorm+gemm") and ("rmsnorm+gemm*+conv1d_decode" if "conv1d_decode" in k else "rmsnorm+gemm*") in FUSED), k
     # state sizes of stateBytes are the graph's tensor sizes
     D, B = model.SYNTH, 3
     g = model.buildModelGraph(D, B)

@@ -47,6 +47,11 @@ export const FUSED_SPECS: Record<string, string> = {
   "mat": " N${i}=${N} epi${i}=${EPI}",
   "gemm+cast+add": "gemv_fused K=${K} pro=${PRO} G=1 N0=${N} epi0=2",
   "conv1d_decode+gdn_delta_rule": "gdn_conv LVH=${LVH} LKD=${LKD} LVD=${LVD}",
+  // slab form of a GDN layer (batch <= SLAB_MAX_BATCH): conv1d is the last step of the qkv rows (epi0=3), the
+  // recurrence runs in four column slabs per head and leaves raw outputs, the out_proj group runs its gated norm (pro=3)
+  "rmsnorm+gemm*+conv1d_decode": "gemv_fused K=${K} pro=2 G=4${MATS}",
+  "gdn_slabs": "gdn_slabs LVH=${LVH} LKD=${LKD} LVD=${LVD}",
+  "gemm+cast+add@raw": "gemv_fused K=${K} pro=3 G=1 N0=${N} epi0=2",
   "qnorm+rope+knorm+ropek+fa2_attn": "fa2_fused HD=${HD} NH=${NH} NKV=${NKV} MAX_LEN=${MAX_LEN} ROT_HALF=${ROT_HALF}",
   "rmsnorm_q8_1": "rmsnorm_q8_1 N=${N}",
   "gemm@q8_1": "gemv_fused K=${K} pro=0 G=1 N0=${N} epi0=${EPI}",
@@ -63,6 +68,7 @@ export const SPEC_SUFFIX: Record<string, string> = {
 };
 
 export const Q8OUT_MIN_BATCH = 8;      // from this batch on producers also emit Q8_1 and the matmuls behind them read it
+export const SLAB_MAX_BATCH = 7;       // up to this batch a GDN layer with ZD = 2048 and projection rows of 1024 / 2048 takes the slab form
 export const LM_HEAD_ROWS = 32768;     // matmuls with more rows keep the stand-alone norm + quantizer
 
 function fill(template: string, vars: Record<string, number | string>): string {
@@ -84,7 +90,8 @@ export function nodeSpec(n: GraphNode, batch = 1, deviceScalars = false, attnExa
 const tn = (io: NodeIO) => io.tensorName;
 
 /** Spec and slot list of a fused group (the counterpart of codegenGroup for the groups fusedPartition forms). */
-export function groupPlan(grp: GraphNode[], batch: number, deviceScalars: boolean, q8Of: Map<string, string>, attnExact = true): KernelPlan {
+export function groupPlan(grp: GraphNode[], batch: number, deviceScalars: boolean, q8Of: Map<string, string>, attnExact = true,
+                          rawOf: Map<string, [string, string]> = new Map()): KernelPlan {
   const ops = grp.map((n) => n.op);
   const key = ops.join("+");
   const bpart = batch !== 1 ? fill(SPEC_SUFFIX.batch, { batch }) : "";
@@ -102,6 +109,15 @@ export function groupPlan(grp: GraphNode[], batch: number, deviceScalars: boolea
     }
     return plan(spec, args);
   }
+  if (ops[0] === "rmsnorm" && ops.length === 6 && ops.filter((o) => o === "gemm").length === 4 && ops.includes("conv1d_decode")) {
+    // norm + qkv, z, a, b + conv1d_decode over the qkv rows (the group is ordered by node id: the conv node sits between the matmuls)
+    const norm = grp[0], gemms = grp.filter((n) => n.op === "gemm"), cv = grp.find((n) => n.op === "conv1d_decode")!;
+    const MATS = gemms.map((m, i) => fill(FUSED_SPECS.mat, { i, N: int(m.params.N), EPI: i === 0 ? 3 : (m.params.cast ? 1 : 0) })).join("");
+    // x, norm_w, then W, conv_state_in, conv_w, conv out, conv_state_new for the qkv rows and W, out for the others
+    const args = [tn(norm.inputs[0]), tn(norm.inputs[1]), tn(gemms[0].inputs[1]), tn(cv.inputs[1]), tn(cv.inputs[2]), tn(cv.outputs[0]), tn(cv.outputs[1])];
+    for (const m of gemms.slice(1)) args.push(tn(m.inputs[1]), tn(m.outputs[0]));
+    return plan(fill(FUSED_SPECS["rmsnorm+gemm*+conv1d_decode"], { K: int(gemms[0].params.K), MATS }) + bpart, args);
+  }
   if (ops[0] === "rmsnorm" && ops.length > 1 && ops.slice(1).every((o) => o === "gemm")) {
     const [norm, ...gemms] = grp;
     const K = int(gemms[0].params.K);
@@ -115,6 +131,11 @@ export function groupPlan(grp: GraphNode[], batch: number, deviceScalars: boolea
     const castOut = tn(c.outputs[0]);
     const res = tn(a.inputs.find((i) => i.tensorName !== castOut)!);
     const N = int(m.params.N), K = int(m.params.K), src = tn(m.inputs[0]);
+    if (rawOf.has(src)) {
+      // the activation is the raw block of a gdn_slabs op: its gated norm is this kernel's prologue
+      const [aux, normW] = rawOf.get(src)!;
+      return plan(fill(FUSED_SPECS["gemm+cast+add@raw"], { K, N }) + bpart, [aux, normW, tn(m.inputs[1]), res, tn(a.outputs[0])]);
+    }
     // the activation already exists as Q8_1 (written by a stand-alone rmsnorm_q8_1 or a q8out producer): pro=0
     const first = q8Of.get(src) ?? src;
     const spec = fill(FUSED_SPECS[key], { K, N, PRO: q8Of.has(src) ? 0 : 1 }) + bpart;
@@ -150,12 +171,27 @@ export function groupPlan(grp: GraphNode[], batch: number, deviceScalars: boolea
 export function compilePartition(graph: Graph, ordered: GraphNode[][], batch = 1, deviceScalars = false, attnExact = true): KernelPlan[] {
   const fused = ordered.some((g) => g.length > 1);
   const q8Of = new Map<string, string>();
+  const rawOf = new Map<string, [string, string]>();    // output of a gdn_delta_rule node in slab form -> [raw block, norm weight]
+  const inConvGroup = new Set<string>();
+  for (const g of ordered) if (g.length === 6) for (const n of g) if (n.op === "conv1d_decode") inConvGroup.add(tn(n.outputs[0]));
   const plans: KernelPlan[] = [];
   for (const grp of ordered) {
-    if (grp.length !== 1) { plans.push(groupPlan(grp, batch, deviceScalars, q8Of, attnExact)); continue; }
+    if (grp.length !== 1) { plans.push(groupPlan(grp, batch, deviceScalars, q8Of, attnExact, rawOf)); continue; }
     const n = grp[0];
     const args = [...n.inputs.map(tn), ...n.outputs.map(tn)];
     const bpart = batch !== 1 ? fill(SPEC_SUFFIX.batch, { batch }) : "";
+    if (fused && n.op === "gdn_delta_rule" && inConvGroup.has(tn(n.inputs[0]))) {
+      // slab form: raw outputs; the one matmul that reads the op's output runs the gated norm in its prologue
+      const out = tn(n.outputs[0]);
+      const cons = graph.tensors.get(out)!.consumers;
+      if (cons.length === 1 && cons[0].op === "gemm" && cons[0].inputs[0].tensorName === out && int(cons[0].params.K) === 2048) {
+        const aux = out + ".raw", LVH = int(n.params.LVH), a = n.inputs.map(tn);
+        rawOf.set(out, [aux, a[6]]);
+        plans.push({ spec: fill(FUSED_SPECS.gdn_slabs, { LVH, LKD: int(n.params.LKD), LVD: int(n.params.LVD) }) + bpart, name: `gdn_slabs_${n.id}`,
+                     args: [...a.slice(0, 6), a[7], aux, tn(n.outputs[1])], grid: n.grid, group: grp, aux: { [aux]: batch * (LVH * 128 * 8 + LVH * 32) } });
+        continue;
+      }
+    }
     if (fused && n.op === "rmsnorm") {
       // a stand-alone norm whose readers are all matmuls also leaves its result as Q8_1; those matmuls read that
       const out = tn(n.outputs[0]);
