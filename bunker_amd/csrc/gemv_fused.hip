@@ -55,19 +55,45 @@ struct FusedArgsX : FusedArgs {
   int64_t x_bstride;     // PRO_GNORM: bytes between two sequences' raw blocks
 };
 
-// A launch with one matrix (out_proj, o_proj, down, lm_head: half of the decode step's launches) gets its arguments in
-// 64 bytes instead of 168: the kernel's first instructions wait for the argument block, and a block that spans fewer
-// cache lines arrives sooner.  The kernel works on the full form, rebuilt in registers.
+// Compact argument blocks.  A kernel's first instructions wait for its argument block, and the block arrives cache line
+// by cache line: every 64 bytes less measured 0.2-0.3 us per launch (one-matrix launches 168 -> 64 bytes: 11 us over the
+// decode step).  The launcher picks the smallest form that holds the launch; the kernel rebuilds the full form in
+// registers (step_first from the row counts) and runs unchanged.
+//   FusedArgs1: one matrix (out_proj, o_proj, down, lm_head: half of the step's launches), 60 bytes
+//   FusedArgs2: the SwiGLU pair, 48 bytes
+//   FusedArgsC: up to four matrices without residuals, 104 bytes; with the conv epilogue's operands (FusedArgsCX) 128
+//               (unused slots repeat the last matrix)
 struct FusedArgs1 {
   FusedGroup g0;
   const void* x;
   const uint16_t* norm_w;
   int64_t x_bstride;
-  int steps, pad;
+  int steps;
 };
-__device__ __forceinline__ const FusedArgs& fused_args_full(const FusedArgs& A) { return A; }
-__device__ __forceinline__ const FusedArgsX& fused_args_full(const FusedArgsX& A) { return A; }
-__device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs1& P) {
+struct FusedArgs2 {
+  const uint8_t *Wg, *Wu;
+  void* out;
+  const void* x;
+  const uint16_t* norm_w;
+  int N, steps;
+};
+struct FusedArgsC {
+  const uint8_t* W[4];
+  void* out[4];
+  const void* x;
+  const uint16_t* norm_w;
+  int N[4];
+  int epi4;              // epilogue of matrix i in bits 8 i .. 8 i + 7
+  int ngroups;
+};
+struct FusedArgsCX : FusedArgsC {
+  const uint16_t* conv_st;
+  uint16_t* conv_st_new;
+  const uint16_t* conv_w;
+};
+__device__ __forceinline__ const FusedArgs& fused_args_full(const FusedArgs& A, int) { return A; }
+__device__ __forceinline__ const FusedArgsX& fused_args_full(const FusedArgsX& A, int) { return A; }
+__device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs1& P, int) {
   FusedArgsX A;
   A.g[0] = P.g0; A.g[1] = P.g0; A.g[2] = P.g0; A.g[3] = P.g0;
   A.step_first[0] = 0; A.step_first[1] = P.steps; A.step_first[2] = P.steps; A.step_first[3] = P.steps; A.step_first[4] = P.steps;
@@ -75,19 +101,35 @@ __device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs1& P) {
   A.conv_st = nullptr; A.conv_st_new = nullptr; A.conv_w = nullptr; A.x_bstride = P.x_bstride;
   return A;
 }
+__device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs2& P, int) {
+  FusedArgsX A;
+  A.g[0].W = P.Wg; A.g[0].out = P.out; A.g[0].res = nullptr; A.g[0].N = P.N; A.g[0].epi = EPI_BF16;
+  A.g[1].W = P.Wu; A.g[1].out = P.out; A.g[1].res = nullptr; A.g[1].N = P.N; A.g[1].epi = EPI_BF16;
+  A.g[2] = A.g[1]; A.g[3] = A.g[1];
+  A.step_first[0] = 0; A.step_first[1] = P.steps; A.step_first[2] = P.steps; A.step_first[3] = P.steps; A.step_first[4] = P.steps;
+  A.ngroups = 2; A.x = P.x; A.norm_w = P.norm_w;
+  A.conv_st = nullptr; A.conv_st_new = nullptr; A.conv_w = nullptr; A.x_bstride = 0;
+  return A;
+}
+// The several-matrix forms are read where they lie (their arrays are indexed by the step's matrix: rebuilt in registers
+// they would end up in private memory); step_first comes from the row counts.
+__device__ __forceinline__ const FusedArgsC& fused_args_full(const FusedArgsC& A, int) { return A; }
+__device__ __forceinline__ const FusedArgsCX& fused_args_full(const FusedArgsCX& A, int) { return A; }
 
 // The operands of one channel of the convolution, requested ahead of the step's arithmetic
 struct ConvRegs {
   uint16_t s0, s1, s2;
   uint2 w;
 };
-__device__ __forceinline__ void conv_regs_load(ConvRegs& c, const FusedArgsX& A, int bidx, int C, int ch) {
+template <typename AX>
+__device__ __forceinline__ void conv_regs_load(ConvRegs& c, const AX& A, int bidx, int C, int ch) {
   ch = min(ch, C - 1);
   const uint16_t* sb = A.conv_st + (int64_t)bidx * 3 * C;
   c.s0 = sb[ch]; c.s1 = sb[C + ch]; c.s2 = sb[2 * C + ch];
   c.w = *(const uint2*)(A.conv_w + 4 * (int64_t)ch);
 }
-__device__ __forceinline__ uint16_t conv_regs_apply(const ConvRegs& c, const FusedArgsX& A, int bidx, int C, int ch, uint16_t x) {
+template <typename AX>
+__device__ __forceinline__ uint16_t conv_regs_apply(const ConvRegs& c, const AX& A, int bidx, int C, int ch, uint16_t x) {
   const float w0 = __uint_as_float(c.w.x << 16), w1 = __uint_as_float(c.w.x & 0xffff0000u);
   const float w2 = __uint_as_float(c.w.y << 16), w3 = __uint_as_float(c.w.y & 0xffff0000u);
   // products of two bf16 values are exact in f32
@@ -140,16 +182,44 @@ struct StepSel {
   int N, epi, row0;
 };
 
+struct StepFirst { int f1, f2, f3, total; };
+__device__ __forceinline__ StepFirst step_first_of(const FusedArgs& A, int) {
+  return StepFirst{A.step_first[1], A.step_first[2], A.step_first[3], A.step_first[4]};
+}
+__device__ __forceinline__ StepFirst step_first_of(const FusedArgsC& P, int rps) {
+  const int s0 = (P.N[0] + rps - 1) / rps;
+  const int s1 = s0 + (P.ngroups > 1 ? (P.N[1] + rps - 1) / rps : 0);
+  const int s2 = s1 + (P.ngroups > 2 ? (P.N[2] + rps - 1) / rps : 0);
+  const int s3 = s2 + (P.ngroups > 3 ? (P.N[3] + rps - 1) / rps : 0);
+  return StepFirst{s0, s1, s2, s3};
+}
+__device__ __forceinline__ int rows_of_first(const FusedArgs& A) { return A.g[0].N; }
+__device__ __forceinline__ int rows_of_first(const FusedArgsC& A) { return A.N[0]; }
+__device__ __forceinline__ const uint8_t* second_matrix(const FusedArgs& A) { return A.g[1].W; }
+__device__ __forceinline__ const uint8_t* second_matrix(const FusedArgsC& A) { return A.W[1]; }
+
 template <int ROWS_PER_STEP>
-__device__ __forceinline__ StepSel select_step(const FusedArgs& A, int s) {
-  const bool s1 = s >= A.step_first[1], s2 = s >= A.step_first[2], s3 = s >= A.step_first[3];
+__device__ __forceinline__ StepSel select_step(const FusedArgs& A, const StepFirst& F, int s) {
+  const bool s1 = s >= F.f1, s2 = s >= F.f2, s3 = s >= F.f3;
   StepSel r;
   r.W = s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
   r.out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
   r.res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
   r.N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
   r.epi = s3 ? A.g[3].epi : s2 ? A.g[2].epi : s1 ? A.g[1].epi : A.g[0].epi;
-  r.row0 = (s - (s3 ? A.step_first[3] : s2 ? A.step_first[2] : s1 ? A.step_first[1] : 0)) * ROWS_PER_STEP;
+  r.row0 = (s - (s3 ? F.f3 : s2 ? F.f2 : s1 ? F.f1 : 0)) * ROWS_PER_STEP;
+  return r;
+}
+template <int ROWS_PER_STEP>
+__device__ __forceinline__ StepSel select_step(const FusedArgsC& A, const StepFirst& F, int s) {
+  const bool s1 = s >= F.f1, s2 = s >= F.f2, s3 = s >= F.f3;
+  StepSel r;
+  r.W = s3 ? A.W[3] : s2 ? A.W[2] : s1 ? A.W[1] : A.W[0];
+  r.out = s3 ? A.out[3] : s2 ? A.out[2] : s1 ? A.out[1] : A.out[0];
+  r.res = nullptr;
+  r.N = s3 ? A.N[3] : s2 ? A.N[2] : s1 ? A.N[1] : A.N[0];
+  r.epi = (A.epi4 >> (s3 ? 24 : s2 ? 16 : s1 ? 8 : 0)) & 0xff;
+  r.row0 = (s - (s3 ? F.f3 : s2 ? F.f2 : s1 ? F.f1 : 0)) * ROWS_PER_STEP;
   return r;
 }
 
@@ -272,7 +342,7 @@ __device__ __forceinline__ void fused_stage_park(const FusedStage<KB, RPI>& g, u
 // the lanes past the row in the last pass read a clamped block and an all-zero activation slice, which adds exact zeros.
 template <int KB, int RPI, int PRO, bool SWIGLU, bool CONV = false, typename ARGS = FusedArgs>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) {
-  const auto& A = fused_args_full(A_in);
+  const auto& A = fused_args_full(A_in, SWIGLU ? RPI / 2 : RPI);
   static_assert(!CONV || (!SWIGLU && RPI == 4 && PRO == PRO_RMSNORM), "the conv epilogue exists for the form the decode step asks for");
   constexpr int NR = (KB + 7) / 8;
   constexpr int RP = KB * 9;                 // 16-byte pieces per row
@@ -291,7 +361,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) 
   const int c = lane & 7, b = lane >> 3;
   const ScaleSel sel = make_scale_sel(c);
   const bool odd = c & 1;
-  const int total = A.step_first[4];
+  const StepFirst F = step_first_of(A, ROWS_PER_STEP);
+  const int total = F.total;
   uint4* tile = tiles[wv];
 
   [[maybe_unused]] ActRegs<KB> act;
@@ -300,7 +371,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) 
   else if constexpr (PRO != PRO_Q8) act_load<PRO, KB>(act, (const uint16_t*)A.x + (int64_t)bidx * K, A.norm_w);
 
   int s = blockIdx.x * GEMV_WAVES + wv;
-  StepSel cur = select_step<ROWS_PER_STEP>(A, s < total ? s : 0);
+  StepSel cur = select_step<ROWS_PER_STEP>(A, F, s < total ? s : 0);
   FusedStage<KB, RPI> g;
   // unconditional (a wave without a step of its own requests step 0): with a branch around these loads the
   // prologue's first wait could not be counted and would drain the weight rows as well
@@ -308,8 +379,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) 
   // long before the step's dots are folded); lanes 0..RPI-1 hold the step's rows
   const int rl_conv = 2 * (lane & 1) + ((lane >> 1) & 1);
   [[maybe_unused]] ConvRegs cr, crn;       // touched only by the CONV form (unused, they would end up as LDS-backed arrays)
-  if constexpr (CONV) conv_regs_load(cr, A, bidx, A.g[0].N, cur.row0 + rl_conv);      // unconditional: rows of the other matrices read a clamped channel
-  fused_stage_load<KB, RPI, SWIGLU>(g, cur.W, A.g[1].W, cur.row0, cur.N, lane);
+  if constexpr (CONV) conv_regs_load(cr, A, bidx, rows_of_first(A), cur.row0 + rl_conv);      // unconditional: rows of the other matrices read a clamped channel
+  fused_stage_load<KB, RPI, SWIGLU>(g, cur.W, second_matrix(A), cur.row0, cur.N, lane);
 
   XQ x[NR];
   if (PRO == PRO_Q8) {
@@ -329,9 +400,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) 
     StepSel nxt = cur;
     if constexpr (CONV) crn = cr;
     if (sn < total) {
-      nxt = select_step<ROWS_PER_STEP>(A, sn);
-      if constexpr (CONV) conv_regs_load(crn, A, bidx, A.g[0].N, nxt.row0 + rl_conv);
-      fused_stage_load<KB, RPI, SWIGLU>(g, nxt.W, A.g[1].W, nxt.row0, nxt.N, lane);
+      nxt = select_step<ROWS_PER_STEP>(A, F, sn);
+      if constexpr (CONV) conv_regs_load(crn, A, bidx, rows_of_first(A), nxt.row0 + rl_conv);
+      fused_stage_load<KB, RPI, SWIGLU>(g, nxt.W, second_matrix(A), nxt.row0, nxt.N, lane);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -386,14 +457,17 @@ bool gemv_fused_fast_path(int K, int batch, bool swiglu) {
 template <int KB, int RPI, bool SWIGLU>
 static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
   const dim3 block(GEMV_WAVES * 64);
-  if constexpr (KB == 8 && !SWIGLU) {
-    if (pro == PRO_GNORM && AX.ngroups > 1) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_GNORM, SWIGLU, false, FusedArgsX>), grid, block, 0, stream(), AX); return; }
-  }
-  if constexpr ((KB == 8 || KB == 4) && !SWIGLU) {
-    if (pro == PRO_RMSNORM && AX.conv_st) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU, true, FusedArgsX>), grid, block, 0, stream(), AX); return; }
-  }
-  if constexpr (!SWIGLU) {
-    if (AX.ngroups == 1) {         // one matrix: the 64-byte argument block
+  bool any_res = false;
+  for (int i = 0; i < AX.ngroups; i++) any_res = any_res || AX.g[i].res != nullptr;
+  if constexpr (SWIGLU) {
+    FusedArgs2 P{};
+    P.Wg = AX.g[0].W; P.Wu = AX.g[1].W; P.out = AX.g[0].out; P.x = AX.x; P.norm_w = AX.norm_w; P.N = AX.g[0].N; P.steps = AX.step_first[4];
+    if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, true, false, FusedArgs2>), grid, block, 0, stream(), P);
+    else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, true, false, FusedArgs2>), grid, block, 0, stream(), P);
+    else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, true, false, FusedArgs2>), grid, block, 0, stream(), P);
+    return;
+  } else {
+    if (AX.ngroups == 1) {         // one matrix
       FusedArgs1 P{};
       P.g0 = AX.g[0]; P.x = AX.x; P.norm_w = AX.norm_w; P.x_bstride = AX.x_bstride; P.steps = AX.step_first[4];
       if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, false, false, FusedArgs1>), grid, block, 0, stream(), P);
@@ -402,11 +476,34 @@ static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
       else if constexpr (KB == 8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_GNORM, false, false, FusedArgs1>), grid, block, 0, stream(), P);
       return;
     }
+    if (!any_res && pro != PRO_GNORM) {      // several matrices, no residual: the 104 / 128-byte forms
+      FusedArgsCX P{};
+      for (int i = 0; i < 4; i++) {
+        const int j = i < AX.ngroups ? i : AX.ngroups - 1;
+        P.W[i] = AX.g[j].W; P.out[i] = AX.g[j].out; P.N[i] = AX.g[j].N; P.epi4 |= (AX.g[j].epi & 0xff) << (8 * i);
+      }
+      P.x = AX.x; P.norm_w = AX.norm_w; P.ngroups = AX.ngroups;
+      P.conv_st = AX.conv_st; P.conv_st_new = AX.conv_st_new; P.conv_w = AX.conv_w;
+      if constexpr (KB == 8 || KB == 4) {
+        if (pro == PRO_RMSNORM && AX.conv_st) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, true, FusedArgsCX>), grid, block, 0, stream(), P); return; }
+      }
+      const FusedArgsC& C = P;
+      if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, false, false, FusedArgsC>), grid, block, 0, stream(), C);
+      else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, false, false, FusedArgsC>), grid, block, 0, stream(), C);
+      else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, false, FusedArgsC>), grid, block, 0, stream(), C);
+      return;
+    }
+    if constexpr (KB == 8) {
+      if (pro == PRO_GNORM) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_GNORM, false, false, FusedArgsX>), grid, block, 0, stream(), AX); return; }
+    }
+    if constexpr (KB == 8 || KB == 4) {
+      if (pro == PRO_RMSNORM && AX.conv_st) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, true, FusedArgsX>), grid, block, 0, stream(), AX); return; }
+    }
+    const FusedArgs& A = AX;
+    if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, false>), grid, block, 0, stream(), A);
+    else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, false>), grid, block, 0, stream(), A);
+    else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false>), grid, block, 0, stream(), A);
   }
-  const FusedArgs& A = AX;
-  if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, SWIGLU>), grid, block, 0, stream(), A);
-  else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, SWIGLU>), grid, block, 0, stream(), A);
-  else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, SWIGLU>), grid, block, 0, stream(), A);
 }
 
 int g_tune_fused_cap = 0;     // workgroups per CU of the fused GEMV (0: chosen by the launcher)
