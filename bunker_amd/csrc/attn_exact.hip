@@ -444,8 +444,20 @@ __global__ __launch_bounds__(EX_THREADS) void attn_exact_kernel(AttnArgs A) {
 
 // Merge of the f64 split partials: one workgroup per (head, query row), thread = dim.  The weights exp(ref_s - max ref)
 // of all splits are computed side by side first (thread = split), the partial outputs are then added in split order.
+// Its argument block holds only what the merge reads (92 bytes: two 64-byte lines of kernel arguments, AttnArgs has five).
+struct AttnMergeArgs {
+  const double* part_o64;
+  const double* part_ml64;
+  const int2* plan;
+  const uint16_t* gate;
+  uint16_t* out;
+  uint8_t* out_q8;
+  float* lse;
+  int64_t gate_bstride, gate_hstride;
+  int NH, NKV, G, splits, slots;
+};
 template <int PRE>
-__global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnArgs A) {
+__global__ __launch_bounds__(256) void attn_exact_merge_kernel(AttnMergeArgs A) {
   __shared__ double wsh[ATT_MAX_SPLITS];
   __shared__ float redm[4];
   __shared__ double redl[4];
@@ -549,9 +561,11 @@ int launch_attn_exact(AttnArgs A, const void* q, const uint32_t* qf_ready, void*
   }
   if (A.splits > 1) {
     const dim3 mgrid(A.NH, batch);
-    if (A.splits <= 4) hipLaunchKernelGGL(attn_exact_merge_kernel<4>, mgrid, dim3(256), 0, stream(), A);
-    else if (A.splits <= 16) hipLaunchKernelGGL(attn_exact_merge_kernel<16>, mgrid, dim3(256), 0, stream(), A);
-    else hipLaunchKernelGGL(attn_exact_merge_kernel<64>, mgrid, dim3(256), 0, stream(), A);
+    const AttnMergeArgs M{A.part_o64, A.part_ml64, A.plan, A.gate, A.out, A.out_q8, A.lse, A.gate_bstride, A.gate_hstride,
+                          A.NH, A.NKV, A.G, A.splits, A.slots};
+    if (A.splits <= 4) hipLaunchKernelGGL(attn_exact_merge_kernel<4>, mgrid, dim3(256), 0, stream(), M);
+    else if (A.splits <= 16) hipLaunchKernelGGL(attn_exact_merge_kernel<16>, mgrid, dim3(256), 0, stream(), M);
+    else hipLaunchKernelGGL(attn_exact_merge_kernel<64>, mgrid, dim3(256), 0, stream(), M);
   }
   BK_LAUNCH_CHECK();
   return BK_OK;

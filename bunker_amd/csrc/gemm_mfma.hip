@@ -51,6 +51,34 @@ struct MfmaArgs {
   uint8_t* out_q8;        // SwiGLU form: g[0] = gate (out = bf16 activation or null), g[1] = up; Q8_1 blocks of the activation
 };
 
+// Compact argument blocks (a launch pays for every 64-byte line of kernel arguments, about a quarter of a microsecond;
+// MfmaArgs has three lines): one matrix in 56 bytes, the SwiGLU pair in 60.  The kernel rebuilds MfmaArgs in registers.
+struct MfmaArgs1 {
+  const uint8_t* W; void* out; const uint16_t* res; const uint8_t* xq;
+  int N, epi, nb, B, tiles, btiles;
+};
+struct MfmaArgsSw {
+  const uint8_t *Wg, *Wu; void* act; uint8_t* act_q8; const uint8_t* xq;
+  int N, nb, B, tiles, btiles;
+};
+__device__ __forceinline__ const MfmaArgs& mfma_args_full(const MfmaArgs& A) { return A; }
+__device__ __forceinline__ MfmaArgs mfma_args_full(const MfmaArgs1& P) {
+  MfmaArgs A;
+  const MfmaGroup g{P.W, P.out, P.res, P.N, P.epi};
+  A.g[0] = g; A.g[1] = g; A.g[2] = g; A.g[3] = g;
+  A.tile_first[0] = 0; A.tile_first[1] = A.tile_first[2] = A.tile_first[3] = A.tile_first[4] = P.tiles;
+  A.xq = P.xq; A.nb = P.nb; A.B = P.B; A.tiles = P.tiles; A.btiles = P.btiles; A.out_q8 = nullptr;
+  return A;
+}
+__device__ __forceinline__ MfmaArgs mfma_args_full(const MfmaArgsSw& P) {
+  MfmaArgs A;
+  const MfmaGroup g0{P.Wg, P.act, nullptr, P.N, 0}, g1{P.Wu, nullptr, nullptr, P.N, 0};
+  A.g[0] = g0; A.g[1] = g1; A.g[2] = g1; A.g[3] = g1;
+  A.tile_first[0] = 0; A.tile_first[1] = A.tile_first[2] = A.tile_first[3] = A.tile_first[4] = P.tiles;
+  A.xq = P.xq; A.nb = P.nb; A.B = P.B; A.tiles = P.tiles; A.btiles = P.btiles; A.out_q8 = P.act_q8;
+  return A;
+}
+
 enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 * GW_ROW, G_WAVE_LDS = GX_BYTES + GW_BYTES + 512 };
 
 // SWIGLU: the workgroup holds 2 NW waves; waves 0..NW-1 form the tile of 32 gate rows, waves NW..2NW-1 the tile of the
@@ -58,8 +86,9 @@ enum : int { GX_ROW = 292, GW_ROW = 144, GX_BYTES = 32 * GX_ROW, GW_BYTES = 32 *
 // TR: weight rows of the tile.  16 or 8 (the other rows of the matrix instruction repeat them and are ignored) for launches
 // with so few tiles that the time is the length of one wave's instruction stream: a half or a quarter of the fold per
 // super-block, two or four times the tiles.
-template <int NW, bool SWIGLU, int TR = 32>
-__global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma_kernel(MfmaArgs A) {
+template <int NW, bool SWIGLU, int TR = 32, typename ARGS = MfmaArgs>
+__global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma_kernel(ARGS A_in) {
+  const auto& A = mfma_args_full(A_in);
   static_assert(TR == 32 || TR == 16 || TR == 8, "tiles of 32, 16 or 8 weight rows");
   static_assert(!(SWIGLU && TR != 32), "the SwiGLU form quantizes 32 outputs at a time");
   constexpr int WAVES = NW * (SWIGLU ? 2 : 1);
@@ -86,7 +115,7 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kw = SWIGLU ? wave % NW : wave;           // this wave's place in the split of K
   const bool s1 = !SWIGLU && tile >= A.tile_first[1], s2 = !SWIGLU && tile >= A.tile_first[2], s3 = !SWIGLU && tile >= A.tile_first[3];
-  const uint8_t* __restrict__ W = SWIGLU ? A.g[wave / NW].W : s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
+  const uint8_t* __restrict__ W = SWIGLU ? (wave >= NW ? A.g[1].W : A.g[0].W) : s3 ? A.g[3].W : s2 ? A.g[2].W : s1 ? A.g[1].W : A.g[0].W;
   void* __restrict__ out = s3 ? A.g[3].out : s2 ? A.g[2].out : s1 ? A.g[1].out : A.g[0].out;
   const uint16_t* __restrict__ res = s3 ? A.g[3].res : s2 ? A.g[2].res : s1 ? A.g[1].res : A.g[0].res;
   const int N = s3 ? A.g[3].N : s2 ? A.g[2].N : s1 ? A.g[1].N : A.g[0].N;
@@ -376,6 +405,20 @@ __global__ __launch_bounds__(64 * NW * (SWIGLU ? 2 : 1)) void gemm_q4k_q8_1_mfma
 int g_tune_gemm_nw = 0;      // waves per tile (1, 2, 4, 8); 0 = chosen from the shape
 int g_tune_gemm_r16 = -1;    // narrow tiles (single batch tile only): 0 off, 1 = 16 weight rows, 2 = 8, -1 = from the shape
 
+template <typename ARGS>
+static void launch_mfma_plain(int tr, int nw, dim3 grid, const ARGS& A) {
+  if (tr == 16) {
+    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 16, ARGS>), grid, dim3(512), 0, stream(), A);
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 16, ARGS>), grid, dim3(256), 0, stream(), A);
+  } else if (tr == 8) {
+    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 8, ARGS>), grid, dim3(512), 0, stream(), A);
+    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 8, ARGS>), grid, dim3(256), 0, stream(), A);
+  } else if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 32, ARGS>), grid, dim3(512), 0, stream(), A);
+  else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 32, ARGS>), grid, dim3(256), 0, stream(), A);
+  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, false, 32, ARGS>), grid, dim3(128), 0, stream(), A);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, false, 32, ARGS>), grid, dim3(64), 0, stream(), A);
+}
+
 int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const void* const* W, void* const* out,
                            const void* const* res, const int* N, const int* epi) {
   BK_REQUIRE(xq && ngroups >= 1 && ngroups <= 4, "gemm_q4k_q8_1_mfma: bad arguments");
@@ -420,16 +463,12 @@ int launch_gemm_group_mfma(const void* xq, int K, int batch, int ngroups, const 
   nw = nw >= 8 ? 8 : (nw >= 4 ? 4 : (nw >= 2 ? 2 : 1));
   A.tiles = tiles; A.btiles = btiles;
   const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
-  if (tr == 16) {
-    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 16>), grid, dim3(512), 0, stream(), A);
-    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 16>), grid, dim3(256), 0, stream(), A);
-  } else if (tr == 8) {
-    if (nw >= 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false, 8>), grid, dim3(512), 0, stream(), A);
-    else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false, 8>), grid, dim3(256), 0, stream(), A);
-  } else if (nw == 8) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<8, false>), grid, dim3(512), 0, stream(), A);
-  else if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, false>), grid, dim3(256), 0, stream(), A);
-  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, false>), grid, dim3(128), 0, stream(), A);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, false>), grid, dim3(64), 0, stream(), A);
+  if (ngroups == 1) {
+    const MfmaArgs1 P{A.g[0].W, A.g[0].out, A.g[0].res, A.xq, A.g[0].N, A.g[0].epi, A.nb, A.B, tiles, btiles};
+    launch_mfma_plain(tr, nw, grid, P);
+  } else {
+    launch_mfma_plain(tr, nw, grid, A);
+  }
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
@@ -474,9 +513,10 @@ int launch_gemm_swiglu_mfma(const void* xq, int K, int batch, const void* Wg, co
   }
   nw = nw >= 4 ? 4 : (nw >= 2 ? 2 : 1);
   const dim3 grid(btiles > 1 ? (unsigned)(8 * ((wgs + 7) / 8)) : (unsigned)tiles);
-  if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, true>), grid, dim3(512), 0, stream(), A);
-  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, true>), grid, dim3(256), 0, stream(), A);
-  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, true>), grid, dim3(128), 0, stream(), A);
+  const MfmaArgsSw P{A.g[0].W, A.g[1].W, act, (uint8_t*)act_q8, A.xq, N, A.nb, A.B, tiles, btiles};
+  if (nw == 4) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<4, true, 32, MfmaArgsSw>), grid, dim3(512), 0, stream(), P);
+  else if (nw == 2) hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<2, true, 32, MfmaArgsSw>), grid, dim3(256), 0, stream(), P);
+  else hipLaunchKernelGGL((gemm_q4k_q8_1_mfma_kernel<1, true, 32, MfmaArgsSw>), grid, dim3(128), 0, stream(), P);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
