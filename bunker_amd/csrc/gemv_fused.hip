@@ -42,6 +42,7 @@ struct FusedArgs {
   FusedGroup g[4];
   int step_first[5];     // first step of each matrix; step_first[i >= ngroups] = total steps
   int ngroups;
+  int nwg;               // workgroups along x (read from here: gridDim would pull 256 bytes of implicit arguments into the block)
   const void* x;         // PRO_Q8: Q8_1 [batch, K/32 blocks]; PRO_GNORM: the GDN step's raw block per sequence; else bf16 [batch, K]
   const uint16_t* norm_w; // PRO_RMSNORM: bf16 [K]; PRO_GNORM: f32 [128]
 };
@@ -59,8 +60,8 @@ struct FusedArgsX : FusedArgs {
 // by cache line: every 64 bytes less measured 0.2-0.3 us per launch (one-matrix launches 168 -> 64 bytes: 11 us over the
 // decode step).  The launcher picks the smallest form that holds the launch; the kernel rebuilds the full form in
 // registers (step_first from the row counts) and runs unchanged.
-//   FusedArgs1: one matrix (out_proj, o_proj, down, lm_head: half of the step's launches), 60 bytes
-//   FusedArgs2: the SwiGLU pair, 48 bytes
+//   FusedArgs1: one matrix (out_proj, o_proj, down, lm_head: half of the step's launches), 64 bytes
+//   FusedArgs2: the SwiGLU pair, 52 bytes
 //   FusedArgsC: up to four matrices without residuals, 104 bytes; with the conv epilogue's operands (FusedArgsCX) 128
 //               (unused slots repeat the last matrix)
 struct FusedArgs1 {
@@ -68,14 +69,14 @@ struct FusedArgs1 {
   const void* x;
   const uint16_t* norm_w;
   int64_t x_bstride;
-  int steps;
+  int steps, nwg;
 };
 struct FusedArgs2 {
   const uint8_t *Wg, *Wu;
   void* out;
   const void* x;
   const uint16_t* norm_w;
-  int N, steps;
+  int N, steps, nwg;
 };
 struct FusedArgsC {
   const uint8_t* W[4];
@@ -84,7 +85,7 @@ struct FusedArgsC {
   const uint16_t* norm_w;
   int N[4];
   int epi4;              // epilogue of matrix i in bits 8 i .. 8 i + 7
-  int ngroups;
+  int ngroups;           // | workgroups along x << 8
 };
 struct FusedArgsCX : FusedArgsC {
   const uint16_t* conv_st;
@@ -96,8 +97,9 @@ __device__ __forceinline__ const FusedArgsX& fused_args_full(const FusedArgsX& A
 __device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs1& P, int) {
   FusedArgsX A;
   A.g[0] = P.g0; A.g[1] = P.g0; A.g[2] = P.g0; A.g[3] = P.g0;
-  A.step_first[0] = 0; A.step_first[1] = P.steps; A.step_first[2] = P.steps; A.step_first[3] = P.steps; A.step_first[4] = P.steps;
-  A.ngroups = 1; A.x = P.x; A.norm_w = P.norm_w;
+  const int steps = P.steps;
+  A.step_first[0] = 0; A.step_first[1] = steps; A.step_first[2] = steps; A.step_first[3] = steps; A.step_first[4] = steps;
+  A.ngroups = 1; A.nwg = P.nwg; A.x = P.x; A.norm_w = P.norm_w;
   A.conv_st = nullptr; A.conv_st_new = nullptr; A.conv_w = nullptr; A.x_bstride = P.x_bstride;
   return A;
 }
@@ -107,7 +109,7 @@ __device__ __forceinline__ FusedArgsX fused_args_full(const FusedArgs2& P, int) 
   A.g[1].W = P.Wu; A.g[1].out = P.out; A.g[1].res = nullptr; A.g[1].N = P.N; A.g[1].epi = EPI_BF16;
   A.g[2] = A.g[1]; A.g[3] = A.g[1];
   A.step_first[0] = 0; A.step_first[1] = P.steps; A.step_first[2] = P.steps; A.step_first[3] = P.steps; A.step_first[4] = P.steps;
-  A.ngroups = 2; A.x = P.x; A.norm_w = P.norm_w;
+  A.ngroups = 2; A.nwg = P.nwg; A.x = P.x; A.norm_w = P.norm_w;
   A.conv_st = nullptr; A.conv_st_new = nullptr; A.conv_w = nullptr; A.x_bstride = 0;
   return A;
 }
@@ -188,11 +190,14 @@ __device__ __forceinline__ StepFirst step_first_of(const FusedArgs& A, int) {
 }
 __device__ __forceinline__ StepFirst step_first_of(const FusedArgsC& P, int rps) {
   const int s0 = (P.N[0] + rps - 1) / rps;
-  const int s1 = s0 + (P.ngroups > 1 ? (P.N[1] + rps - 1) / rps : 0);
-  const int s2 = s1 + (P.ngroups > 2 ? (P.N[2] + rps - 1) / rps : 0);
-  const int s3 = s2 + (P.ngroups > 3 ? (P.N[3] + rps - 1) / rps : 0);
+  const int ng = P.ngroups & 0xff;
+  const int s1 = s0 + (ng > 1 ? (P.N[1] + rps - 1) / rps : 0);
+  const int s2 = s1 + (ng > 2 ? (P.N[2] + rps - 1) / rps : 0);
+  const int s3 = s2 + (ng > 3 ? (P.N[3] + rps - 1) / rps : 0);
   return StepFirst{s0, s1, s2, s3};
 }
+__device__ __forceinline__ int workgroups_x(const FusedArgs& A) { return A.nwg; }
+__device__ __forceinline__ int workgroups_x(const FusedArgsC& A) { return (int)((unsigned)A.ngroups >> 8); }
 __device__ __forceinline__ int rows_of_first(const FusedArgs& A) { return A.g[0].N; }
 __device__ __forceinline__ int rows_of_first(const FusedArgsC& A) { return A.N[0]; }
 __device__ __forceinline__ const uint8_t* second_matrix(const FusedArgs& A) { return A.g[1].W; }
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_fused_kernel(ARGS A_in) 
 
   const int lane = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nwaves = gridDim.x * GEMV_WAVES;
+  const int nwaves = workgroups_x(A) * GEMV_WAVES;
   const int bidx = blockIdx.y;
   const int c = lane & 7, b = lane >> 3;
   const ScaleSel sel = make_scale_sel(c);
@@ -461,7 +466,7 @@ static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
   for (int i = 0; i < AX.ngroups; i++) any_res = any_res || AX.g[i].res != nullptr;
   if constexpr (SWIGLU) {
     FusedArgs2 P{};
-    P.Wg = AX.g[0].W; P.Wu = AX.g[1].W; P.out = AX.g[0].out; P.x = AX.x; P.norm_w = AX.norm_w; P.N = AX.g[0].N; P.steps = AX.step_first[4];
+    P.Wg = AX.g[0].W; P.Wu = AX.g[1].W; P.out = AX.g[0].out; P.x = AX.x; P.norm_w = AX.norm_w; P.N = AX.g[0].N; P.steps = AX.step_first[4]; P.nwg = (int)grid.x;
     if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, true, false, FusedArgs2>), grid, block, 0, stream(), P);
     else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, true, false, FusedArgs2>), grid, block, 0, stream(), P);
     else hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, true, false, FusedArgs2>), grid, block, 0, stream(), P);
@@ -469,7 +474,7 @@ static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
   } else {
     if (AX.ngroups == 1) {         // one matrix
       FusedArgs1 P{};
-      P.g0 = AX.g[0]; P.x = AX.x; P.norm_w = AX.norm_w; P.x_bstride = AX.x_bstride; P.steps = AX.step_first[4];
+      P.g0 = AX.g[0]; P.x = AX.x; P.norm_w = AX.norm_w; P.x_bstride = AX.x_bstride; P.steps = AX.step_first[4]; P.nwg = (int)grid.x;
       if (pro == PRO_Q8) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_Q8, false, false, FusedArgs1>), grid, block, 0, stream(), P);
       else if (pro == PRO_BF16) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_BF16, false, false, FusedArgs1>), grid, block, 0, stream(), P);
       else if (pro == PRO_RMSNORM) hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, false, FusedArgs1>), grid, block, 0, stream(), P);
@@ -482,7 +487,7 @@ static void launch_fused_pro(int pro, dim3 grid, const FusedArgsX& AX) {
         const int j = i < AX.ngroups ? i : AX.ngroups - 1;
         P.W[i] = AX.g[j].W; P.out[i] = AX.g[j].out; P.N[i] = AX.g[j].N; P.epi4 |= (AX.g[j].epi & 0xff) << (8 * i);
       }
-      P.x = AX.x; P.norm_w = AX.norm_w; P.ngroups = AX.ngroups;
+      P.x = AX.x; P.norm_w = AX.norm_w; P.ngroups = AX.ngroups | (int)(grid.x << 8);
       P.conv_st = AX.conv_st; P.conv_st_new = AX.conv_st_new; P.conv_w = AX.conv_w;
       if constexpr (KB == 8 || KB == 4) {
         if (pro == PRO_RMSNORM && AX.conv_st) { hipLaunchKernelGGL((gemv_fused_kernel<KB, RPI, PRO_RMSNORM, false, true, FusedArgsCX>), grid, block, 0, stream(), P); return; }
@@ -560,6 +565,8 @@ int launch_gemv_fused(int pro, const void* x, const void* norm_w, int K, int bat
   } else {
     wgs = gemv_grid_for(wgs);
   }
+  BK_REQUIRE(wgs < (1 << 23), "gemv_fused: %d workgroups exceed what the argument block encodes", wgs);
+  A.nwg = wgs;
   const dim3 grid(wgs, batch);
   if (swiglu && KB == 4) launch_fused_pro<4, 4, true>(pro, grid, A);
   else if (swiglu) launch_fused_pro<8, 4, true>(pro, grid, A);

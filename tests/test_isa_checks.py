@@ -92,3 +92,27 @@ def test_lds_transfers_written_as_instructions_own_m0(tmp_path_factory, source, 
         assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, name
         assert int(re.search(r"\.sgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, name
         assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", meta).group(1)) == 0, name
+
+
+@pytest.mark.parametrize("source,kernel,kernarg_sizes", [
+    # SwiGLU pair 52 (padded to 56), one matrix 64, several matrices 104 / 128 with the convolution's operands, general
+    # 176 / 208; no implicit arguments behind them (the kernel reads the grid size from its block, not from gridDim)
+    ("gemv_fused.hip", "gemv_fused_kernel", {56, 64, 104, 128, 176, 208}),
+    ("gdn.hip", "gdn_slab_kernel", {80}),
+    ("gemm_mfma.hip", "gemm_q4k_q8_1_mfma_kernel", {56, 64, 184}),
+])
+def test_argument_blocks_stay_compact_and_in_registers(tmp_path_factory, source, kernel, kernarg_sizes):
+    """The decode step's kernels take the smallest by-value argument block their form needs (a launch pays for every
+    64-byte line of it) and rebuild the general block in registers.  That only works while the compiler keeps the rebuilt
+    block out of private memory and LDS: no kernel of these families may have a private segment, and every argument-block
+    size the launchers rely on must be there."""
+    asm = _compile_to_asm(tmp_path_factory, source)
+    seen = set()
+    for m in re.finditer(r"\.kernarg_segment_size:\s+(\d+)\n(.*?)\.name:\s+(\S+)\n(.*?)\.wavefront_size", asm, flags=re.S):
+        if kernel not in m.group(3):
+            continue
+        meta = m.group(2) + m.group(4)
+        seen.add(int(m.group(1)))
+        assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", meta).group(1)) == 0, m.group(3)
+        assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", meta).group(1)) == 0, m.group(3)
+    assert seen and seen <= kernarg_sizes and min(seen) == min(kernarg_sizes), seen
