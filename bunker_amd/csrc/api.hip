@@ -374,7 +374,7 @@ static int run_fa2_prefill(Kernel& k, const uint64_t* s) {
   if (rc) return rc;
   if (k.get("tiled", 0))
     return launch_attn_prefill_tiled(qn, P<void>(s[9]), P<void>(s[10]), table, pos, max_len, P<uint16_t>(s[0]) + HD, (int64_t)NH * 2 * HD, 2 * HD,
-                                     P<void>(s[11]), T, NH, NKV, HD, 16);
+                                     P<void>(s[11]), T, NH, NKV, HD, 16, ws, k.scratch_bytes - qn_bytes - qf_bytes);
   return launch_attn_decode(qn, P<void>(s[9]), P<void>(s[10]), table, 0, pos, 0, 1, max_len, P<uint16_t>(s[0]) + HD,
                             (int64_t)NH * 2 * HD, 2 * HD, P<void>(s[11]), nullptr, ws, k.scratch_bytes - qn_bytes - qf_bytes,
                             T, NH, NKV, HD, 16, (int)k.get("splits", 0), nullptr, k.get("pair", 0) ? 2 : 1, exact, qf);
@@ -488,7 +488,8 @@ static int build_kernel(Kernel& k) {
     int splits = (int)k.get("splits", 0);
     if (splits <= 0) { splits = attn_choose_splits((T + tpw - 1) / tpw, NKV, max_len); k.p["splits"] = splits; }
     const size_t qbytes = fa2_qn_bytes(T, (int)k.get("NH", 0), (int)k.get("HD", 0));
-    if ((rc = alloc_scratch(k, qbytes + fa2_ws_bytes(T, NKV, splits, exact)))) return rc;
+    const size_t ws_bytes = tiled ? attn_prefill_workspace_bytes(T, NHq, NKV, max_len) : fa2_ws_bytes(T, NKV, splits, exact);
+    if ((rc = alloc_scratch(k, qbytes + ws_bytes))) return rc;
     if (exact) BK_HIP(hipMemset(k.scratch, 0, k.scratch_bytes));
     k.run = run_fa2_prefill; k.nslots = 12;
     return BK_OK;
@@ -552,6 +553,7 @@ int bk_tune_set(const char* key, int value) {
   else if (!strcmp(key, "fused_cap")) bk::g_tune_fused_cap = value;
   else if (!strcmp(key, "attn_nt")) bk::g_tune_attn_nt = value;
   else if (!strcmp(key, "attn_bal")) bk::g_tune_attn_bal = value;
+  else if (!strcmp(key, "prefill_ksplit")) { BK_REQUIRE(value >= 0 && value <= 4, "bk_tune_set: prefill_ksplit=%d outside 0..4", value); bk::g_tune_prefill_ksplit = value; }
   else if (!strcmp(key, "gemm_r16")) bk::g_tune_gemm_r16 = value;
   else if (!strcmp(key, "small_rows")) bk::g_tune_small_rows = value;
   else if (!strcmp(key, "gdn_nt")) bk::g_tune_gdn_nt = value;

@@ -14,9 +14,12 @@
 // stand, and its A operand, the same 8 tokens of one dim, is one 16-byte read of a V row.  Softmax is the running-maximum form in f32 (base-2 exponent); the weights enter the
 // second product as bf16.  Results agree with the f64 checker to the 2e-2 of the matrix-instruction decode kernel,
 // not to the bit: the double-precision kernel (attn_exact.hip) stays the default of the prompt path.
+#include <algorithm>
 #include "attn_args.h"
 
 namespace bk {
+
+int g_tune_prefill_ksplit = 0;    // runs along K/V of the tiled prompt attention (0: from the shape)
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
@@ -43,17 +46,27 @@ struct PrefillAttnArgs {
   uint16_t* out;                   // bf16 [T, NH, 256]
   int T, NH, NKV, G, gshift, QT, max_ctx;
   float scale_log2;                // softmax scale times log2(e)
+  // ksplit > 1: blockIdx.z cuts the K/V tiles of a workgroup into ksplit runs (a launch with fewer workgroups than CUs);
+  // every run leaves its rows unnormalised, a second kernel joins them
+  int ksplit;
+  float* part_o;                   // f32 [ksplit, T, NH, 256]
+  float* part_ml;                  // f32 [ksplit, T, NH, 2]: reference exponent (base 2), sum of weights
 };
 
-// K/V tiles travel from memory straight into LDS (lds_dma16: lane l of a wave fills the l-th 16-byte
-// slot of a 1 KiB piece of LDS from an address of its own choosing), two tiles deep: no registers hold them and no
-// wave spends instructions on the copy.  A slot's position is fixed by the lane, so rows cannot be padded against bank
-// conflicts; instead the 16-byte units of a row are stored exclusive-or'ed with a few bits of the row number
-// (K: unit ^ (row % 16); V: unit ^ ((dim / 2) % 8)), which spreads the 32 rows of an operand read over all banks.
+// K/V tiles travel from memory straight into LDS (lds_dma16_s: lane l of a wave fills the l-th 16-byte slot of a 1 KiB
+// piece of LDS from an address of its own choosing), two tiles deep: no registers hold them and no wave spends
+// instructions on the copy.  A slot's position is fixed by the lane, so rows cannot be padded against bank conflicts;
+// instead a piece holds exactly what one operand read of the matrix instructions takes, in lane order or a permutation of
+// it inside each group of 16 lanes, and every transfer reads from one page (a scalar base per page, a constant offset
+// per lane: no address arithmetic in the tile loop):
+//   K piece (page p, dim group sp): slot 16 c + t = dims 32 sp + 8 c .. + 8 of token t of the page (c = 0..3);
+//     the read of dim slice sl = 2 sp + e for token rows 32 u + tau(col) finds token tau at piece (2 u + tau / 16, sp),
+//     slot 16 (2 e + half) + tau % 16
+//   V piece (page jj, dim tile dt): slot 32 h + c = tokens 8 h .. + 8 of the page for dim 32 dt + c: lane l reads slot l
 __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArgs A) {
   __shared__ __align__(1024) unsigned char lds_tiles[2 * PF_BUF];
   __shared__ int lds_len[PF_ROWS];
-  __shared__ int lds_bt[PF_MAX_PAGES];
+  __shared__ __align__(16) int lds_bt[PF_MAX_PAGES + 4];        // (+ 4: the last tile's four entries always exist)
   __shared__ int lds_maxlen;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5, col = lane & 31;
@@ -70,10 +83,15 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   }
   __syncthreads();
   const int maxlen = lds_maxlen;
-  if (maxlen == 0) return;
+  if (maxlen == 0) return;                  // no row has a context: nothing is written (the join skips such rows too)
   const int npages = (maxlen + ATT_PAGE - 1) / ATT_PAGE;
-  const int ntiles = (maxlen + PF_TILE - 1) / PF_TILE;
-  for (int i = tid; i < npages; i += PF_THREADS) lds_bt[i] = A.block_table[i];
+  const int ntiles_all = (maxlen + PF_TILE - 1) / PF_TILE;
+  // this workgroup's run of tiles (the whole context unless the launch is cut along K/V)
+  const int zsplit = blockIdx.z;
+  const int tile_lo = A.ksplit > 1 ? (int)((int64_t)zsplit * ntiles_all / A.ksplit) : 0;
+  const int ntiles = A.ksplit > 1 ? (int)((int64_t)(zsplit + 1) * ntiles_all / A.ksplit) : ntiles_all;
+  // a page past the longest row (the last tile may be short) reads the last page again; its tokens are masked below
+  for (int i = tid; i < 4 * ntiles_all; i += PF_THREADS) lds_bt[i] = A.block_table[min(i, npages - 1)];
   __syncthreads();
 
   // this lane's query row: token t0 + m / G, head kvh * G + m % G
@@ -88,27 +106,24 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     for (int s = 0; s < 16; s++) qreg[s] = *(const uint4*)(qp + 16 * s);
   }
 
-  // A page past the longest row (the last tile may be short) reads the last page again; its tokens are masked below.
-  auto page_base = [&](int pg) -> int64_t { return ((int64_t)lds_bt[min(pg, npages - 1)] * A.NKV + kvh) * (ATT_PAGE * ATT_HD); };
-  // Copy of tile `tile` into buffer tile % 2.  Round i of wave w fills the 1 KiB piece 4 i + w: K rows 2 (4 i + w) and
-  // + 1 (lane / 32 picks the row, lane % 32 the slot), V dim rows 8 (4 i + w) .. + 8 (lane / 8 the row, lane % 8 the slot).
+  // Copy of tile `tile` into buffer tile % 2.  Round i of wave w fills piece 4 i + w of K and of V: page i / 2 of the
+  // tile, K dim group / V dim tile 4 (i % 2) + w.
+  const uint32_t kvoff0 = (uint32_t)((lane & 15) * (ATT_HD * 2) + (lane >> 4) * 16 + wave * 64);      // bytes inside the page's K block; + 256 for odd i
+  const uint32_t vvoff0 = (uint32_t)((32 * wave + col) * (ATT_PAGE * 2) + half * 16);                 // bytes inside the page's V block; + 4096 for odd i
+  const uint32_t kvoff1 = kvoff0 + 256, vvoff1 = vvoff0 + 4096;
+  const int64_t page_bytes = (int64_t)A.NKV * (ATT_PAGE * ATT_HD * 2);
+  const unsigned char* kc_head = (const unsigned char*)A.kc + (int64_t)kvh * (ATT_PAGE * ATT_HD * 2);
+  const unsigned char* vc_head = (const unsigned char*)A.vc + (int64_t)kvh * (ATT_PAGE * ATT_HD * 2);
   auto copy_tile = [&](int tile) {
     unsigned char* kb = lds_tiles + (tile & 1) * PF_BUF;
     unsigned char* vb = kb + PF_KBYTES;
+    const int4 pg4 = *(const int4*)&lds_bt[4 * tile];
+    const int pg[4] = {__builtin_amdgcn_readfirstlane(pg4.x), __builtin_amdgcn_readfirstlane(pg4.y),
+                       __builtin_amdgcn_readfirstlane(pg4.z), __builtin_amdgcn_readfirstlane(pg4.w)};
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int piece = 4 * i + wave;
-      const int row = 2 * piece + (lane >> 5), unit = (lane & 31) ^ (row & 15);
-      const uint16_t* src = A.kc + page_base(tile * 4 + (row >> 4)) + (row & 15) * ATT_HD + unit * 8;
-      lds_dma16(src, kb + piece * 1024);
-    }
+    for (int i = 0; i < 8; i++) lds_dma16_s(kc_head + pg[i >> 1] * page_bytes, (i & 1) ? kvoff1 : kvoff0, kb + (4 * i + wave) * 1024);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int piece = 4 * i + wave;
-      const int dim = 8 * piece + (lane >> 3), unit = (lane & 7) ^ ((dim >> 1) & 7);     // unit = 2 * page + half of the page's tokens
-      const uint16_t* src = A.vc + page_base(tile * 4 + (unit >> 1)) + dim * ATT_PAGE + (unit & 1) * 8;
-      lds_dma16(src, vb + piece * 1024);
-    }
+    for (int i = 0; i < 8; i++) lds_dma16_s(vc_head + pg[i >> 1] * page_bytes, (i & 1) ? vvoff1 : vvoff0, vb + (4 * i + wave) * 1024);
   };
   // What the cache holds behind the longest row need not be a number, and 0 * NaN would reach the output: the values
   // of those tokens become zeros in LDS (the tile that holds the end of the rows only; thread = dim).
@@ -117,8 +132,8 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     __syncthreads();
     const int first_bad = maxlen - tile * PF_TILE;
     if (tile < ntiles && first_bad < PF_TILE) {
-      unsigned char* vrow = lds_tiles + (tile & 1) * PF_BUF + PF_KBYTES + tid * (PF_TILE * 2);
-      for (int tk = max(first_bad, 0); tk < PF_TILE; tk++) *(uint16_t*)(vrow + (((tk >> 3) ^ ((tid >> 1) & 7)) * 16) + (tk & 7) * 2) = 0;
+      unsigned char* vt = lds_tiles + (tile & 1) * PF_BUF + PF_KBYTES + ((tid >> 5) * 64 + (tid & 31)) * 16;      // dim tid: piece (jj, tid / 32), slot 32 h + tid % 32
+      for (int tk = max(first_bad, 0); tk < PF_TILE; tk++) *(uint16_t*)(vt + (tk >> 4) * 8192 + ((tk >> 3) & 1) * 512 + (tk & 7) * 2) = 0;
       __syncthreads();
     }
   };
@@ -134,22 +149,18 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   int wave_minlen = mylen;
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) wave_minlen = min(wave_minlen, __shfl_xor(wave_minlen, off));
+  wave_minlen = __builtin_amdgcn_readfirstlane(wave_minlen);       // (the same in every lane: a scalar branch below, not a masked region)
 
   // Row `col` of the first product's A operand is K token tau(col) of the 32 (bits 2 and 3 of col exchanged): the
   // result registers 8 jj .. 8 jj + 7 of a lane then belong to the 8 consecutive tokens 16 jj + 8 half .. + 8, which is
   // one 16-byte unit of a V row — the B operand of the second product needs no shuffle and its A operand is one read.
   const int tau = (col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1);
-  const int khs = half ^ (tau & 15);           // unit 2 sl + half of K row 32 u + tau sits at ((2 sl) ^ khs) * 16
-  const int vhs = half ^ ((col >> 1) & 7);     // unit 2 jj + half of V row 32 dt + col sits at ((2 jj) ^ vhs) * 16
-  int koff[8], voff[4];
-#pragma unroll
-  for (int sl = 0; sl < 8; sl++) koff[sl] = tau * (ATT_HD * 2) + (((2 * sl) ^ khs) * 16);      // sl + 8: 256 bytes further
-#pragma unroll
-  for (int jj = 0; jj < 4; jj++) voff[jj] = col * (PF_TILE * 2) + (((2 * jj) ^ vhs) * 16);
+  const int kread_off = (tau >> 4) * 8192 + ((tau & 15) + 16 * half) * 16;      // + u * 16384 + (sl / 2) * 1024 + (sl % 2) * 512
+  const int vread_off = lane * 16;                                            // + (jj * 8 + dt) * 1024
 
-  copy_tile(0);
-  land_tile(0);
-  for (int tile = 0; tile < ntiles; tile++) {
+  if (tile_lo < ntiles) copy_tile(tile_lo);
+  land_tile(tile_lo);
+  for (int tile = tile_lo; tile < ntiles; tile++) {
     const int tok_base = tile * PF_TILE;
     const unsigned char* lds_k = lds_tiles + (tile & 1) * PF_BUF;
     const unsigned char* lds_v = lds_k + PF_KBYTES;
@@ -171,7 +182,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int sl = 2 * bt + (i >> 1);
-          dst[i] = *(const uint4*)(lds_k + koff[sl & 7] + (sl >> 3) * 256 + (i & 1) * 32 * (ATT_HD * 2));
+          dst[i] = *(const uint4*)(lds_k + kread_off + (i & 1) * 16384 + (sl >> 1) * 1024 + (sl & 1) * 512);
         }
       };
       kread(0, ka[0]);
@@ -187,6 +198,12 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // (the scores leave the matrix unit's registers here, once: without this the masked branch below makes the compiler
+    // read them out twice, in front of the branch and behind it)
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) { float x = s[u][r]; asm volatile("" : "+v"(x)); s[u][r] = x; }
     // ---- running-maximum softmax of the row (base 2).  The maximum is taken over the raw scores (the scale is positive);
     // scale and subtraction are one fused multiply-add in front of the hardware exponential (v_exp_f32: 1 ulp, results
     // below 2^-126 become 0 — far inside the 2e-2 of this kernel).
@@ -239,7 +256,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
       uint4 va[2][4];
       auto vread = [&](int b, uint4 (&dst)[4]) {       // batch b: slice b / 2, dim tiles 4 (b % 2) .. + 4
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(lds_v + voff[b >> 1] + (4 * (b & 1) + i) * 32 * (PF_TILE * 2));
+        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(lds_v + vread_off + ((b >> 1) * 8 + 4 * (b & 1) + i) * 1024);
       };
       vread(0, va[0]);
 #pragma unroll
@@ -261,6 +278,18 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   // ---- output: the row's two lanes hold dims 32 dt + 8 (r / 4) + 4 half + r % 4
   const float ltot = lrow + __shfl_xor(lrow, 32);
   if (mylen <= 0 || tq >= A.T) return;
+  if (A.ksplit > 1) {
+    // the run's share of the row as it stands: a row that saw no token in this run leaves (-inf, 0) and is skipped by the join
+    const int64_t prow = ((int64_t)zsplit * A.T + tq) * A.NH + head;
+    if (half == 0) *(float2*)(A.part_ml + prow * 2) = make_float2(mrow, ltot);
+    float* po = A.part_o + prow * ATT_HD;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++)
+        *(float4*)(po + 32 * dt + 8 * g + 4 * half) = make_float4(o[dt][4 * g], o[dt][4 * g + 1], o[dt][4 * g + 2], o[dt][4 * g + 3]);
+    return;
+  }
   const float inv = ltot > 0.0f ? 1.0f / ltot : 0.0f;
   uint16_t* op = A.out + ((int64_t)tq * A.NH + head) * ATT_HD;
   const uint16_t* gp = A.gate ? A.gate + (int64_t)tq * A.gate_bstride + (int64_t)head * A.gate_hstride : nullptr;
@@ -283,15 +312,56 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     }
 }
 
+// Join of the runs of a launch cut along K/V: one workgroup per (token, head), thread = dim.
+__global__ __launch_bounds__(ATT_HD) void attn_prefill_join_kernel(PrefillAttnArgs A) {
+  const int t = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  if (min(max(A.pos[t] + 1, 0), A.max_ctx) <= 0) return;         // a row without context is left alone, as in the uncut launch
+  float m[4], l[4], M = -INFINITY;
+#pragma unroll
+  for (int z = 0; z < 4; z++) {
+    const float2 ml = z < A.ksplit ? *(const float2*)(A.part_ml + (((int64_t)z * A.T + t) * A.NH + head) * 2) : make_float2(-INFINITY, 0.0f);
+    m[z] = ml.x; l[z] = ml.y;
+    M = fmaxf(M, m[z]);
+  }
+  float L = 0.0f, acc = 0.0f;
+#pragma unroll
+  for (int z = 0; z < 4; z++) {
+    if (z < A.ksplit && m[z] != -INFINITY) {                      // (wave-uniform)
+      const float w = __builtin_amdgcn_exp2f(m[z] - M);
+      L += l[z] * w;
+      acc += A.part_o[(((int64_t)z * A.T + t) * A.NH + head) * ATT_HD + d] * w;
+    }
+  }
+  float v = L > 0.0f ? acc * (1.0f / L) : 0.0f;
+  if (A.gate) v = __fmul_rn(v, sigmoid_f64(bf16_to_f32(A.gate[(int64_t)t * A.gate_bstride + (int64_t)head * A.gate_hstride + d])));
+  A.out[((int64_t)t * A.NH + head) * ATT_HD + d] = f32_to_bf16(v);
+}
+
 bool attn_prefill_tiled_serves(int NH, int NKV, int max_ctx) {
   if (NKV <= 0 || NH % NKV) return false;
   const int G = NH / NKV;
   return (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && (max_ctx + ATT_PAGE - 1) / ATT_PAGE <= PF_MAX_PAGES;
 }
 
+// How many runs along K/V a launch is cut into: as many as it takes to give every CU a workgroup (at most 4), while a run
+// keeps at least 8 tiles of the longest context.
+int attn_prefill_ksplit(int T, int NH, int NKV, int max_ctx) {
+  if (g_tune_prefill_ksplit > 0) return g_tune_prefill_ksplit > 4 ? 4 : g_tune_prefill_ksplit;
+  const int QT = PF_ROWS / (NH / NKV);
+  const int wgs = ((T + QT - 1) / QT) * NKV;
+  int ks = num_cus() / (wgs > 0 ? wgs : 1);
+  const int by_len = ((max_ctx + PF_TILE - 1) / PF_TILE) / 8;
+  if (ks > by_len) ks = by_len;
+  return ks < 1 ? 1 : (ks > 4 ? 4 : ks);
+}
+size_t attn_prefill_workspace_bytes(int T, int NH, int NKV, int max_ctx) {
+  const int ks = attn_prefill_ksplit(T, NH, NKV, max_ctx);
+  return ks > 1 ? (size_t)ks * T * NH * (ATT_HD + 2) * sizeof(float) : 0;
+}
+
 int launch_attn_prefill_tiled(const void* q, const void* kc, const void* vc, const int32_t* block_table, const int32_t* pos, int max_ctx,
                               const void* gate, int64_t gate_bstride, int64_t gate_hstride, void* out, int T, int NH, int NKV, int HD,
-                              int page_size) {
+                              int page_size, void* workspace, size_t workspace_bytes) {
   BK_REQUIRE(q && kc && vc && block_table && pos && out, "attn_prefill: null pointer");
   BK_REQUIRE(HD == ATT_HD && page_size == ATT_PAGE, "attn_prefill: this build serves head_dim 256 and 16-token pages (got %d, %d)", HD, page_size);
   BK_REQUIRE(T >= 1 && T <= 65535 * 8 && NKV >= 1 && NKV <= 65535 && max_ctx >= 1, "attn_prefill: bad T=%d / NKV=%d / max_ctx=%d", T, NKV, max_ctx);
@@ -308,8 +378,19 @@ int launch_attn_prefill_tiled(const void* q, const void* kc, const void* vc, con
   while ((1 << A.gshift) < A.G) A.gshift++;
   A.QT = PF_ROWS / A.G;
   A.scale_log2 = (float)(1.4426950408889634 / sqrt((double)ATT_HD));
-  const dim3 grid((T + A.QT - 1) / A.QT, NKV);
+  A.ksplit = attn_prefill_ksplit(T, NH, NKV, max_ctx);
+  {   // a workspace smaller than the cut asks for (none at all: the plain launch) holds fewer runs
+    const size_t per_run = (size_t)T * NH * (ATT_HD + 2) * sizeof(float);
+    const int fits = workspace ? (int)std::min<size_t>(workspace_bytes / per_run, 4) : 0;
+    if (A.ksplit > fits) A.ksplit = fits > 1 ? fits : 1;
+  }
+  if (A.ksplit > 1) {
+    A.part_o = (float*)workspace;
+    A.part_ml = A.part_o + (size_t)A.ksplit * T * NH * ATT_HD;
+  }
+  const dim3 grid((T + A.QT - 1) / A.QT, NKV, A.ksplit);
   hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS), 0, stream(), A);
+  if (A.ksplit > 1) hipLaunchKernelGGL(attn_prefill_join_kernel, dim3(T, NH), dim3(ATT_HD), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }

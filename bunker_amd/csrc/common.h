@@ -265,6 +265,11 @@ __device__ __forceinline__ double block_sum_f64(double v, double* lds) {
 __device__ __forceinline__ void lds_dma16(const void* src, const void* lds_piece) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
 }
+// the same with the address as a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane: a run of
+// transfers from one page costs no vector arithmetic
+__device__ __forceinline__ void lds_dma16_s(const void* sbase, uint32_t voff, const void* lds_piece) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
+}
 __device__ __forceinline__ void lds_dma4(const void* src, const void* lds_piece) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"((uint32_t)(uintptr_t)lds_piece) : "memory", "m0");
 }
