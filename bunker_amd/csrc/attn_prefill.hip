@@ -15,6 +15,7 @@
 // second product as bf16.  Results agree with the f64 checker to the 2e-2 of the matrix-instruction decode kernel,
 // not to the bit: the double-precision kernel (attn_exact.hip) stays the default of the prompt path.
 #include <algorithm>
+#include <type_traits>
 #include "attn_args.h"
 
 namespace bk {
@@ -106,24 +107,28 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     for (int s = 0; s < 16; s++) qreg[s] = *(const uint4*)(qp + 16 * s);
   }
 
-  // Copy of tile `tile` into buffer tile % 2.  Round i of wave w fills piece 4 i + w of K and of V: page i / 2 of the
-  // tile, K dim group / V dim tile 4 (i % 2) + w.
+  // Transfers of the K and of the V part of a tile into buffer tile % 2.  Round i of wave w fills piece 4 i + w: page
+  // i / 2 of the tile, K dim group / V dim tile 4 (i % 2) + w.  `off` holds the byte offsets of the tile's four pages in
+  // the caches (scalar registers).
   const uint32_t kvoff0 = (uint32_t)((lane & 15) * (ATT_HD * 2) + (lane >> 4) * 16 + wave * 64);      // bytes inside the page's K block; + 256 for odd i
   const uint32_t vvoff0 = (uint32_t)((32 * wave + col) * (ATT_PAGE * 2) + half * 16);                 // bytes inside the page's V block; + 4096 for odd i
   const uint32_t kvoff1 = kvoff0 + 256, vvoff1 = vvoff0 + 4096;
   const int64_t page_bytes = (int64_t)A.NKV * (ATT_PAGE * ATT_HD * 2);
   const unsigned char* kc_head = (const unsigned char*)A.kc + (int64_t)kvh * (ATT_PAGE * ATT_HD * 2);
   const unsigned char* vc_head = (const unsigned char*)A.vc + (int64_t)kvh * (ATT_PAGE * ATT_HD * 2);
-  auto copy_tile = [&](int tile) {
-    unsigned char* kb = lds_tiles + (tile & 1) * PF_BUF;
-    unsigned char* vb = kb + PF_KBYTES;
-    const int4 pg4 = *(const int4*)&lds_bt[4 * tile];
-    const int pg[4] = {__builtin_amdgcn_readfirstlane(pg4.x), __builtin_amdgcn_readfirstlane(pg4.y),
-                       __builtin_amdgcn_readfirstlane(pg4.z), __builtin_amdgcn_readfirstlane(pg4.w)};
-#pragma unroll
-    for (int i = 0; i < 8; i++) lds_dma16_s(kc_head + pg[i >> 1] * page_bytes, (i & 1) ? kvoff1 : kvoff0, kb + (4 * i + wave) * 1024);
-#pragma unroll
-    for (int i = 0; i < 8; i++) lds_dma16_s(vc_head + pg[i >> 1] * page_bytes, (i & 1) ? vvoff1 : vvoff0, vb + (4 * i + wave) * 1024);
+  struct PageOff { int64_t b[4]; };
+  auto page_offsets = [&](const int4& pg4) {        // pg4: the four block-table entries, the same in every lane
+    PageOff r;
+    r.b[0] = __builtin_amdgcn_readfirstlane(pg4.x) * page_bytes; r.b[1] = __builtin_amdgcn_readfirstlane(pg4.y) * page_bytes;
+    r.b[2] = __builtin_amdgcn_readfirstlane(pg4.z) * page_bytes; r.b[3] = __builtin_amdgcn_readfirstlane(pg4.w) * page_bytes;
+    return r;
+  };
+  auto tile_entries = [&](int tile) { return *(const int4*)&lds_bt[4 * tile]; };
+  auto copy_k1 = [&](int tile, const PageOff& off, int i) {
+    lds_dma16_s(kc_head + off.b[i >> 1], (i & 1) ? kvoff1 : kvoff0, lds_tiles + (tile & 1) * PF_BUF + (4 * i + wave) * 1024);
+  };
+  auto copy_v1 = [&](int tile, const PageOff& off, int i) {
+    lds_dma16_s(vc_head + off.b[i >> 1], (i & 1) ? vvoff1 : vvoff0, lds_tiles + (tile & 1) * PF_BUF + PF_KBYTES + (4 * i + wave) * 1024);
   };
   // What the cache holds behind the longest row need not be a number, and 0 * NaN would reach the output: the values
   // of those tokens become zeros in LDS (the tile that holds the end of the rows only; thread = dim).
@@ -158,85 +163,155 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   const int kread_off = (tau >> 4) * 8192 + ((tau & 15) + 16 * half) * 16;      // + u * 16384 + (sl / 2) * 1024 + (sl % 2) * 512
   const int vread_off = lane * 16;                                            // + (jj * 8 + dt) * 1024
 
-  if (tile_lo < ntiles) copy_tile(tile_lo);
-  land_tile(tile_lo);
-  for (int tile = tile_lo; tile < ntiles; tile++) {
-    const int tok_base = tile * PF_TILE;
-    const unsigned char* lds_k = lds_tiles + (tile & 1) * PF_BUF;
-    const unsigned char* lds_v = lds_k + PF_KBYTES;
-    // the next tile goes to the other buffer, which every wave left at the last barrier
-    if (tile + 1 < ntiles) copy_tile(tile + 1);
-    {
+  // ---- The tile loop, software-pipelined by hand: a wave is alone on its SIMD, so the matrix unit only stays busy while
+  // the same wave issues other work between two matrix instructions.  Iteration t runs
+  //   A: the first product of tile t + 1 (32 matrix instructions), between them the softmax of tile t and the eight
+  //      transfers of K of tile t + 2,
+  //   B: the second product of tile t (32 matrix instructions), between them the eight transfers of V of tile t + 1 (in
+  //      its first half) and the read-out of the scores of tile t + 1 (in its second half).
+  // The transfers go into the buffers that iteration t - 1 finished with.  They stand between the matrix instructions
+  // because a wave waits at the issue of a transfer until the CU's path from the caches to LDS has taken it (about 30
+  // cycles; all sixteen in one burst at the top of the iteration: 1600 of 5200 cycles per tile), and without a branch
+  // around them because behind a branch the compiler gathers the softmax in front of the whole product; past the last
+  // tile the last tile simply travels again, into a buffer nobody reads any more.  One wait + barrier per iteration: both
+  // parts are read right behind it (K of tile t + 2 by A of iteration t + 1, V of tile t + 1 by its B).
+  f32x16_t s[2];                        // scores of the current tile, in vector registers
+  uint4 pb[4];
+  float alpha = 1.0f;
 
-    // ---- scores, transposed: s[u][r] = S^T[token 32 u + 16 (r / 8) + 8 half + r % 8, this lane's row].  The A operands
-    // come from LDS in batches of eight 16-byte reads (four dim slices x the two token halves), requested a batch ahead
-    // of the eight matrix instructions that use them: a read directly in front of its instruction costs the whole LDS
-    // latency per instruction, with one wave per SIMD and nothing else to run.
-    f32x16_t s[2];
-    {
-      f32x16_t zero16;
+  // phase A.  MM: compute sn = S^T of the K tile at lds_k.  SM: softmax of s -> pb, alpha, mrow, lrow.
+  auto phase_a = [&](auto MMc, auto SMc, const unsigned char* lds_k, f32x16_t (&sn)[2], int ktile, const PageOff& koffs) {
+    constexpr bool MM = decltype(MMc)::value, SM = decltype(SMc)::value;
+    f32x16_t zero16;
 #pragma unroll
-      for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
-      uint4 ka[2][4];
-      auto kread = [&](int bt, uint4 (&dst)[4]) {
+    for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
+    uint4 ka[2][4];
+    auto kread = [&](int bt, uint4 (&dst)[4]) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int sl = 2 * bt + (i >> 1);
-          dst[i] = *(const uint4*)(lds_k + kread_off + (i & 1) * 16384 + (sl >> 1) * 1024 + (sl & 1) * 512);
-        }
-      };
-      kread(0, ka[0]);
+      for (int i = 0; i < 4; i++) {
+        const int sl = 2 * bt + (i >> 1);
+        dst[i] = *(const uint4*)(lds_k + kread_off + (i & 1) * 16384 + (sl >> 1) * 1024 + (sl & 1) * 512);
+      }
+    };
+    float mloc = -INFINITY, mnew = 0.0f, msub = 0.0f, psum = 0.0f, mloc2 = 0.0f;
+    if constexpr (MM) kread(0, ka[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int bt = 0; bt < 8; bt++) {
+    for (int bt = 0; bt < 8; bt++) {
+      if constexpr (MM) {
         if (bt + 1 < 8) kread(bt + 1, ka[(bt + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 4; i++)
-          s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[bt & 1][i]),
-                                                             __builtin_bit_cast(bf16x8_t, qreg[2 * bt + (i >> 1)]),
-                                                             (bt == 0 && i < 2) ? zero16 : s[i & 1], 0, 0, 0);   // (an inline 0 operand)
+          sn[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[bt & 1][i]),
+                                                              __builtin_bit_cast(bf16x8_t, qreg[2 * bt + (i >> 1)]),
+                                                              (bt == 0 && i < 2) ? zero16 : sn[i & 1], 0, 0, 0);
+      }
+      if constexpr (SM) {
+        // running-maximum softmax of the row (base 2), cut into eight pieces.  The maximum is taken over the raw scores
+        // (the scale is positive); scale and subtraction are one fused multiply-add in front of the hardware exponential
+        // (v_exp_f32: 1 ulp, results below 2^-126 become 0 - far inside the 2e-2 of this kernel).
+        if (bt == 0 || bt == 1) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[bt][r]);
+          if (bt == 1) mloc2 = __shfl_xor(mloc, 32);
+        }
+        if (bt == 2) {
+          mloc = fmaxf(mloc, mloc2) * A.scale_log2;
+          // The reference exponent of a row follows its maximum only when that has grown by more than 2^24 (or is the
+          // first): weights up to 2^24 are as exact in bf16 and f32 as weights up to 1, and the 128 accumulators of a
+          // lane need their rescaling pass in a few early tiles only.
+          mnew = (mloc > mrow + 24.0f) ? mloc : mrow;
+          msub = mnew == -INFINITY ? 0.0f : mnew;             // a row without any token so far: every weight is 0
+          alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mrow - mnew);   // (first tile with a token: exp2(-inf) = 0 times the zeros)
+          mrow = mnew;
+        }
+        if (bt >= 3 && bt <= 6) {
+          const int j = bt - 3;
+          float p[8];
+#pragma unroll
+          for (int e = 0; e < 8; e++) { p[e] = __builtin_amdgcn_exp2f(__fmaf_rn(s[j >> 1][8 * (j & 1) + e], A.scale_log2, -msub)); psum += p[e]; }
+          pb[j] = make_uint4(pk_bf16(p[0], p[1]), pk_bf16(p[2], p[3]), pk_bf16(p[4], p[5]), pk_bf16(p[6], p[7]));
+        }
+        if (bt == 7) lrow = lrow * alpha + psum;
+      }
+      if constexpr (MM && SM) {
+        // one matrix instruction, one operand read, then this piece's share of the vector work, four times
+        constexpr int NV = 7;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x402, NV, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (MM && SM) {
+        copy_k1(ktile, koffs, bt);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // (the scores leave the matrix unit's registers here, once: without this the masked branch below makes the compiler
-    // read them out twice, in front of the branch and behind it)
-#pragma unroll
-    for (int u = 0; u < 2; u++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) { float x = s[u][r]; asm volatile("" : "+v"(x)); s[u][r] = x; }
-    // ---- running-maximum softmax of the row (base 2).  The maximum is taken over the raw scores (the scale is positive);
-    // scale and subtraction are one fused multiply-add in front of the hardware exponential (v_exp_f32: 1 ulp, results
-    // below 2^-126 become 0 — far inside the 2e-2 of this kernel).
+  };
+  // the rows that end inside the tile are cut off
+  auto mask_scores = [&](int tile) {
+    const int tok_base = tile * PF_TILE;
     if (tok_base + PF_TILE > wave_minlen) {                         // (wave-uniform) the tile crosses the end of a row
 #pragma unroll
       for (int u = 0; u < 2; u++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
+        for (int r = 0; r < 16; r++) {
           if (tok_base + 32 * u + 16 * (r >> 3) + 8 * half + (r & 7) >= mylen) s[u][r] = -INFINITY;
+          if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);       // (a few comparison masks at a time: all 32 at once spill scalar registers)
+        }
     }
-    float mloc = -INFINITY;
+  };
+  // scores 8 q .. 8 q + 7 of sn leave the matrix unit's registers (once: pinned, or the masked branch makes the compiler
+  // read them out in front of the branch and again behind it)
+  auto take_scores = [&](f32x16_t (&sn)[2], int q) {
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+    for (int e = 0; e < 8; e++) { float x = sn[q >> 1][8 * (q & 1) + e]; asm volatile("" : "+v"(x)); s[q >> 1][8 * (q & 1) + e] = x; }
+  };
+  using std::true_type;
+  using std::false_type;
+
+  PageOff offs_next{};                  // pages of tile t + 1 (V transfers of iteration t; they were the K transfers of t - 1)
+  if (tile_lo < ntiles) {
+    const PageOff o0 = page_offsets(tile_entries(tile_lo));
+    offs_next = page_offsets(tile_entries(min(tile_lo + 1, ntiles - 1)));
 #pragma unroll
-      for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[u][r]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * A.scale_log2;
-    // The reference exponent of a row follows its maximum only when that has grown by more than 2^24 (or is the first):
-    // weights up to 2^24 are as exact in bf16 and f32 as weights up to 1, and the 128 accumulators of a lane need their
-    // rescaling pass in a few early tiles only instead of in every tile where some row of the wave sees a new maximum.
-    const float mnew = (mloc > mrow + 24.0f) ? mloc : mrow;
-    const float msub = mnew == -INFINITY ? 0.0f : mnew;             // a row without any token so far: every weight is 0
-    const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(mrow - mnew);   // (first tile with a token: exp2(-inf) = 0 times the zeros)
-    mrow = mnew;
-    float psum = 0.0f;
-    uint4 pb[4];
+    for (int i = 0; i < 8; i++) copy_k1(tile_lo, o0, i);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      float p[8];
+    for (int i = 0; i < 8; i++) copy_v1(tile_lo, o0, i);
 #pragma unroll
-      for (int e = 0; e < 8; e++) { p[e] = __builtin_amdgcn_exp2f(__fmaf_rn(s[j >> 1][8 * (j & 1) + e], A.scale_log2, -msub)); psum += p[e]; }
-      pb[j] = make_uint4(pk_bf16(p[0], p[1]), pk_bf16(p[2], p[3]), pk_bf16(p[4], p[5]), pk_bf16(p[6], p[7]));
-    }
-    lrow = lrow * alpha + psum;
+    for (int i = 0; i < 8; i++) copy_k1(tile_lo + 1, offs_next, i);
+  }
+  land_tile(tile_lo);
+  if (tile_lo < ntiles) {
+    f32x16_t sn[2];
+    phase_a(true_type{}, false_type{}, lds_tiles + (tile_lo & 1) * PF_BUF, sn, 0, offs_next);
+#pragma unroll
+    for (int q = 0; q < 4; q++) take_scores(sn, q);
+    mask_scores(tile_lo);
+  }
+#ifdef PF_PROF
+  long long pc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, pt = clock64(), pn;
+#define PF_MARK(k) { __builtin_amdgcn_sched_barrier(0); pn = clock64(); pc[k] += pn - pt; pt = pn; __builtin_amdgcn_sched_barrier(0); }
+#else
+#define PF_MARK(k)
+#endif
+  int4 entries2 = tile_lo < ntiles ? tile_entries(min(tile_lo + 2, ntiles - 1)) : make_int4(0, 0, 0, 0);   // block-table entries of tile t + 2
+  for (int tile = tile_lo; tile < ntiles; tile++) {
+    PF_MARK(0)
+    const unsigned char* lds_v = lds_tiles + (tile & 1) * PF_BUF + PF_KBYTES;
+    const unsigned char* lds_kn = lds_tiles + ((tile + 1) & 1) * PF_BUF;
+    const PageOff voffs = offs_next;                       // tile t + 1
+    const PageOff koffs = page_offsets(entries2);         // tile t + 2 (read from LDS an iteration ago)
+    offs_next = koffs;
+    entries2 = tile_entries(min(tile + 3, ntiles - 1));
+    PF_MARK(1)
+    f32x16_t sn[2];
+    if (tile + 1 < ntiles) phase_a(true_type{}, true_type{}, lds_kn, sn, tile + 2, koffs);
+    else phase_a(false_type{}, true_type{}, lds_kn, sn, 0, koffs);
+    PF_MARK(2)
     if (__builtin_expect(__ballot(alpha != 1.0f) != 0ull, 0)) {        // (rare after the first tiles, see above)
 #pragma unroll
       for (int dt = 0; dt < 8; dt++)
@@ -250,8 +325,9 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
           o[dt][r] = x * alpha;
         }
     }
-    // ---- values: O^T[dim 32 dt + .., row] += V^T . P^T over the four 16-token slices, the A operands again a batch
-    // (one slice, eight dim tiles) ahead
+    PF_MARK(3)
+    // ---- values: O^T[dim 32 dt + .., row] += V^T . P^T over the four 16-token slices, the A operands a batch
+    // (one slice, four dim tiles) ahead
     {
       uint4 va[2][4];
       auto vread = [&](int b, uint4 (&dst)[4]) {       // batch b: slice b / 2, dim tiles 4 (b % 2) .. + 4
@@ -269,11 +345,21 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[b & 1][i]), __builtin_bit_cast(bf16x8_t, pb[b >> 1]), o[dt], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+        if (b < 4) { copy_v1(tile + 1, voffs, 2 * b); copy_v1(tile + 1, voffs, 2 * b + 1); }      // (early: they must have arrived at the end of the iteration)
+        if (b >= 4) take_scores(sn, b - 4);           // (sn is complete long before; past the last tile it holds nothing and is not used)
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    }
-    land_tile(tile + 1);           // (also the barrier behind which this tile's buffer may be overwritten)
+    PF_MARK(4)
+    if (tile + 1 < ntiles) mask_scores(tile + 1);
+    PF_MARK(5)
+    land_tile(tile + 1);           // (also the barrier behind which this tile's buffers may be overwritten)
+    PF_MARK(6)
   }
+#ifdef PF_PROF
+  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
+    printf("wave %d tiles %d: top %lld copy %lld A %lld rescale %lld B %lld take %lld land %lld\n", wave, ntiles - tile_lo, pc[0], pc[1], pc[2], pc[3], pc[4], pc[5], pc[6]);
+#endif
 
   // ---- output: the row's two lanes hold dims 32 dt + 8 (r / 4) + 4 half + r % 4
   const float ltot = lrow + __shfl_xor(lrow, 32);

@@ -331,6 +331,59 @@ def test_fa2_prefill_tiled_attention_rows_in_any_order_and_a_long_context(orc):
             rt.cuFree(p)
 
 
+def test_fa2_prefill_tiled_attention_cut_along_the_context(orc):
+    """A launch with fewer workgroups than CUs is cut along K/V into 2..4 runs whose unnormalised rows a second kernel
+    joins (tuning key prefill_ksplit; 0 = chosen from the shape, here 4).  Every cut agrees with the checker row by row,
+    also where a run of a short row holds no token at all (rows of 1501..1540 tokens in runs of 6 tiles), and with the
+    uncut launch to a few bf16 steps."""
+    print("fa2_prefill tiled, cut along K/V", flush=True)
+    g = synth.rng(4242)
+    NH, NKV, HD, HALF, MAXL, T, pos0 = 16, 2, 256, 32, 2048, 40, 1500
+    pages = MAXL // 16
+    cos_t, sin_t = orc.rope_tables(MAXL, 64, 1e7)
+    kc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    vc = bf(g.standard_normal((pages, NKV, 16, HD)).astype(np.float32))
+    table = g.permutation(pages).astype(np.int32)
+    for tok in range(pos0 + T, MAXL):                  # behind the prompt: not numbers
+        kc[table[tok // 16], :, tok % 16, :] = 0x7fc0
+        vc[table[tok // 16], :, tok % 16, :] = 0xffc1
+    qgate = bf(g.standard_normal((T, NH, 2, HD)).astype(np.float32))
+    k = bf(g.standard_normal((T, NKV, HD)).astype(np.float32)); v = bf(g.standard_normal((T, NKV, HD)).astype(np.float32))
+    qw = bf((g.standard_normal(HD) * 0.1).astype(np.float32)); kw = bf((g.standard_normal(HD) * 0.1).astype(np.float32))
+    pos = (pos0 + np.arange(T)).astype(np.int32)
+    pos[3] = 70                                        # one row far shorter than the rest: most runs hold none of its tokens
+    ptrs = [rt.to_device(a) for a in (qgate, k, v, qw, kw, cos_t, sin_t, pos, table)]
+    outs = {}
+    try:
+        for ks in (1, 2, 3, 4, 0):
+            rt.tune_set("prefill_ksplit", ks)
+            dkc, dvc = rt.to_device(kc), rt.to_device(rt.v_pages_to_device_layout(vc))
+            dout = rt.cuAlloc(T * NH * HD * 2)
+            rt.cuMemset(dout, 0xff, T * NH * HD * 2)
+            _launch(f"fa2_prefill HD={HD} NH={NH} NKV={NKV} MAX_LEN={MAXL} ROT_HALF={HALF} T={T} exact=0", ptrs + [dkc, dvc, dout])
+            outs[ks] = rt.from_device(dout, (T, NH, HD), np.uint16)
+            for p in (dkc, dvc, dout):
+                rt.cuFree(p)
+    finally:
+        rt.tune_set("prefill_ksplit", 0)
+    order = np.argsort(pos, kind="stable")              # the op appends every token before any row attends
+    for t in range(T):
+        kn = orc.rope(orc.headnorm(k[t].ravel(), kw, NKV, HD, HD), cos_t, sin_t, pos[t], NKV, HD, HALF)
+        orc.kv_append(kn.reshape(NKV, HD), v[t], kc, vc, table, pos[t], NKV, HD, 16)
+    for ks, out in outs.items():
+        assert not np.any(out == 0xffff), ks
+        worst = 0.0
+        for t in order:
+            qn = orc.rope(orc.headnorm(qgate[t].ravel(), qw, NH, HD, 2 * HD), cos_t, sin_t, pos[t], NH, HD, HALF).reshape(1, NH, HD)
+            ro, _ = orc.attn_decode_paged(qn, kc, vc, table[None], np.array([pos[t] + 1], np.int32), 1, NH, NKV, HD, 16,
+                                          gate=qgate[t].ravel()[HD:], gate_bstride=0, gate_hstride=2 * HD)
+            worst = max(worst, float(np.abs(f32(out[t]).astype(np.float64) - f32(ro[0])).max()))
+        assert worst <= 2e-2, (ks, worst)
+        assert np.abs(f32(out).astype(np.float64) - f32(outs[1])).max() <= 2e-2, ks
+    for p in ptrs:
+        rt.cuFree(p)
+
+
 @pytest.mark.parametrize("n_prompt,chunk", [(23, 8), (9, 16)])
 def test_prefill_then_decode_equals_token_by_token(orc, n_prompt, chunk):
     """TINY model, two sequences in the cache; the prompt goes to sequence 1 in chunks (with a shorter last chunk),
