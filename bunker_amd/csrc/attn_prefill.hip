@@ -200,11 +200,13 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     for (int bt = 0; bt < 8; bt++) {
       if constexpr (MM) {
         if (bt + 1 < 8) kread(bt + 1, ka[(bt + 1) & 1]);
+        // (the operand requested last is used first: the one wait in front of it covers the other three, and the
+        // requests of the next batch, issued in front of this batch's products, have four products' time to arrive)
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 3; i >= 0; i--)
           sn[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[bt & 1][i]),
                                                               __builtin_bit_cast(bf16x8_t, qreg[2 * bt + (i >> 1)]),
-                                                              (bt == 0 && i < 2) ? zero16 : sn[i & 1], 0, 0, 0);
+                                                              (bt == 0 && i >= 2) ? zero16 : sn[i & 1], 0, 0, 0);
       }
       if constexpr (SM) {
         // running-maximum softmax of the row (base 2), cut into eight pieces.  The maximum is taken over the raw scores
@@ -235,12 +237,12 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
         if (bt == 7) lrow = lrow * alpha + psum;
       }
       if constexpr (MM && SM) {
-        // one matrix instruction, one operand read, then this piece's share of the vector work, four times
+        // the next batch's four operand reads, then one matrix instruction and this piece's share of the vector work, four times
         constexpr int NV = 7;
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x402, NV, 0);
         }
       }
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
         if (b + 1 < 8) vread(b + 1, va[(b + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 3; i >= 0; i--) {                  // (last request first, as above)
           const int dt = 4 * (b & 1) + i;
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[b & 1][i]), __builtin_bit_cast(bf16x8_t, pb[b >> 1]), o[dt], 0, 0, 0);
         }
