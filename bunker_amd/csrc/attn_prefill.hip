@@ -400,29 +400,44 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     }
 }
 
-// Join of the runs of a launch cut along K/V: one workgroup per (token, head), thread = dim.
-__global__ __launch_bounds__(ATT_HD) void attn_prefill_join_kernel(PrefillAttnArgs A) {
-  const int t = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+// Join of the runs of a launch cut along K/V: a wave per (token, head), lane = four dims, four rows per workgroup.
+__global__ __launch_bounds__(256) void attn_prefill_join_kernel(PrefillAttnArgs A) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);        // row = t * NH + head
+  if (r >= (int64_t)A.T * A.NH) return;
+  const int t = (int)(r / A.NH), head = (int)(r - (int64_t)t * A.NH), d = 4 * lane;
   if (min(max(A.pos[t] + 1, 0), A.max_ctx) <= 0) return;         // a row without context is left alone, as in the uncut launch
   float m[4], l[4], M = -INFINITY;
+  float4 o[4];
 #pragma unroll
-  for (int z = 0; z < 4; z++) {
-    const float2 ml = z < A.ksplit ? *(const float2*)(A.part_ml + (((int64_t)z * A.T + t) * A.NH + head) * 2) : make_float2(-INFINITY, 0.0f);
-    m[z] = ml.x; l[z] = ml.y;
+  for (int z = 0; z < 4; z++) {                                   // all requests first (a run that does not exist reads run 0 again)
+    const int64_t pr = (int64_t)(z < A.ksplit ? z : 0) * A.T * A.NH + r;
+    const float2 ml = *(const float2*)(A.part_ml + pr * 2);
+    o[z] = *(const float4*)(A.part_o + pr * ATT_HD + d);
+    m[z] = z < A.ksplit ? ml.x : -INFINITY; l[z] = ml.y;
     M = fmaxf(M, m[z]);
   }
-  float L = 0.0f, acc = 0.0f;
+  uint2 gw = make_uint2(0, 0);
+  if (A.gate) gw = *(const uint2*)(A.gate + (int64_t)t * A.gate_bstride + (int64_t)head * A.gate_hstride + d);
+  float L = 0.0f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
   for (int z = 0; z < 4; z++) {
-    if (z < A.ksplit && m[z] != -INFINITY) {                      // (wave-uniform)
+    if (m[z] != -INFINITY) {                                      // (wave-uniform; a run in which the row saw no token holds nothing usable)
       const float w = __builtin_amdgcn_exp2f(m[z] - M);
       L += l[z] * w;
-      acc += A.part_o[(((int64_t)z * A.T + t) * A.NH + head) * ATT_HD + d] * w;
+      acc.x += o[z].x * w; acc.y += o[z].y * w; acc.z += o[z].z * w; acc.w += o[z].w * w;
     }
   }
-  float v = L > 0.0f ? acc * (1.0f / L) : 0.0f;
-  if (A.gate) v = __fmul_rn(v, sigmoid_f64(bf16_to_f32(A.gate[(int64_t)t * A.gate_bstride + (int64_t)head * A.gate_hstride + d])));
-  A.out[((int64_t)t * A.NH + head) * ATT_HD + d] = f32_to_bf16(v);
+  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  float v[4] = {acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
+  if (A.gate) {
+    v[0] = __fmul_rn(v[0], sigmoid_f64(__uint_as_float(gw.x << 16)));
+    v[1] = __fmul_rn(v[1], sigmoid_f64(__uint_as_float(gw.x & 0xffff0000u)));
+    v[2] = __fmul_rn(v[2], sigmoid_f64(__uint_as_float(gw.y << 16)));
+    v[3] = __fmul_rn(v[3], sigmoid_f64(__uint_as_float(gw.y & 0xffff0000u)));
+  }
+  *(uint2*)(A.out + r * ATT_HD + d) = make_uint2(pk_bf16(v[0], v[1]), pk_bf16(v[2], v[3]));
 }
 
 bool attn_prefill_tiled_serves(int NH, int NKV, int max_ctx) {
@@ -478,7 +493,7 @@ int launch_attn_prefill_tiled(const void* q, const void* kc, const void* vc, con
   }
   const dim3 grid((T + A.QT - 1) / A.QT, NKV, A.ksplit);
   hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS), 0, stream(), A);
-  if (A.ksplit > 1) hipLaunchKernelGGL(attn_prefill_join_kernel, dim3(T, NH), dim3(ATT_HD), 0, stream(), A);
+  if (A.ksplit > 1) hipLaunchKernelGGL(attn_prefill_join_kernel, dim3((unsigned)(((int64_t)T * NH + 3) / 4)), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();
   return BK_OK;
 }
