@@ -553,6 +553,7 @@ int bk_tune_set(const char* key, int value) {
   else if (!strcmp(key, "fused_cap")) bk::g_tune_fused_cap = value;
   else if (!strcmp(key, "attn_nt")) bk::g_tune_attn_nt = value;
   else if (!strcmp(key, "attn_bal")) bk::g_tune_attn_bal = value;
+  else if (!strcmp(key, "prefill_xmap")) bk::g_tune_prefill_xmap = value != 0;
   else if (!strcmp(key, "prefill_ksplit")) { BK_REQUIRE(value >= 0 && value <= 4, "bk_tune_set: prefill_ksplit=%d outside 0..4", value); bk::g_tune_prefill_ksplit = value; }
   else if (!strcmp(key, "gemm_r16")) bk::g_tune_gemm_r16 = value;
   else if (!strcmp(key, "small_rows")) bk::g_tune_small_rows = value;

@@ -21,6 +21,7 @@
 namespace bk {
 
 int g_tune_prefill_ksplit = 0;    // runs along K/V of the tiled prompt attention (0: from the shape)
+int g_tune_prefill_xmap = 1;      // 0: plain three-dimensional grid instead of the XCD-aware mapping
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
@@ -49,7 +50,7 @@ struct PrefillAttnArgs {
   float scale_log2;                // softmax scale times log2(e)
   // ksplit > 1: blockIdx.z cuts the K/V tiles of a workgroup into ksplit runs (a launch with fewer workgroups than CUs);
   // every run leaves its rows unnormalised, a second kernel joins them
-  int ksplit;
+  int ksplit, nx, xmap;             // nx: query tiles; xmap: 0 = three-dimensional grid, 1 / 2 = XCD-aware one-dimensional grid (see the kernel)
   float* part_o;                   // f32 [ksplit, T, NH, 256]
   float* part_ml;                  // f32 [ksplit, T, NH, 2]: reference exponent (base 2), sum of weights
 };
@@ -71,8 +72,22 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   __shared__ int lds_maxlen;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5, col = lane & 31;
-  const int kvh = blockIdx.y;
-  const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * A.QT;      // the longest rows (last tokens) start first
+  // Workgroup -> (query tile x, KV head, run).  The workgroups of one (KV head, run) read the same K/V tiles at about the
+  // same time: where the number of such groups divides 8 or is a multiple of it (xmap > 0) the launch is one-dimensional
+  // and a group's workgroups run on the same XCD(s) - consecutive workgroup ids go round the 8 XCDs - so that a tile comes
+  // from memory once per group and its other readers find it in that XCD's L2; the query tiles of a group are dealt out
+  // to its XCDs in turn, longest rows first on each.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if (A.xmap > 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, groups = A.NKV * max(A.ksplit, 1);
+    int g;
+    if (A.xmap == 1) { const int P = 8 / groups; g = xcd / P; bx = slot * P + xcd % P; }     // P XCDs per group
+    else { g = xcd * (groups >> 3) + slot / A.nx; bx = slot % A.nx; }                          // groups / 8 groups per XCD
+    if (bx >= A.nx) return;
+    by = g % A.NKV; bz = g / A.NKV;
+  }
+  const int kvh = by;
+  const int t0 = (A.nx - 1 - bx) * A.QT;      // the longest rows (last tokens) start first
 
   if (tid == 0) lds_maxlen = 0;
   __syncthreads();
@@ -88,7 +103,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
   const int npages = (maxlen + ATT_PAGE - 1) / ATT_PAGE;
   const int ntiles_all = (maxlen + PF_TILE - 1) / PF_TILE;
   // this workgroup's run of tiles (the whole context unless the launch is cut along K/V)
-  const int zsplit = blockIdx.z;
+  const int zsplit = bz;
   const int tile_lo = A.ksplit > 1 ? (int)((int64_t)zsplit * ntiles_all / A.ksplit) : 0;
   const int ntiles = A.ksplit > 1 ? (int)((int64_t)(zsplit + 1) * ntiles_all / A.ksplit) : ntiles_all;
   // a page past the longest row (the last tile may be short) reads the last page again; its tokens are masked below
@@ -359,7 +374,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArg
     PF_MARK(6)
   }
 #ifdef PF_PROF
-  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
+  if (bx == 3 && by == 0 && bz == 0 && lane == 0)
     printf("wave %d tiles %d: top %lld copy %lld A %lld rescale %lld B %lld take %lld land %lld\n", wave, ntiles - tile_lo, pc[0], pc[1], pc[2], pc[3], pc[4], pc[5], pc[6]);
 #endif
 
@@ -491,7 +506,12 @@ int launch_attn_prefill_tiled(const void* q, const void* kc, const void* vc, con
     A.part_o = (float*)workspace;
     A.part_ml = A.part_o + (size_t)A.ksplit * T * NH * ATT_HD;
   }
-  const dim3 grid((T + A.QT - 1) / A.QT, NKV, A.ksplit);
+  A.nx = (T + A.QT - 1) / A.QT;
+  const int groups = NKV * A.ksplit;
+  A.xmap = g_tune_prefill_xmap == 0 ? 0 : (8 % groups == 0 ? 1 : (groups % 8 == 0 ? 2 : 0));
+  dim3 grid(A.nx, NKV, A.ksplit);
+  if (A.xmap == 1) grid = dim3(8 * ((A.nx + 8 / groups - 1) / (8 / groups)));
+  else if (A.xmap == 2) grid = dim3(A.nx * groups);
   hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS), 0, stream(), A);
   if (A.ksplit > 1) hipLaunchKernelGGL(attn_prefill_join_kernel, dim3((unsigned)(((int64_t)T * NH + 3) / 4)), dim3(256), 0, stream(), A);
   BK_LAUNCH_CHECK();

@@ -118,7 +118,7 @@ int launch_attn_decode(const void* q, const void* kc, const void* vc, const int3
                        const uint32_t* qf_ready = nullptr, const AttnPrepFuse* prep = nullptr);
 // attn_prefill.hip: causal attention of T prompt tokens, query tile x K/V tile on the bf16 matrix cores
 bool attn_prefill_tiled_serves(int NH, int NKV, int max_ctx);
-extern int g_tune_prefill_ksplit;
+extern int g_tune_prefill_ksplit, g_tune_prefill_xmap;
 size_t attn_prefill_workspace_bytes(int T, int NH, int NKV, int max_ctx);     // partial rows of a launch cut along K/V
 int launch_attn_prefill_tiled(const void* q, const void* kc, const void* vc, const int32_t* block_table, const int32_t* pos, int max_ctx,
                               const void* gate, int64_t gate_bstride, int64_t gate_hstride, void* out, int T, int NH, int NKV, int HD,

@@ -99,7 +99,8 @@ BK_API int bk_graph_node_count(uint64_t graph, int* count);
  * GDN core op), "gdn_nt" / "attn_nt" (state / cache pages through nontemporal accesses), "attn_bal" (attention splits
  * under lengths in device memory: 0 = equal ranges of max_ctx, 2 = of each sequence's own length, 1 = the batch's
  * workgroups shared out by length, -1 = 1 for long ranges, else 2), "prefill_ksplit" (runs along K/V of the tiled prompt
- * attention, 1..4; 0 = from the shape; read when an fa2_prefill handle is created).  No counterpart in the reference. */
+ * attention, 1..4; 0 = from the shape; read when an fa2_prefill handle is created), "prefill_xmap" (0: that kernel's workgroups in grid
+ * order instead of grouped by XCD).  No counterpart in the reference. */
 BK_API int bk_tune_set(const char* key, int value);
 
 /* ---- per-op launch surface: replaces compileAndLoad + cuLaunch
