@@ -245,7 +245,8 @@ def test_fa2_prefill_appends_and_attends_causally(orc, T, pos0, exact):
         rt.cuFree(p)
 
 
-@pytest.mark.parametrize("NH,NKV,T,pos0", [(16, 2, 200, 70), (16, 2, 64, 0), (8, 2, 97, 33), (4, 4, 130, 5), (16, 1, 50, 17), (4, 2, 129, 0)])
+@pytest.mark.parametrize("NH,NKV,T,pos0", [(16, 2, 200, 70), (16, 2, 64, 0), (8, 2, 97, 33), (4, 4, 130, 5), (16, 1, 50, 17), (4, 2, 129, 0),
+                                            (16, 16, 150, 20)])      # (16 KV heads: two groups of workgroups per XCD)
 def test_fa2_prefill_tiled_attention_against_the_checker(orc, NH, NKV, T, pos0):
     """exact=0 runs the query-tile x K/V-tile kernel (bf16 matrix cores): every row within 2e-2 of the f64 checker, for
     every group size it serves, ragged last query tile, a context that starts in the middle of a K/V tile, a permuted page
